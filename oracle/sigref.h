@@ -1,0 +1,42 @@
+/*
+ * sigref.h -- CPU oracle for the truncated path signature (TEST INFRASTRUCTURE ONLY).
+ *
+ * A dependency-free C restatement of the reference CPU library's forward and
+ * backward signature algorithm.  It exists to check the GPU library and to be
+ * timed as the CPU baseline; nothing in the shipped package may link or call it.
+ */
+#ifndef SIGREF_H
+#define SIGREF_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* siglib/cpsig/cp_utils.cpp:91-105: (d^(N+1)-1)/(d-1); 0 on uint64 overflow. */
+uint64_t sigref_sig_length(uint64_t dimension, uint64_t degree);
+/* siglib/cpsig/cp_utils.cpp:40-50: level_index[k] = (d^k-1)/(d-1), n entries. */
+int sigref_level_index(uint64_t *level_index, uint64_t dimension, uint64_t n);
+/* number of hardware threads n_jobs = -1 resolves to */
+int sigref_max_threads(void);
+/* siglib/cpsig/multithreading.cpp:43-81: contiguous chunks over min(threads, batch) workers. */
+void sigref_run_batch(uint64_t batch, int n_jobs, void *ctx, void (*worker)(void *, uint64_t, uint64_t));
+
+/* Same argument meaning as the reference's signature_{f,d} / sig_backprop_{f,d}
+ * (siglib/cpsig/cpsig.h:311-346) without the correction arguments.
+ * Return 0 ok, 1 out of memory, 2 invalid argument, 10 overflow. */
+int sigref_signature_f(const float *path, float *out, uint64_t batch, uint64_t dimension,
+                       uint64_t length, uint64_t degree, int time_aug, int lead_lag,
+                       float end_time, int horner, int scalar_term, int n_jobs);
+int sigref_signature_d(const double *path, double *out, uint64_t batch, uint64_t dimension,
+                       uint64_t length, uint64_t degree, int time_aug, int lead_lag,
+                       double end_time, int horner, int scalar_term, int n_jobs);
+int sigref_sig_backprop_f(const float *path, float *out, const float *sig_derivs, const float *sig,
+                          uint64_t batch, uint64_t dimension, uint64_t length, uint64_t degree,
+                          int time_aug, int lead_lag, float end_time, int scalar_term, int n_jobs);
+int sigref_sig_backprop_d(const double *path, double *out, const double *sig_derivs, const double *sig,
+                          uint64_t batch, uint64_t dimension, uint64_t length, uint64_t degree,
+                          int time_aug, int lead_lag, double end_time, int scalar_term, int n_jobs);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,113 @@
+"""ctypes binding of the CPU oracle ``libsigref.so`` (TEST INFRASTRUCTURE ONLY).
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg may import this
+module; the shipped package never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libsigref.so")
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile beside this file."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    u64, i32 = ctypes.c_uint64, ctypes.c_int
+    lib.sigref_sig_length.restype = u64
+    lib.sigref_sig_length.argtypes = (u64, u64)
+    lib.sigref_max_threads.restype = i32
+    for suf, real in (("f", ctypes.c_float), ("d", ctypes.c_double)):
+        ptr = ctypes.POINTER(real)
+        f = getattr(lib, "sigref_signature_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, u64, u64, u64, u64, i32, i32, real, i32, i32, i32)
+        g = getattr(lib, "sigref_sig_backprop_" + suf)
+        g.restype = i32
+        g.argtypes = (ptr, ptr, ptr, ptr, u64, u64, u64, u64, i32, i32, real, i32, i32)
+    return lib
+
+
+LIB = _load()
+
+
+def max_threads():
+    return int(LIB.sigref_max_threads())
+
+
+def sig_length(dimension, degree):
+    return int(LIB.sigref_sig_length(dimension, degree))
+
+
+def _suffix(dtype):
+    if dtype == np.float32:
+        return "f", ctypes.c_float
+    if dtype == np.float64:
+        return "d", ctypes.c_double
+    raise TypeError("oracle supports float32 and float64 only")
+
+
+def _aug_dim(d, time_aug, lead_lag):
+    return (2 * d if lead_lag else d) + (1 if time_aug else 0)
+
+
+def signature(path, degree, time_aug=False, lead_lag=False, end_time=1.0, horner=True,
+              scalar_term=False, n_jobs=1):
+    """Oracle forward pass. ``path`` is (B, len, d) or (len, d), float32/float64."""
+    path = np.ascontiguousarray(path)
+    single = path.ndim == 2
+    if single:
+        path = path[None]
+    batch, length, dim = path.shape
+    suf, real = _suffix(path.dtype)
+    n = sig_length(_aug_dim(dim, time_aug, lead_lag), degree) - (0 if scalar_term else 1)
+    out = np.empty((batch, n), dtype=path.dtype)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_signature_" + suf)(
+        path.ctypes.data_as(ptr), out.ctypes.data_as(ptr), batch, dim, length, degree,
+        int(time_aug), int(lead_lag), float(end_time), int(horner), int(scalar_term), n_jobs)
+    if rc:
+        raise RuntimeError("sigref_signature returned %d" % rc)
+    return out[0] if single else out
+
+
+def sig_backprop(path, sig, sig_derivs, degree, time_aug=False, lead_lag=False, end_time=1.0,
+                 n_jobs=1):
+    """Oracle backward pass; scalar_term is inferred from the width of ``sig``."""
+    path = np.ascontiguousarray(path)
+    single = path.ndim == 2
+    if single:
+        path, sig, sig_derivs = path[None], np.asarray(sig)[None], np.asarray(sig_derivs)[None]
+    batch, length, dim = path.shape
+    suf, real = _suffix(path.dtype)
+    full = sig_length(_aug_dim(dim, time_aug, lead_lag), degree)
+    sig = np.ascontiguousarray(sig, dtype=path.dtype)
+    sig_derivs = np.ascontiguousarray(sig_derivs, dtype=path.dtype)
+    if sig.shape[-1] == full:
+        scalar_term = True
+    elif sig.shape[-1] == full - 1:
+        scalar_term = False
+    else:
+        raise ValueError("sig has the wrong width")
+    if sig_derivs.shape != sig.shape:
+        raise ValueError("sig_derivs and sig must have the same shape")
+    out = np.empty_like(path)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_backprop_" + suf)(
+        path.ctypes.data_as(ptr), out.ctypes.data_as(ptr), sig_derivs.ctypes.data_as(ptr),
+        sig.ctypes.data_as(ptr), batch, dim, length, degree, int(time_aug), int(lead_lag),
+        float(end_time), int(scalar_term), n_jobs)
+    if rc:
+        raise RuntimeError("sigref_sig_backprop returned %d" % rc)
+    return out[0] if single else out

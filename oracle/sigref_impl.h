@@ -1,0 +1,389 @@
+/*
+ * sigref_impl.h -- type-generic body of the CPU oracle (TEST INFRASTRUCTURE ONLY).
+ *
+ * Included twice by sigref.c, once with REAL=float / SUF=_f and once with
+ * REAL=double / SUF=_d.  Every function restates, in plain C, what one function
+ * of the reference CPU library computes; the reference location is cited above
+ * each function (paths relative to the reference repository root).
+ *
+ * Buffers called "full" carry the scalar term at index 0 and level k starts at
+ * offset lvl[k] = (d^k - 1)/(d - 1).
+ */
+
+#define CAT_(a, b) a##b
+#define CAT(a, b) CAT_(a, b)
+#define FN(name) CAT(name, SUF)
+
+/* Virtual augmented path: siglib/cpsig/cp_path.h:46-62 (dims), :207-385 (points).
+ * lead-lag: point i has lag = x[i/2], lead = x[i/2 + (i odd)]; time is the last
+ * channel.  The reference keeps `time` as a running value advanced by
+ * += time_step / -= time_step from the position the iterator was created at;
+ * callers below reproduce that by carrying the time of each of their two
+ * cursors themselves and passing it in. */
+typedef struct {
+    const REAL *x;
+    uint64_t d_raw, len_raw;
+    uint64_t d, len;
+    int time_aug, lead_lag;
+    REAL time_step;
+} FN(vpath);
+
+static void FN(vpath_init)(FN(vpath) *p, const REAL *x, uint64_t d_raw, uint64_t len_raw,
+                           int time_aug, int lead_lag, REAL end_time)
+{
+    p->x = x;
+    p->d_raw = d_raw;
+    p->len_raw = len_raw;
+    p->time_aug = time_aug;
+    p->lead_lag = lead_lag;
+    p->d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    p->len = lead_lag ? 2 * len_raw - 1 : len_raw;
+    p->time_step = p->len > 1 ? end_time / (REAL)(p->len - 1) : (REAL)0;
+}
+
+/* value of channel c of augmented point i, given that point's running time */
+static inline REAL FN(vpath_at)(const FN(vpath) *p, uint64_t i, uint64_t c, REAL time)
+{
+    if (!p->lead_lag) {
+        if (c < p->d_raw) return p->x[i * p->d_raw + c];
+        return time;
+    }
+    const uint64_t row = i / 2, odd = i & 1;
+    if (c < p->d_raw) return p->x[row * p->d_raw + c];
+    if (c < 2 * p->d_raw) return p->x[(row + odd) * p->d_raw + (c - p->d_raw)];
+    return time;
+}
+
+/* siglib/cpsig/cp_signature.h:365-389 linear_signature_: exp of one segment,
+ * level k = level (k-1) (x) z / k.  `full` layout. */
+static void FN(segment_exp)(const REAL *z, REAL *out, uint64_t d, uint64_t degree, const uint64_t *lvl)
+{
+    out[0] = (REAL)1;
+    if (degree == 0) return;
+    for (uint64_t i = 0; i < d; ++i) out[1 + i] = z[i];
+    for (uint64_t k = 2; k <= degree; ++k) {
+        const REAL inv = (REAL)1 / (REAL)k;
+        const REAL *left = out + lvl[k - 1];
+        REAL *res = out + lvl[k];
+        const uint64_t nleft = lvl[k] - lvl[k - 1];
+        for (uint64_t i = 0; i < nleft; ++i) {
+            const REAL s = left[i] * inv;
+            for (uint64_t j = 0; j < d; ++j) res[i * d + j] = out[1 + j] * s;
+        }
+    }
+}
+
+/* siglib/cpsig/cp_signature.h:464-499 (loop body of signature_horner_) and
+ * :549-603 signature_horner_step_: S <- S (x) exp(z), Horner form, in place,
+ * descending target level so lower levels still hold the old values.
+ * `h` needs d^(degree-1) entries. */
+static void FN(horner_step)(REAL *S, const REAL *z, uint64_t d, uint64_t degree,
+                            const uint64_t *lvl, REAL *h)
+{
+    for (uint64_t t = degree; t > 1; --t) {
+        const REAL inv_t = (REAL)1 / (REAL)t;
+        for (uint64_t i = 0; i < d; ++i) h[i] = z[i] * inv_t;
+        for (uint64_t l = 1; l + 1 < t; ++l) {
+            const uint64_t n = lvl[l + 1] - lvl[l];
+            const REAL inv = (REAL)1 / (REAL)(t - l);
+            const REAL *Sl = S + lvl[l];
+            for (uint64_t i = n; i-- > 0;) {
+                const REAL s = (h[i] + Sl[i]) * inv;
+                for (uint64_t j = 0; j < d; ++j) h[i * d + j] = z[j] * s;
+            }
+        }
+        const uint64_t n = lvl[t] - lvl[t - 1];
+        const REAL *Sl = S + lvl[t - 1];
+        REAL *St = S + lvl[t];
+        for (uint64_t i = n; i-- > 0;) {
+            const REAL s = h[i] + Sl[i];
+            for (uint64_t j = 0; j < d; ++j) St[i * d + j] += z[j] * s;
+        }
+    }
+    for (uint64_t j = 0; j < d; ++j) S[1 + j] += z[j];
+}
+
+/* siglib/cpsig/cp_sig_combine.h:35-66 sig_combine_inplace_: a <- a (x) b. */
+static void FN(chen_inplace)(REAL *a, const REAL *b, uint64_t degree, const uint64_t *lvl)
+{
+    a[0] = (REAL)1;
+    for (uint64_t t = degree; t > 0; --t) {
+        REAL *res = a + lvl[t];
+        for (uint64_t left = t - 1; left > 0; --left) {
+            const uint64_t right = t - left;
+            const uint64_t nl = lvl[left + 1] - lvl[left];
+            const uint64_t nr = lvl[right + 1] - lvl[right];
+            const REAL *al = a + lvl[left];
+            const REAL *br = b + lvl[right];
+            for (uint64_t i = 0; i < nl; ++i)
+                for (uint64_t j = 0; j < nr; ++j) res[i * nr + j] += al[i] * br[j];
+        }
+        const uint64_t nt = lvl[t + 1] - lvl[t];
+        for (uint64_t j = 0; j < nt; ++j) res[j] += b[lvl[t] + j];
+    }
+}
+
+/* One path, full layout.  horner != 0: siglib/cpsig/cp_signature.h:426-500
+ * signature_horner_; horner == 0: :391-424 signature_naive_.  Requires
+ * p->len >= 2 and degree >= 2. */
+static int FN(one_path_sig)(const FN(vpath) *p, REAL *out, uint64_t degree, int horner)
+{
+    const uint64_t d = p->d;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *z = (REAL *)malloc(d * sizeof(REAL));
+    if (!lvl || !z) { free(lvl); free(z); return 1; }
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t full = lvl[degree + 1];
+    const uint64_t hsz = horner ? (lvl[degree] - lvl[degree - 1]) : full;
+    REAL *work = (REAL *)malloc(hsz * sizeof(REAL));
+    if (!work) { free(lvl); free(z); return 1; }
+
+    REAL t_prev = (REAL)0, t_next = p->time_step; /* cursors start at indices 0 and 1 */
+    for (uint64_t i = 0; i < d; ++i) z[i] = FN(vpath_at)(p, 1, i, t_next) - FN(vpath_at)(p, 0, i, t_prev);
+    FN(segment_exp)(z, out, d, degree, lvl);
+
+    for (uint64_t s = 1; s + 1 < p->len; ++s) {
+        t_prev += p->time_step;
+        t_next += p->time_step;
+        for (uint64_t i = 0; i < d; ++i)
+            z[i] = FN(vpath_at)(p, s + 1, i, t_next) - FN(vpath_at)(p, s, i, t_prev);
+        if (horner) {
+            FN(horner_step)(out, z, d, degree, lvl, work);
+        } else {
+            FN(segment_exp)(z, work, d, degree, lvl);
+            FN(chen_inplace)(out, work, degree, lvl);
+        }
+    }
+    free(work); free(z); free(lvl);
+    return 0;
+}
+
+/* siglib/cpsig/cp_signature.h:1098-1203 sig_backprop_inplace_: reverse sweep for
+ * one path.  S (full layout, signature of the whole path) and G (full layout,
+ * upstream gradient, scalar slot ignored) are both overwritten.  out has
+ * len_raw*d_raw entries, already zeroed. */
+static int FN(one_path_backprop)(const FN(vpath) *p, REAL *out, REAL *G, REAL *S, uint64_t degree)
+{
+    const uint64_t d = p->d, dr = p->d_raw;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    if (!lvl) return 1;
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t top = lvl[degree] - lvl[degree - 1]; /* d^(degree-1) */
+    REAL *h = (REAL *)malloc((lvl[degree] ? lvl[degree] : 1) * sizeof(REAL));
+    REAL *hd = (REAL *)malloc((top ? top : 1) * sizeof(REAL));
+    REAL *z = (REAL *)malloc(3 * d * sizeof(REAL));
+    REAL *hs = (REAL *)malloc((top ? top : 1) * sizeof(REAL));
+    if (!h || !hd || !z || !hs) { free(lvl); free(h); free(hd); free(z); free(hs); return 1; }
+    REAL *dz = z + d, *part = z + 2 * d;
+
+    /* cursors: prev at index len-2, next at len-1; both iterators were created
+     * at end() (time = len*time_step) and walked back with -= time_step */
+    REAL t_next = (REAL)p->len * p->time_step;
+    REAL t_prev = t_next;
+    t_prev -= p->time_step; t_prev -= p->time_step;
+    t_next -= p->time_step;
+    uint64_t pos = p->len_raw - 1; /* raw row that receives +dz */
+    int parity = 0;
+
+    for (uint64_t s = p->len - 1; s > 0; --s) { /* segment (s-1) -> s */
+        for (uint64_t i = 0; i < d; ++i)
+            z[i] = FN(vpath_at)(p, s - 1, i, t_prev) - FN(vpath_at)(p, s, i, t_next);
+        FN(horner_step)(S, z, d, degree, lvl, hs); /* un-multiply: S <- S (x) exp(-dx) */
+        for (uint64_t i = 0; i < d; ++i) { z[i] = -z[i]; dz[i] = G[1 + i]; }
+
+        for (uint64_t T = 2; T <= degree; ++T) {
+            const REAL inv_T = (REAL)1 / (REAL)T;
+            for (uint64_t i = 0; i < d; ++i) h[1 + i] = z[i] * inv_T;
+            for (uint64_t l = 1; l + 1 < T; ++l) {
+                const uint64_t n = lvl[l + 1] - lvl[l];
+                const REAL sc = (REAL)1 / (REAL)(T - l);
+                for (uint64_t i = 0; i < n; ++i) {
+                    const REAL v = (h[lvl[l] + i] + S[lvl[l] + i]) * sc;
+                    for (uint64_t j = 0; j < d; ++j) h[lvl[l + 1] + i * d + j] = z[j] * v;
+                }
+            }
+            const REAL *incoming = G + lvl[T];
+            for (uint64_t l = T - 1; l > 0; --l) {
+                const uint64_t n = lvl[l + 1] - lvl[l];
+                const REAL sc = (REAL)1 / (REAL)(T - l);
+                for (uint64_t j = 0; j < d; ++j) part[j] = (REAL)0;
+                for (uint64_t i = 0; i < n; ++i) {
+                    const REAL v = (h[lvl[l] + i] + S[lvl[l] + i]) * sc;
+                    const REAL *row = incoming + i * d;
+                    REAL red = (REAL)0;
+                    for (uint64_t j = 0; j < d; ++j) {
+                        part[j] += row[j] * v;
+                        red += row[j] * z[j];
+                    }
+                    red *= sc;
+                    hd[i] = red;
+                    G[lvl[l] + i] += red;
+                }
+                for (uint64_t j = 0; j < d; ++j) dz[j] += part[j];
+                incoming = hd;
+            }
+            for (uint64_t i = 0; i < d; ++i) dz[i] += hd[i] * inv_T;
+        }
+
+        /* siglib/cpsig/cp_signature.h:1189-1201: raw channels only; with lead-lag
+         * the odd->even segment moved the lag half, the even->odd one the lead half */
+        const REAL *src = dz + ((p->lead_lag && parity) ? dr : 0);
+        for (uint64_t c = 0; c < dr; ++c) {
+            out[pos * dr + c] += src[c];
+            out[(pos - 1) * dr + c] -= src[c];
+        }
+        if (s > 1) {
+            t_prev -= p->time_step;
+            t_next -= p->time_step;
+            if (!p->lead_lag || parity) --pos;
+            parity = !parity;
+        }
+    }
+    free(lvl); free(h); free(hd); free(z); free(hs);
+    return 0;
+}
+
+/* ---- batch drivers -------------------------------------------------------- */
+
+typedef struct {
+    const REAL *path; REAL *out;
+    const REAL *derivs; const REAL *sig;
+    uint64_t d_raw, len_raw, degree;
+    int time_aug, lead_lag, horner, scalar_term;
+    REAL end_time;
+    uint64_t full_len, stride;
+    int status;
+} FN(job);
+
+static void FN(sig_worker)(void *ctx, uint64_t b0, uint64_t b1)
+{
+    FN(job) *J = (FN(job) *)ctx;
+    REAL *buf = NULL;
+    if (!J->scalar_term) {
+        buf = (REAL *)malloc(J->full_len * sizeof(REAL));
+        if (!buf) { J->status = 1; return; }
+    }
+    for (uint64_t b = b0; b < b1; ++b) {
+        FN(vpath) p;
+        FN(vpath_init)(&p, J->path + b * J->d_raw * J->len_raw, J->d_raw, J->len_raw,
+                       J->time_aug, J->lead_lag, J->end_time);
+        REAL *o = J->out + b * J->stride;
+        if (J->degree == 1) {
+            /* siglib/cpsig/cp_signature.h:845-851,863-868: endpoint difference */
+            /* the end() cursor holds len*time_step and is stepped back once */
+            const REAL t_last = (REAL)p.len * p.time_step - p.time_step;
+            if (J->scalar_term) *o++ = (REAL)1;
+            for (uint64_t c = 0; c < p.d; ++c)
+                o[c] = FN(vpath_at)(&p, p.len - 1, c, t_last) - FN(vpath_at)(&p, 0, c, (REAL)0);
+            continue;
+        }
+        REAL *dst = J->scalar_term ? o : buf;
+        const int rc = FN(one_path_sig)(&p, dst, J->degree, J->horner);
+        if (rc) { J->status = rc; break; }
+        if (!J->scalar_term) memcpy(o, buf + 1, (J->full_len - 1) * sizeof(REAL));
+    }
+    free(buf);
+}
+
+/* siglib/cpsig/cp_signature.h:719-889 signature_ (the correction path and the
+ * small-dimension batch-SIMD path are alternative schedules of the same
+ * arithmetic and are not restated). */
+int FN(sigref_signature)(const REAL *path, REAL *out, uint64_t batch, uint64_t d_raw,
+                         uint64_t len_raw, uint64_t degree, int time_aug, int lead_lag,
+                         REAL end_time, int horner, int scalar_term, int n_jobs)
+{
+    if (d_raw == 0) return 2;
+    if (n_jobs == 0) return 2;
+    FN(vpath) p0;
+    FN(vpath_init)(&p0, NULL, d_raw, len_raw, time_aug, lead_lag, end_time);
+    const uint64_t full = sigref_sig_length(p0.d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+
+    if (len_raw == 0 || p0.len <= 1) {
+        for (uint64_t i = 0; i < stride * batch; ++i) out[i] = (REAL)0;
+        if (scalar_term)
+            for (uint64_t b = 0; b < batch; ++b) out[b * stride] = (REAL)1;
+        return 0;
+    }
+    if (degree == 0) {
+        if (scalar_term)
+            for (uint64_t b = 0; b < batch; ++b) out[b] = (REAL)1;
+        return 0;
+    }
+    if (p0.d == 1) {
+        /* siglib/cpsig/cp_signature.h:770-784: d == 1 closed form Delta^k / k! */
+        for (uint64_t b = 0; b < batch; ++b) {
+            const REAL *x = path + b * len_raw;
+            const REAL inc = x[len_raw - 1] - x[0];
+            REAL v = (REAL)1;
+            REAL *o = out + b * stride;
+            if (scalar_term) *o++ = v;
+            for (uint64_t k = 1; k <= degree; ++k) { v *= inc / (REAL)k; *o++ = v; }
+        }
+        return 0;
+    }
+    FN(job) J;
+    memset(&J, 0, sizeof J);
+    J.path = path; J.out = out; J.d_raw = d_raw; J.len_raw = len_raw; J.degree = degree;
+    J.time_aug = time_aug; J.lead_lag = lead_lag; J.horner = horner; J.scalar_term = scalar_term;
+    J.end_time = end_time; J.full_len = full; J.stride = stride; J.status = 0;
+    sigref_run_batch(batch, n_jobs, &J, FN(sig_worker));
+    return J.status;
+}
+
+static void FN(bp_worker)(void *ctx, uint64_t b0, uint64_t b1)
+{
+    FN(job) *J = (FN(job) *)ctx;
+    REAL *S = (REAL *)malloc(2 * J->full_len * sizeof(REAL));
+    if (!S) { J->status = 1; return; }
+    REAL *G = S + J->full_len;
+    for (uint64_t b = b0; b < b1; ++b) {
+        /* siglib/cpsig/cp_signature.h:958-975: work on private full-size copies,
+         * prepending sig[0] = 1 and deriv[0] = 0 when the scalar term is absent */
+        if (J->scalar_term) {
+            memcpy(S, J->sig + b * J->stride, J->full_len * sizeof(REAL));
+            memcpy(G, J->derivs + b * J->stride, J->full_len * sizeof(REAL));
+        } else {
+            S[0] = (REAL)1; G[0] = (REAL)0;
+            memcpy(S + 1, J->sig + b * J->stride, J->stride * sizeof(REAL));
+            memcpy(G + 1, J->derivs + b * J->stride, J->stride * sizeof(REAL));
+        }
+        FN(vpath) p;
+        FN(vpath_init)(&p, J->path + b * J->d_raw * J->len_raw, J->d_raw, J->len_raw,
+                       J->time_aug, J->lead_lag, J->end_time);
+        const int rc = FN(one_path_backprop)(&p, J->out + b * J->d_raw * J->len_raw, G, S, J->degree);
+        if (rc) { J->status = rc; break; }
+    }
+    free(S);
+}
+
+/* siglib/cpsig/cp_signature.h:909-1019 sig_backprop_ (general path; the
+ * small-signature batch-SIMD variant :42-227 is an alternative schedule of the
+ * same arithmetic and is not restated). */
+int FN(sigref_sig_backprop)(const REAL *path, REAL *out, const REAL *sig_derivs, const REAL *sig,
+                            uint64_t batch, uint64_t d_raw, uint64_t len_raw, uint64_t degree,
+                            int time_aug, int lead_lag, REAL end_time, int scalar_term, int n_jobs)
+{
+    for (uint64_t i = 0; i < batch * d_raw * len_raw; ++i) out[i] = (REAL)0;
+    if (d_raw == 0) return 2;
+    if (n_jobs == 0) return 2;
+    FN(vpath) p0;
+    FN(vpath_init)(&p0, NULL, d_raw, len_raw, time_aug, lead_lag, end_time);
+    const uint64_t full = sigref_sig_length(p0.d, degree);
+    if (full == 0) return 10;
+    if (len_raw == 0 || p0.len <= 1 || degree == 0) return 0;
+
+    FN(job) J;
+    memset(&J, 0, sizeof J);
+    J.path = path; J.out = out; J.derivs = sig_derivs; J.sig = sig;
+    J.d_raw = d_raw; J.len_raw = len_raw; J.degree = degree;
+    J.time_aug = time_aug; J.lead_lag = lead_lag; J.scalar_term = scalar_term;
+    J.end_time = end_time; J.full_len = full; J.stride = scalar_term ? full : full - 1; J.status = 0;
+    sigref_run_batch(batch, n_jobs, &J, FN(bp_worker));
+    return J.status;
+}
+
+#undef FN
+#undef CAT
+#undef CAT_
