@@ -1,0 +1,100 @@
+/*
+ * cusig_amd.h -- C ABI of the MI355X (gfx950) truncated-signature library.
+ *
+ * The shared object is named libcusig.so and exports, with identical names,
+ * argument lists and status codes, the entry points that the reference binds
+ * from its GPU plugin for the batched signature path, so the reference's
+ * Python loader and wrappers work on it unchanged.
+ *
+ * Conventions (all entry points):
+ *   - pointers are DEVICE pointers of the current HIP device; dense row-major
+ *     buffers allocated by the caller; inputs are never modified;
+ *   - `dimension` / `length` are the RAW path sizes (before lead-lag / time
+ *     augmentation);
+ *   - synchronous: device work has completed when the call returns;
+ *   - never throws; returns 0 on success, 1 allocation failure, 2 invalid
+ *     argument, 3 out of range, 10 runtime error (e.g. size overflow or a shape
+ *     this build has no kernel for), 11 unknown, 100000 + hipError_t for device
+ *     errors; a human-readable message for the calling thread is available from
+ *     cusig_last_error_message().
+ */
+#ifndef CUSIG_AMD_H
+#define CUSIG_AMD_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+#define CUSIG_AMD_NOEXCEPT noexcept
+extern "C" {
+#else
+#define CUSIG_AMD_NOEXCEPT
+#endif
+
+#define CUSIG_AMD_API __attribute__((visibility("default")))
+
+/* Truncated signature of a batch of paths.
+ * path [batch, length, dimension]; out [batch, S] with S = sum_{k=1..degree} d^k
+ * (+1 leading scalar when scalar_term), d = augmented dimension; level-major,
+ * row-major words inside a level.
+ * Replaces: siglib/cusig/cu_signature.cu:3497-3517 (signature_cuda_f / _d),
+ * bound by pysiglib/load_siglib.py:484-488, called from pysiglib/sig.py:288-294. */
+CUSIG_AMD_API int signature_cuda_f(const float* path, float* out, uint64_t batch_size, uint64_t dimension,
+                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag, float end_time,
+                                   bool horner, bool scalar_term, const float* correction,
+                                   uint64_t correction_len, uint64_t correction_batch_stride,
+                                   uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int signature_cuda_d(const double* path, double* out, uint64_t batch_size, uint64_t dimension,
+                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                   double end_time, bool horner, bool scalar_term, const double* correction,
+                                   uint64_t correction_len, uint64_t correction_batch_stride,
+                                   uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
+
+/* Gradient of a scalar loss w.r.t. the raw path, given the signature and the
+ * loss gradient w.r.t. the signature (both [batch, S], same layout as above).
+ * out [batch, length, dimension] is fully overwritten.
+ * Replaces: siglib/cusig/cu_signature.cu:3524-3544 (sig_backprop_cuda_f / _d),
+ * bound by pysiglib/load_siglib.py:490-494, called from pysiglib/sig_backprop.py:245-251. */
+CUSIG_AMD_API int sig_backprop_cuda_f(const float* path, float* out, const float* sig_derivs, const float* sig,
+                                      uint64_t batch_size, uint64_t dimension, uint64_t length, uint64_t degree,
+                                      bool time_aug, bool lead_lag, float end_time, bool scalar_term,
+                                      const float* correction, uint64_t correction_len,
+                                      uint64_t correction_batch_stride,
+                                      uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const double* sig_derivs,
+                                      const double* sig, uint64_t batch_size, uint64_t dimension,
+                                      uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                      double end_time, bool scalar_term, const double* correction,
+                                      uint64_t correction_len, uint64_t correction_batch_stride,
+                                      uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
+
+/* Message of the last failing call made by the calling thread ("" if none).
+ * Replaces: cusig_last_error_message, probed by pysiglib/load_siglib.py:108-110
+ * and read by pysiglib/error_codes.py:28-42. */
+CUSIG_AMD_API const char* cusig_last_error_message(void) CUSIG_AMD_NOEXCEPT;
+
+/* Releases the library's device workspaces; idempotent, never fails.
+ * Replaces: siglib/cusig/cache_lifecycle/cusig_lifecycle.cu:31-50, registered at
+ * interpreter exit by pysiglib/load_siglib.py:647-664. */
+CUSIG_AMD_API void cusig_shutdown(void) CUSIG_AMD_NOEXCEPT;
+
+/* (d^(degree+1) - 1)/(d - 1), 0 on 64-bit overflow.  Same contract as the CPU
+ * library's sig_length (siglib/cpsig/cp_utils.cpp:91-105), which the reference's
+ * Python wrapper calls to size its outputs (pysiglib/sig_length.py:91-94). */
+CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree) CUSIG_AMD_NOEXCEPT;
+
+/* Measurement hooks used by the benchmark (no counterpart in the reference):
+ * when enabled, the sweep kernel of every following call is bracketed with HIP
+ * events on the stream it is launched on. */
+CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
+/* Which kernel instance serves (dtype, augmented dimension, degree): returns 1 and
+ * fills tail / k / specialised, or 0 if the shape has no kernel. */
+CUSIG_AMD_API int cusig_amd_kernel_choice(int backward, int is_f64, uint64_t dimension, uint64_t degree,
+                                          int* tail, int* k, int* specialised) CUSIG_AMD_NOEXCEPT;
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUSIG_AMD_H */

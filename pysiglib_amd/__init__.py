@@ -1,0 +1,9 @@
+"""MI355X-native batched truncated path signatures (forward and backward).
+
+Drop-in for ``pysiglib.sig`` / ``pysiglib.sig_backprop`` / ``pysiglib.torch_api.sig`` on GPU tensors.
+"""
+from . import torch_api
+from .sig import sig, sig_backprop, signature
+from .sig_length import sig_length
+
+__all__ = ["sig", "signature", "sig_backprop", "sig_length", "torch_api"]

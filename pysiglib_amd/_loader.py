@@ -1,0 +1,72 @@
+"""Loads the HIP shared library ``csrc/libcusig.so`` and binds its C ABI.
+
+Mirrors the role of the reference's loader for its GPU plugin
+(pysiglib/load_siglib.py:73-130,484-494,647-664): per-dtype function tables for
+the two hot entry points, the last-error getter and a shutdown hook at exit.
+There is no CPU fallback: if the library is missing, importing this module
+raises.
+"""
+import atexit
+import ctypes
+import os
+from ctypes import POINTER, c_bool, c_char_p, c_double, c_float, c_int, c_uint64
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libcusig.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "pysiglib_amd: %s is missing. Build it first: python -c 'import __graft_entry__ as g; g.build()' "
+        "(or `make -C pysiglib_amd/csrc gen all`)." % LIB_PATH)
+
+CUSIG = ctypes.CDLL(LIB_PATH)
+
+CUSIG.cusig_last_error_message.argtypes = ()
+CUSIG.cusig_last_error_message.restype = c_char_p
+CUSIG.cusig_shutdown.argtypes = ()
+CUSIG.cusig_shutdown.restype = None
+CUSIG.cusig_amd_sig_length.argtypes = (c_uint64, c_uint64)
+CUSIG.cusig_amd_sig_length.restype = c_uint64
+CUSIG.cusig_amd_set_profiling.argtypes = (c_int,)
+CUSIG.cusig_amd_set_profiling.restype = None
+CUSIG.cusig_amd_last_kernel_ms.argtypes = ()
+CUSIG.cusig_amd_last_kernel_ms.restype = c_float
+CUSIG.cusig_amd_last_kernel_name.argtypes = ()
+CUSIG.cusig_amd_last_kernel_name.restype = c_char_p
+CUSIG.cusig_amd_kernel_choice.argtypes = (c_int, c_int, c_uint64, c_uint64, POINTER(c_int), POINTER(c_int), POINTER(c_int))
+CUSIG.cusig_amd_kernel_choice.restype = c_int
+
+DTYPES = {"float32": c_float, "float64": c_double}
+_SUFFIX = {"float32": "_f", "float64": "_d"}
+
+
+def _table(name, argtypes_of):
+    table = {}
+    for dtype, real in DTYPES.items():
+        fn = getattr(CUSIG, name + _SUFFIX[dtype])
+        fn.argtypes = argtypes_of(real)
+        fn.restype = c_int
+        table[dtype] = fn
+    return table
+
+
+CUSIG_SIGNATURE = _table("signature_cuda", lambda r: (
+    POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_uint64, c_bool, c_bool, r, c_bool, c_bool,
+    POINTER(r), c_uint64, c_uint64, c_uint64))
+
+CUSIG_SIG_BACKPROP = _table("sig_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_uint64, c_bool, c_bool, r,
+    c_bool, POINTER(r), c_uint64, c_uint64, c_uint64))
+
+
+def last_error_message():
+    msg = CUSIG.cusig_last_error_message()
+    return msg.decode("utf-8", errors="replace") if msg else ""
+
+
+@atexit.register
+def _shutdown():
+    try:
+        CUSIG.cusig_shutdown()
+    except Exception:  # pragma: no cover - interpreter teardown
+        pass

@@ -1,0 +1,487 @@
+// C ABI of the MI355X signature library: the four hot entry points of the
+// reference's GPU plugin (siglib/cusig/cu_signature.cu:3494-3545) plus its
+// lifecycle symbols, re-implemented on the gfx950 tree kernels.
+//
+// Every entry point is synchronous (device work has completed on return), never
+// throws across the ABI, returns the reference's status codes
+// (siglib/cusig/cu_macros.h:27-89) and leaves a message in a thread-local buffer
+// (siglib/shared/last_error.h:22-41).
+#include <hip/hip_runtime.h>
+
+#include <charconv>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+
+#include "../../include/cusig_amd.h"
+#include "sig_kernels.h"
+#include "sig_registry.h"
+
+namespace sigamd {
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+static thread_local char g_last_error[4096] = {0};
+
+static void clear_last_error() { g_last_error[0] = 0; }
+static void set_last_error(const char* msg)
+{
+    std::snprintf(g_last_error, sizeof g_last_error, "%s", msg ? msg : "");
+}
+
+struct HipFailure : std::runtime_error {
+    int code;
+    HipFailure(hipError_t e, const char* what_)
+        : std::runtime_error(std::string("HIP Error (") + std::to_string(int(e)) + "): " + hipGetErrorString(e) +
+                             " [" + what_ + "]"),
+          code(int(e)) {}
+};
+
+#define SIG_HIP(call)                                              \
+    do {                                                           \
+        hipError_t e__ = (call);                                   \
+        if (e__ != hipSuccess) throw ::sigamd::HipFailure(e__, #call); \
+    } while (0)
+
+template <typename F>
+static int guarded(F&& body) noexcept
+{
+    clear_last_error();
+    try {
+        body();
+    } catch (const std::bad_alloc&) {
+        set_last_error("Failed to allocate memory");
+        return 1;
+    } catch (const std::invalid_argument& e) {
+        set_last_error(e.what());
+        return 2;
+    } catch (const std::out_of_range& e) {
+        set_last_error(e.what());
+        return 3;
+    } catch (const HipFailure& e) {
+        set_last_error(e.what());
+        (void)hipGetLastError();   // do not let a sticky launch error leak into the caller's next call
+        return 100000 + e.code;
+    } catch (const std::runtime_error& e) {
+        set_last_error(e.what());
+        return 10;
+    } catch (...) {
+        set_last_error("Unknown exception");
+        return 11;
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// sizes (siglib/cpsig/cp_utils.cpp:22-38,91-105): 0 signals uint64 overflow
+// ---------------------------------------------------------------------------
+static uint64_t pow_u64(uint64_t base, uint64_t e)
+{
+    uint64_t r = 1;
+    while (e > 0) {
+        if (e & 1) {
+            if (r != 0 && base > UINT64_MAX / r) return 0;
+            r *= base;
+        }
+        e >>= 1;
+        if (e > 0) {
+            if (base != 0 && base > UINT64_MAX / base) return 0;
+            base *= base;
+        }
+    }
+    return r;
+}
+
+static uint64_t sig_length_u64(uint64_t d, uint64_t degree)
+{
+    if (d == 0) return 1;
+    if (d == 1) return degree + 1;
+    const uint64_t p = pow_u64(d, degree + 1);
+    return p ? (p - 1) / (d - 1) : 0;
+}
+
+static uint64_t checked_mul(uint64_t a, uint64_t b, const char* what)
+{
+    if (a != 0 && b > UINT64_MAX / a) throw std::overflow_error(std::string(what) + ": size overflow");
+    return a * b;
+}
+
+// ---------------------------------------------------------------------------
+// kernel table
+// ---------------------------------------------------------------------------
+struct Table {
+    std::map<std::tuple<int, int, int>, const KernelEntry*> fwd, bwd;
+    Table()
+    {
+        int n = 0;
+        const EntryList* lists = all_entry_lists(&n);
+        for (int i = 0; i < n; ++i)
+            for (int j = 0; j < lists[i].count; ++j) {
+                const KernelEntry* e = &lists[i].entries[j];
+                auto key = std::make_tuple(e->is_f64, e->D, e->N);
+                if (e->fwd) fwd[key] = e;
+                if (e->bwd) bwd[key] = e;
+            }
+    }
+};
+
+static const Table& table()
+{
+    static const Table t;
+    return t;
+}
+
+static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64_t degree)
+{
+    const auto& m = backward ? table().bwd : table().fwd;
+    if (d <= 0x7fffffff && degree <= 0x7fffffff) {
+        auto it = m.find(std::make_tuple(int(f64), int(d), int(degree)));
+        if (it != m.end()) return it->second;
+        it = m.find(std::make_tuple(int(f64), 0, int(degree)));
+        if (it != m.end()) return it->second;
+    }
+    return nullptr;
+}
+
+// ---------------------------------------------------------------------------
+// per-device workspace (grow-only; released by cusig_shutdown).  The mutex also
+// serialises concurrent host threads on the shared buffers, as the reference
+// does for its backward workspaces (siglib/cusig/cu_signature.cu:2971).
+// ---------------------------------------------------------------------------
+struct Workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+static std::mutex g_ws_mutex;
+static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
+
+static void* workspace(int slot, size_t bytes)
+{
+    int dev = 0;
+    SIG_HIP(hipGetDevice(&dev));
+    Workspace& w = g_ws[{dev, slot}];
+    if (w.bytes < bytes) {
+        if (w.ptr) {
+            SIG_HIP(hipFree(w.ptr));
+            w.ptr = nullptr;
+            w.bytes = 0;
+        }
+        const size_t want = bytes + bytes / 8;
+        if (hipMalloc(&w.ptr, want) != hipSuccess) {
+            (void)hipGetLastError();
+            w.ptr = nullptr;
+            throw std::bad_alloc();
+        }
+        w.bytes = want;
+    }
+    return w.ptr;
+}
+
+static void release_workspaces() noexcept
+{
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    for (auto& kv : g_ws) {
+        if (kv.second.ptr) {
+            int cur = 0;
+            if (hipGetDevice(&cur) == hipSuccess && hipSetDevice(kv.first.first) == hipSuccess) {
+                (void)hipFree(kv.second.ptr);
+                (void)hipSetDevice(cur);
+            }
+        }
+    }
+    g_ws.clear();
+    (void)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// kernel timing hook for the benchmark
+// ---------------------------------------------------------------------------
+static bool g_profile = false;
+static float g_last_ms = -1.f;
+static char g_last_name[128] = {0};
+static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+
+struct MainKernelTimer {
+    hipStream_t s;
+    bool on;
+    MainKernelTimer(hipStream_t stream, const char* name) : s(stream), on(g_profile)
+    {
+        if (!on) return;
+        if (!g_ev0) {
+            SIG_HIP(hipEventCreate(&g_ev0));
+            SIG_HIP(hipEventCreate(&g_ev1));
+        }
+        std::snprintf(g_last_name, sizeof g_last_name, "%s", name);
+        SIG_HIP(hipEventRecord(g_ev0, s));
+    }
+    void stop()
+    {
+        if (!on) return;
+        SIG_HIP(hipEventRecord(g_ev1, s));
+        SIG_HIP(hipEventSynchronize(g_ev1));
+        SIG_HIP(hipEventElapsedTime(&g_last_ms, g_ev0, g_ev1));
+    }
+};
+
+// ---------------------------------------------------------------------------
+// shared argument handling
+// ---------------------------------------------------------------------------
+static void validate_correction(const void* correction, uint64_t correction_len, uint64_t dimension,
+                                uint64_t degree, bool lead_lag)
+{
+    // siglib/cpsig/cp_signature.h:229-256
+    if (correction == nullptr && correction_len != 0)
+        throw std::invalid_argument("correction pointer is null but correction_len is nonzero");
+    if (lead_lag && correction_len != 0)
+        throw std::invalid_argument("correction cannot be used with lead_lag=true");
+    if (correction_len == 0) return;
+    if (degree < 2) throw std::invalid_argument("correction must be empty when degree < 2");
+    uint64_t offset = 0, level_size = dimension;
+    bool ok = false;
+    for (uint64_t level = 2; level <= degree; ++level) {
+        level_size *= dimension;
+        offset += level_size;
+        if (offset == correction_len) { ok = true; break; }
+        if (offset > correction_len) break;
+    }
+    if (!ok) throw std::invalid_argument("correction length must be a prefix of tensor levels 2..degree");
+    throw std::runtime_error("per-segment correction is not implemented in this build");
+}
+
+static unsigned grid_for(uint64_t work)
+{
+    uint64_t blocks = (work + kBlock - 1) / kBlock;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+    return unsigned(blocks);
+}
+
+struct Shape {
+    uint64_t d_aug, len_aug, L, full_len, stride;
+};
+
+static Shape make_shape(uint64_t dimension, uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                        bool scalar_term)
+{
+    Shape s;
+    s.d_aug = (lead_lag ? 2 * dimension : dimension) + (time_aug ? 1 : 0);
+    s.len_aug = (lead_lag && length > 0) ? 2 * length - 1 : length;
+    s.L = s.len_aug > 0 ? s.len_aug - 1 : 0;
+    s.full_len = sig_length_u64(s.d_aug, degree);
+    if (s.full_len == 0) throw std::overflow_error("signature length overflows 64 bits");
+    s.stride = scalar_term ? s.full_len : s.full_len - 1;
+    return s;
+}
+
+template <typename T>
+static void compute_increments(const T* path, T* inc, uint64_t batch, uint64_t dimension, uint64_t length,
+                               bool time_aug, bool lead_lag, T end_time, const Shape& s, hipStream_t stream)
+{
+    const T time_step = s.len_aug > 1 ? end_time / T(s.len_aug - 1) : T(0);
+    hipLaunchKernelGGL((increments_kernel<T>), dim3(grid_for(batch * s.L * s.d_aug)), dim3(kBlock), 0, stream,
+                       path, inc, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
+                       int(lead_lag), time_step);
+    SIG_HIP(hipGetLastError());
+}
+
+// ---------------------------------------------------------------------------
+// forward  (dispatch mirrors siglib/cpsig/cp_signature.h:740-851 and
+// siglib/cusig/cu_signature.cu:2592-2657)
+// ---------------------------------------------------------------------------
+template <typename T>
+static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimension, uint64_t length,
+                           uint64_t degree, bool time_aug, bool lead_lag, T end_time, bool /*horner*/,
+                           bool scalar_term, const T* correction, uint64_t correction_len)
+{
+    if (dimension == 0) throw std::invalid_argument("signature_cuda received path of dimension 0");
+    validate_correction(correction, correction_len, dimension, degree, lead_lag);
+    if (batch == 0) return;
+    if (dimension > 0x3fffffff || degree > 0x7fffffff || length > (uint64_t(1) << 40))
+        throw std::invalid_argument("signature_cuda: shape out of range");
+    const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
+    checked_mul(checked_mul(batch, s.stride, "signature output"), sizeof(T), "signature output");
+    hipStream_t stream = nullptr;
+    SIG_HIP(hipDeviceSynchronize());   // inputs may have been produced on any stream
+
+    const int sc = scalar_term ? 1 : 0;
+    if (s.len_aug <= 1) {
+        if (s.stride)
+            hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
+                               out, int64_t(batch), int64_t(s.stride), sc);
+    } else if (degree == 0) {
+        if (scalar_term)
+            hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out,
+                               int64_t(batch), int64_t(1), 1);
+    } else if (s.d_aug == 1) {
+        hipLaunchKernelGGL((dim_one_fwd_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, path, out,
+                           int64_t(batch), int64_t(length), int(degree), sc);
+    } else if (degree == 1) {
+        const T time_step = end_time / T(s.len_aug - 1);
+        hipLaunchKernelGGL((degree_one_fwd_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
+                           path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
+                           int(lead_lag), time_step, sc);
+    } else {
+        const KernelEntry* e = find_entry(false, sizeof(T) == 8, s.d_aug, degree);
+        if (!e)
+            throw std::runtime_error("signature_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
+                                     ", degree " + std::to_string(degree) + " in this build");
+        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+        FwdParams p;
+        p.inc = inc; p.out = out; p.batch = int64_t(batch); p.L = int64_t(s.L); p.d = int(s.d_aug);
+        p.out_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
+        MainKernelTimer timer(stream, e->name);
+        SIG_HIP(e->fwd(p));
+        timer.stop();
+        SIG_HIP(hipStreamSynchronize(stream));
+        return;
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+// ---------------------------------------------------------------------------
+// backward  (siglib/cpsig/cp_signature.h:909-1019, siglib/cusig/cu_signature.cu:3417-3488)
+// ---------------------------------------------------------------------------
+template <typename T>
+static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const T* sig, uint64_t batch,
+                              uint64_t dimension, uint64_t length, uint64_t degree, bool time_aug,
+                              bool lead_lag, T end_time, bool scalar_term, const T* correction,
+                              uint64_t correction_len)
+{
+    if (dimension == 0) throw std::invalid_argument("sig_backprop_cuda received path of dimension 0");
+    validate_correction(correction, correction_len, dimension, degree, lead_lag);
+    if (batch == 0) return;
+    if (dimension > 0x3fffffff || degree > 0x7fffffff || length > (uint64_t(1) << 40))
+        throw std::invalid_argument("sig_backprop_cuda: shape out of range");
+    const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
+    const uint64_t out_elems = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
+    hipStream_t stream = nullptr;
+    SIG_HIP(hipDeviceSynchronize());
+    const int sc = scalar_term ? 1 : 0;
+
+    if (s.len_aug <= 1 || degree == 0) {
+        if (out_elems)
+            hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, out,
+                               int64_t(out_elems));
+    } else if (degree == 1) {
+        hipLaunchKernelGGL((degree_one_bwd_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream,
+                           sig_derivs, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
+                           int(lead_lag), sc);
+    } else {
+        const KernelEntry* e = find_entry(true, sizeof(T) == 8, s.d_aug, degree);
+        if (!e)
+            throw std::runtime_error("sig_backprop_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
+                                     ", degree " + std::to_string(degree) + " in this build");
+        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        const size_t inc_bytes = checked_mul(inc_elems, sizeof(T), "increments");
+        T* inc = static_cast<T*>(workspace(0, inc_bytes));
+        T* dzinc = static_cast<T*>(workspace(1, inc_bytes));
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+        hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(inc_elems)), dim3(kBlock), 0, stream, dzinc,
+                           int64_t(inc_elems));
+        SIG_HIP(hipGetLastError());
+        BwdParams p;
+        p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
+        p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
+        MainKernelTimer timer(stream, e->name);
+        SIG_HIP(e->bwd(p));
+        timer.stop();
+        hipLaunchKernelGGL((path_grad_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, dzinc, out,
+                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+        SIG_HIP(hipGetLastError());
+        SIG_HIP(hipStreamSynchronize(stream));
+        return;
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+}  // namespace sigamd
+
+using namespace sigamd;
+
+extern "C" {
+
+CUSIG_AMD_API int signature_cuda_f(const float* path, float* out, uint64_t batch_size, uint64_t dimension,
+                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag, float end_time,
+                                   bool horner, bool scalar_term, const float* correction,
+                                   uint64_t correction_len, uint64_t, uint64_t) noexcept
+{
+    return guarded([&] {
+        signature_impl<float>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
+                              horner, scalar_term, correction, correction_len);
+    });
+}
+
+CUSIG_AMD_API int signature_cuda_d(const double* path, double* out, uint64_t batch_size, uint64_t dimension,
+                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                   double end_time, bool horner, bool scalar_term, const double* correction,
+                                   uint64_t correction_len, uint64_t, uint64_t) noexcept
+{
+    return guarded([&] {
+        signature_impl<double>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
+                               horner, scalar_term, correction, correction_len);
+    });
+}
+
+CUSIG_AMD_API int sig_backprop_cuda_f(const float* path, float* out, const float* sig_derivs, const float* sig,
+                                      uint64_t batch_size, uint64_t dimension, uint64_t length, uint64_t degree,
+                                      bool time_aug, bool lead_lag, float end_time, bool scalar_term,
+                                      const float* correction, uint64_t correction_len, uint64_t,
+                                      uint64_t) noexcept
+{
+    return guarded([&] {
+        sig_backprop_impl<float>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
+                                 lead_lag, end_time, scalar_term, correction, correction_len);
+    });
+}
+
+CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const double* sig_derivs,
+                                      const double* sig, uint64_t batch_size, uint64_t dimension,
+                                      uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                      double end_time, bool scalar_term, const double* correction,
+                                      uint64_t correction_len, uint64_t, uint64_t) noexcept
+{
+    return guarded([&] {
+        sig_backprop_impl<double>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
+                                  lead_lag, end_time, scalar_term, correction, correction_len);
+    });
+}
+
+CUSIG_AMD_API const char* cusig_last_error_message(void) noexcept { return g_last_error; }
+
+CUSIG_AMD_API void cusig_shutdown(void) noexcept { release_workspaces(); }
+
+CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree) noexcept
+{
+    return sig_length_u64(dimension, degree);
+}
+
+CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) noexcept { g_profile = enabled != 0; }
+
+CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; }
+
+CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
+
+CUSIG_AMD_API int cusig_amd_kernel_choice(int backward, int is_f64, uint64_t dimension, uint64_t degree,
+                                          int* tail, int* k, int* specialised) noexcept
+{
+    const KernelEntry* e = find_entry(backward != 0, is_f64 != 0, dimension, degree);
+    if (!e) return 0;
+    if (tail) *tail = e->tail;
+    if (k) *k = e->k;
+    if (specialised) *specialised = e->D != 0;
+    return 1;
+}
+
+}  // extern "C"

@@ -1,0 +1,41 @@
+// Launch wrappers instantiated once per (T, D, N, TAIL, K).
+#pragma once
+#include "sig_kernels.h"
+#include "sig_registry.h"
+
+namespace sigamd {
+
+constexpr int64_t kMaxGridX = 2147483647LL;
+constexpr size_t kMaxDynLds = 64 * 1024;
+
+template <typename T, int D, int N, int TAIL, int K>
+hipError_t launch_tree_fwd(const FwdParams& p)
+{
+    const TreeGeom g = make_geom(p.d, N - TAIL, K);
+    const int64_t waves = total_waves(g, p.batch);
+    const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), 0, p.stream,
+                       static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
+                       p.out_stride, p.scalar);
+    return hipGetLastError();
+}
+
+template <typename T, int D, int N, int TAIL, int K>
+hipError_t launch_tree_bwd(const BwdParams& p)
+{
+    const TreeGeom g = make_geom(p.d, N - TAIL, K);
+    const int64_t waves = total_waves(g, p.batch);
+    const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
+    size_t lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
+    int use_lds = 1;
+    if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
+    hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
+                       static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
+                       static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,
+                       p.sig_stride, p.scalar, use_lds);
+    return hipGetLastError();
+}
+
+}  // namespace sigamd

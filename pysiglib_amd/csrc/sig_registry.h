@@ -1,0 +1,49 @@
+// Host-side table of compiled tree-kernel instances and their launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sigamd {
+
+struct FwdParams {
+    const void* inc;
+    void* out;
+    int64_t batch, L;
+    int d;
+    int64_t out_stride;
+    int scalar;
+    hipStream_t stream;
+};
+
+struct BwdParams {
+    const void* inc;
+    const void* sig;
+    const void* gsig;
+    void* dzinc;
+    int64_t batch, L;
+    int d;
+    int64_t sig_stride;
+    int scalar;
+    hipStream_t stream;
+};
+
+typedef hipError_t (*FwdFn)(const FwdParams&);
+typedef hipError_t (*BwdFn)(const BwdParams&);
+
+// D == 0: run-time dimension.  Exactly one of fwd / bwd is set.
+struct KernelEntry {
+    int is_f64, D, N, tail, k;
+    FwdFn fwd;
+    BwdFn bwd;
+    const char* name;
+};
+
+// every generated instance file contributes one array
+struct EntryList {
+    const KernelEntry* entries;
+    int count;
+};
+
+const EntryList* all_entry_lists(int* n_lists);   // defined in the generated registry
+
+}  // namespace sigamd

@@ -1,0 +1,316 @@
+// Register-resident prefix-tree kernels for the truncated path signature on gfx950.
+//
+// One lane owns a word prefix p of length M = N - TAIL together with
+//   * the chain  S_1[p_1], S_2[p_1 p_2], ..., S_M[p]           (M values, recomputed
+//     redundantly by every lane that shares part of the prefix), and
+//   * a slice of the subtree below p: at subtree depth 1 the K letters
+//     a0 .. a0+K-1 (a0 = K * group), below that all D letters, down to depth TAIL.
+// All of it lives in VGPRs for the whole sweep over the path; HBM sees the
+// increments (read through the scalar cache when a wave serves one path) and
+// one final store.  The update of a coefficient only reads coefficients of its
+// own prefixes, so lanes never exchange signature state.
+//
+// The arithmetic is the reference's Horner step
+// (siglib/cpsig/cp_signature.h:464-499 forward, :1137-1187 backward) regrouped
+// per word; see the comments on fwd_step / pullback below.
+//
+// D > 0: compile-time path dimension.  D == 0: run-time dimension (TAIL must be 1).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sigamd {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+__host__ __device__ constexpr int64_t ipow64(int64_t b, int e)
+{
+    int64_t r = 1;
+    for (int i = 0; i < e; ++i) r *= b;
+    return r;
+}
+
+template <typename T>
+__device__ __forceinline__ constexpr T rcp(int k) { return T(1) / T(k); }
+
+template <typename T>
+__device__ __forceinline__ T fmadd(T a, T b, T c) { return __builtin_fma(a, b, c); }
+template <>
+__device__ __forceinline__ float fmadd<float>(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+// Launch geometry shared by host and device.
+//   wide:   the prefixes of one path fill whole waves; lane order is group-major
+//           with the prefix range padded to a multiple of 64, so path index and
+//           group are wave-uniform (increments become scalar loads).
+//   packed: lanes of one path are contiguous (prefix-major, group fastest);
+//           if a path needs <= 64 lanes several whole paths share a wave,
+//           otherwise a path takes ceil(lanes/64) waves.
+struct TreeGeom {
+    int64_t P;          // number of prefixes D^M
+    int ng;             // groups at subtree depth 1
+    int wide;
+    int64_t p_pad;      // wide: P rounded up to 64
+    int64_t lpp;        // lanes per path (wide: ng * p_pad; packed: ng * P)
+    int ppw;            // packed, lpp <= 64: whole paths per wave, else 1
+    int64_t wpp;        // waves per path when a path spans waves, else 1
+};
+
+__host__ __device__ inline TreeGeom make_geom(int d, int m, int k)
+{
+    TreeGeom g;
+    g.P = ipow64(d, m);
+    g.ng = (d + k - 1) / k;
+    g.wide = g.P >= 48;
+    if (g.wide) {
+        g.p_pad = (g.P + kWave - 1) / kWave * kWave;
+        g.lpp = g.ng * g.p_pad;
+        g.ppw = 1;
+        g.wpp = g.lpp / kWave;
+    } else {
+        g.p_pad = g.P;
+        g.lpp = g.ng * g.P;
+        if (g.lpp <= kWave) { g.ppw = int(kWave / g.lpp); g.wpp = 1; }
+        else { g.ppw = 1; g.wpp = (g.lpp + kWave - 1) / kWave; }
+    }
+    return g;
+}
+
+inline int64_t total_waves(const TreeGeom& g, int64_t batch)
+{
+    if (g.ppw > 1) return (batch + g.ppw - 1) / g.ppw;
+    return batch * g.wpp;
+}
+
+struct LaneId {
+    int64_t b;      // path index
+    int64_t q;      // prefix number in [0, P)
+    int g;          // group
+    int slot;       // index of the path inside its wave (packed, several paths per wave)
+    bool active;
+};
+
+template <bool WIDE>
+__device__ __forceinline__ LaneId lane_id(const TreeGeom& G, int64_t batch)
+{
+    LaneId id;
+    const int lane = threadIdx.x & (kWave - 1);
+    int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    id.slot = 0;
+    if constexpr (WIDE) {
+        // wave-uniform quantities are forced into SGPRs
+        const uint32_t wlo = __builtin_amdgcn_readfirstlane(uint32_t(wave));
+        const uint32_t whi = __builtin_amdgcn_readfirstlane(uint32_t(uint64_t(wave) >> 32));
+        wave = int64_t((uint64_t(whi) << 32) | wlo);
+        id.b = wave / G.wpp;
+        const int64_t w = wave % G.wpp;
+        const int64_t wpg = G.p_pad / kWave;
+        id.g = int(w / wpg);
+        id.q = (w % wpg) * kWave + lane;
+        id.active = id.b < batch && id.q < G.P;
+    } else {
+        int64_t lip;
+        if (G.ppw > 1) {
+            id.slot = lane / int(G.lpp);
+            id.b = wave * G.ppw + id.slot;
+            lip = lane % int(G.lpp);
+            id.active = id.slot < G.ppw && id.b < batch;
+        } else {
+            id.b = wave / G.wpp;
+            lip = (wave % G.wpp) * kWave + lane;
+            id.active = id.b < batch && lip < G.lpp;
+        }
+        id.q = lip / G.ng;
+        id.g = int(lip % G.ng);
+    }
+    return id;
+}
+
+// ---------------------------------------------------------------------------
+// Per-lane signature state and the Horner step on it.
+// ---------------------------------------------------------------------------
+template <typename T, int D, int N, int TAIL, int K>
+struct Tree {
+    static_assert(TAIL >= 1 && TAIL < N, "need a non-empty prefix and a non-empty subtree");
+    static_assert(D > 0 || TAIL == 1, "run-time dimension supports depth-1 subtrees only");
+    static constexpr int M = N - TAIL;
+    static constexpr int DD = D > 0 ? D : 1;
+    // subtree depth e (1-based) holds K * D^(e-1) values starting at off(e)
+    __host__ __device__ static constexpr int cnt(int e) { return K * int(ipow64(DD, e - 1)); }
+    __host__ __device__ static constexpr int off(int e)
+    {
+        int o = 0;
+        for (int i = 1; i < e; ++i) o += cnt(i);
+        return o;
+    }
+    static constexpr int SUB = off(TAIL + 1);
+
+    T c[M];       // chain: c[l-1] = S_l[p_1..p_l]
+    T s[SUB];     // subtree slice
+
+    // Letters seen by one step: z[j] for the compile-time letters below subtree
+    // depth 1, zs[a] = z[a0 + a] for the depth-1 slice, pz[l] = z[p_{l+1}].
+    struct Inc {
+        T z[DD];
+        T zs[K];
+        T pz[M];
+    };
+
+    // U_t at chain depth `depth` (1 <= depth <= min(t-1, M)):
+    //   U(1) = z[p_1]/t + S_1[p_1];  U(l+1) = U(l) * z[p_{l+1}] / (t-l) + S_{l+1}[..]
+    // All intermediate values are returned in u[0..depth).
+    template <int t, int depth>
+    __device__ __forceinline__ void chain_u(const Inc& in, T (&u)[M > 0 ? M : 1]) const
+    {
+        u[0] = fmadd(in.pz[0], rcp<T>(t), c[0]);
+#pragma unroll
+        for (int l = 1; l < depth; ++l) u[l] = fmadd(u[l - 1] * rcp<T>(t - l), in.pz[l], c[l]);
+    }
+
+    template <int E>
+    __device__ __forceinline__ static T zc(const Inc& in, int ch)
+    {
+        if constexpr (E == 1) return in.zs[ch];
+        else return in.z[ch];
+    }
+
+    // Descend the subtree for target depth I (target level t = M + I).  `upar`
+    // is U_t of the parent (depth E-1 node `pidx`; the root is the prefix p).
+    template <int E, int I>
+    __device__ __forceinline__ void fwd_desc(const Inc& in, T upar, int pidx)
+    {
+        constexpr int NCH = (E == 1) ? K : DD;
+        if constexpr (E == I) {
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch)
+                s[off(E) + pidx * NCH + ch] = fmadd(upar, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+        } else {
+            const T ur = upar * rcp<T>(I - E + 1);
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) {
+                const T uc = fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+                fwd_desc<E + 1, I>(in, uc, pidx * NCH + ch);
+            }
+        }
+    }
+
+    template <int t>
+    __device__ __forceinline__ void fwd_level(const Inc& in)
+    {
+        if constexpr (t == 1) {
+            c[0] += in.pz[0];
+        } else if constexpr (t <= M) {
+            T u[M > 0 ? M : 1];
+            chain_u<t, t - 1>(in, u);
+            c[t - 1] = fmadd(u[t - 2], in.pz[t - 1], c[t - 1]);
+        } else {
+            T u[M > 0 ? M : 1];
+            chain_u<t, M>(in, u);
+            fwd_desc<1, t - M>(in, u[M - 1], 0);
+        }
+        if constexpr (t > 1) fwd_level<t - 1>(in);
+    }
+
+    // S <- S (x) exp(z): target levels in descending order so that every read of
+    // a lower level still sees the value from before the step
+    // (siglib/cpsig/cp_signature.h:464-499).
+    __device__ __forceinline__ void fwd_step(const Inc& in) { fwd_level<N>(in); }
+};
+
+// Adjoint state of one lane: partial adjoints of the shared chain (seeded in one
+// lane only; the recursion is linear in the adjoint so the partials add up) and
+// the adjoints of the owned subtree slice.
+template <typename T, int D, int N, int TAIL, int K>
+struct TreeAdj {
+    using Tr = Tree<T, D, N, TAIL, K>;
+    static constexpr int M = Tr::M;
+    static constexpr int DD = Tr::DD;
+    T gc[M];
+    T gs[Tr::SUB];
+
+    // Per-step increment gradient pieces of this lane:
+    //   dj[j]  -> letter j            (compile-time letters, subtree depth >= 2)
+    //   da[a]  -> letter a0 + a       (subtree depth 1)
+    //   dc[l]  -> letter p_{l+1}      (chain)
+    struct DInc {
+        T dj[DD];
+        T da[K];
+        T dc[M];
+    };
+
+    // Post-order pullback through the subtree for target depth I.  Returns the
+    // adjoint flowing into the parent's Horner value ("reduced" in
+    // siglib/cpsig/cp_signature.h:1158-1180); children adjoints are the upstream
+    // gradient at depth I and the recursion's return values above it.
+    template <int E, int I>
+    __device__ __forceinline__ T bwd_desc(const Tr& S, const typename Tr::Inc& in, DInc& dz, T upar, int pidx)
+    {
+        constexpr int NCH = (E == 1) ? K : DD;
+        constexpr T sc = rcp<T>(I - E + 1);
+        const T v = (I - E + 1 == 1) ? upar : upar * sc;
+        T red = T(0);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            const int ci = Tr::off(E) + pidx * NCH + ch;
+            T adj;
+            if constexpr (E == I) {
+                adj = gs[ci];
+            } else {
+                const T uc = fmadd(v, Tr::template zc<E>(in, ch), S.s[ci]);
+                adj = bwd_desc<E + 1, I>(S, in, dz, uc, pidx * NCH + ch);
+                gs[ci] += adj;
+            }
+            if constexpr (E == 1) dz.da[ch] = fmadd(adj, v, dz.da[ch]);
+            else dz.dj[ch] = fmadd(adj, v, dz.dj[ch]);
+            red = fmadd(adj, Tr::template zc<E>(in, ch), red);
+        }
+        return (I - E + 1 == 1) ? red : red * sc;
+    }
+
+    // Walk the adjoint `adj` of chain node `from` (1-based depth) up to the root.
+    template <int t, int from>
+    __device__ __forceinline__ void chain_up(const typename Tr::Inc& in, DInc& dz, const T (&u)[M > 0 ? M : 1], T adj)
+    {
+#pragma unroll
+        for (int l = from - 1; l >= 1; --l) {
+            // node p_1..p_l, child letter p_{l+1}
+            const T sc = rcp<T>(t - l);
+            const T v = u[l - 1] * sc;
+            dz.dc[l] = fmadd(adj, v, dz.dc[l]);
+            adj = adj * in.pz[l] * sc;
+            gc[l - 1] += adj;
+        }
+        dz.dc[0] = fmadd(adj, rcp<T>(t), dz.dc[0]);
+    }
+
+    template <int t>
+    __device__ __forceinline__ void bwd_level(const Tr& S, const typename Tr::Inc& in, DInc& dz)
+    {
+        if constexpr (t == 1) {
+            dz.dc[0] += gc[0];
+        } else if constexpr (t <= M) {
+            T u[M > 0 ? M : 1];
+            S.template chain_u<t, t - 1>(in, u);
+            chain_up<t, t>(in, dz, u, gc[t - 1]);
+        } else {
+            T u[M > 0 ? M : 1];
+            S.template chain_u<t, M>(in, u);
+            const T red = bwd_desc<1, t - M>(S, in, dz, u[M - 1], 0);
+            gc[M - 1] += red;
+            chain_up<t, M>(in, dz, u, red);
+        }
+        if constexpr (t < N) bwd_level<t + 1>(S, in, dz);
+    }
+
+    // Pull the adjoint back through one step S_after = S (x) exp(z), where S is
+    // the state BEFORE the step.  Target levels ascend so that the adjoint of
+    // level t is consumed before higher levels add into it
+    // (siglib/cpsig/cp_signature.h:1147-1187).
+    __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
+    {
+        bwd_level<1>(S, in, dz);
+    }
+};
+
+}  // namespace sigamd
