@@ -69,11 +69,14 @@ struct LaneCtx {
     __device__ __forceinline__ void init(int d_rt, int64_t batch)
     {
         d = D > 0 ? D : d_rt;
-        G = make_geom(d, M, K);
+        G = make_geom(d, M, K, D > 0);
         id = lane_id<WIDE>(G, batch);
         // idle lanes shadow a valid lane so that every load stays in bounds;
         // they never store and never contribute
-        if (!id.active) {
+        if constexpr (WIDE) {
+            // path and group stay wave-uniform (waves past the batch exit before loading)
+            if (id.q >= G.P) id.q = G.P - 1;
+        } else if (!id.active) {
             if (id.b >= batch) id.b = batch - 1;
             if (id.q >= G.P) id.q = G.P - 1;
             if (id.g >= G.ng) id.g = G.ng - 1;
@@ -107,6 +110,23 @@ struct LaneCtx {
         return o;
     }
 };
+
+// Nothing may be scheduled across this point: the loads above it are issued
+// before any of the arithmetic below it.
+__device__ __forceinline__ void loads_issued()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// all outstanding vector- and scalar-memory loads have landed
+__device__ __forceinline__ void wait_all_loads()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
 
 template <typename T, int D, int N, int TAIL, int K>
 __device__ __forceinline__ typename Tree<T, D, N, TAIL, K>::Inc negate(const typename Tree<T, D, N, TAIL, K>::Inc& in)
@@ -145,16 +165,25 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
 #pragma unroll
     for (int i = 0; i < Tr::SUB; ++i) S.s[i] = T(0);
 
-    const T* row = inc + cx.id.b * L * d;
-    typename Tr::Inc cur, nxt;
-    cx.load_inc(cur, row);
-    for (int64_t t = 0; t < L; ++t) {
-        const T* nrow = (t + 1 < L) ? row + d : row;
-        cx.load_inc(nxt, nrow);        // prefetch the next increment
-        S.fwd_step(cur);
-        cur = nxt;
-        row = nrow;
+    // Two increment buffers used alternately: the loads of step t+1 are issued
+    // before the arithmetic of step t and waited for after it, so neither the
+    // scalar-cache nor the vector-memory latency sits on the critical path.
+    const T* base = inc + cx.id.b * L * d;
+    typename Tr::Inc za, zb;
+    cx.load_inc(za, base);
+    wait_all_loads();
+    int64_t t = 0;
+    for (; t + 2 <= L; t += 2) {
+        cx.load_inc(zb, base + (t + 1) * d);
+        loads_issued();
+        S.fwd_step(za);
+        wait_all_loads();
+        cx.load_inc(za, base + ((t + 2 < L) ? t + 2 : t + 1) * d);
+        loads_issued();
+        S.fwd_step(zb);
+        wait_all_loads();
     }
+    if (t < L) S.fwd_step(za);
 
     if (!cx.id.active) return;
     T* o = out + cx.id.b * out_stride;
@@ -188,6 +217,12 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
 // back through the step, emit the increment gradient.
 // (siglib/cpsig/cp_signature.h:1137-1187)
 // ---------------------------------------------------------------------------
+// LDS tile of the wide-layout reduction: one row per (step-in-chunk, letter), two
+// half-rows of 32 lanes padded to 33 so that writers and the summing lanes both
+// hit distinct banks.
+constexpr int kRedStride = 66;
+__host__ __device__ constexpr int bwd_chunk(int d) { return (31 / d) < 1 ? 1 : ((31 / d) > 8 ? 8 : (31 / d)); }
+
 template <typename T>
 __device__ __forceinline__ void lds_add(T* p, T v)
 {
@@ -252,31 +287,66 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         }
     });
 
-    // ---- per-wave accumulator for the increment gradient ----------------
+    // ---- reduction of the per-lane increment-gradient pieces ------------
+    // wide layout: every lane writes its D partial sums of a step into a
+    // [row = step-in-chunk * D + letter][lane] tile in LDS (chain pieces are added
+    // into the lane's own column); once the chunk is full each row is summed by
+    // a pair of lanes and added to dz[b][t][letter] in HBM.  packed layout:
+    // per-wave accumulator [path-in-wave][letter] updated with LDS atomics.
     const int lane = threadIdx.x & (kWave - 1);
     const int wave_in_block = threadIdx.x >> 6;
+    constexpr bool WIDE = Cx::WIDE;
+    constexpr int CH = bwd_chunk(Tr::DD);
     const int slots = cx.G.ppw;
-    T* wacc = lds + int64_t(wave_in_block) * slots * d;
-    T* acc = wacc + int64_t(cx.id.slot) * d;
-    if (use_lds) {
-        for (int e = lane; e < slots * d; e += kWave) wacc[e] = T(0);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
+    T* wbuf;
+    if constexpr (WIDE) wbuf = lds + wave_in_block * (CH * Tr::DD * kRedStride);
+    else wbuf = lds + int64_t(wave_in_block) * slots * d;
+    T* acc = wbuf + int64_t(cx.id.slot) * d;
+    const int woff = (lane >> 5) * 33 + (lane & 31);
+    if constexpr (!WIDE) {
+        if (use_lds) {
+            for (int e = lane; e < slots * d; e += kWave) wbuf[e] = T(0);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_wave_barrier();
+        }
     }
     int64_t b_first;
     {
         const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + wave_in_block;
         b_first = (cx.G.ppw > 1) ? wave * cx.G.ppw : (wave / cx.G.wpp);
     }
+    int cs = 0;                 // rows of the current chunk already filled (in steps)
+    int64_t t_chunk = L - 1;    // step held by chunk slot 0
 
-    const T* row = inc + (cx.id.b * L + (L - 1)) * d;
-    typename Tr::Inc cur, nxt;
-    cx.load_inc(cur, row);
-    for (int64_t t = L - 1; t >= 0; --t) {
-        const T* nrow = (t > 0) ? row - d : row;
-        cx.load_inc(nxt, nrow);
+    auto reduce_chunk = [&](int n_slots) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const int n_rows = n_slots * Tr::DD;
+        for (int h = lane; h < 2 * n_rows; h += kWave) {
+            const int rowi = h >> 1, half = h & 1;
+            const T* src = wbuf + rowi * kRedStride + half * 33;
+            T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
+#pragma unroll
+            for (int i = 0; i < 32; i += 4) {
+                s0 += src[i];
+                s1 += src[i + 1];
+                s2 += src[i + 2];
+                s3 += src[i + 3];
+            }
+            T sum = (s0 + s1) + (s2 + s3);
+            sum += __shfl_xor(sum, 1);
+            if (half == 0) {
+                const int slot = rowi / Tr::DD, j = rowi % Tr::DD;
+                dev_add(&dzinc[(cx.id.b * L + (t_chunk - slot)) * d + j], sum);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+    };
 
-        S.fwd_step(negate<T, D, N, TAIL, K>(cur));     // state before the step
+    auto do_step = [&](const typename Tr::Inc& z, int64_t t) {
+        S.fwd_step(negate<T, D, N, TAIL, K>(z));     // state before the step
         typename Ad::DInc dz;
 #pragma unroll
         for (int j = 0; j < Tr::DD; ++j) dz.dj[j] = T(0);
@@ -284,46 +354,83 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         for (int a = 0; a < K; ++a) dz.da[a] = T(0);
 #pragma unroll
         for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
-        A.pullback(S, cur, dz);
+        A.pullback(S, z, dz);
 
-        T* grow_t = dzinc + (cx.id.b * L + t) * d;
-        if (use_lds) {
+        if constexpr (WIDE) {
+            T* tile = wbuf + cs * (Tr::DD * kRedStride) + woff;
+#pragma unroll
+            for (int j = 0; j < Tr::DD; ++j) tile[j * kRedStride] = (active && TAIL >= 2) ? dz.dj[j] : T(0);
             if (active) {
+                // depth-1 letters (wave-uniform rows) and chain letters (per-lane rows) are
+                // added into the lane's own column; LDS executes a wave's operations in order
+#pragma unroll
+                for (int a = 0; a < K; ++a)
+                    if (cx.a0 + a < Tr::DD) lds_add(&tile[(cx.a0 + a) * kRedStride], dz.da[a]);
+#pragma unroll
+                for (int l = 0; l < M; ++l) lds_add(&tile[cx.p[l] * kRedStride], dz.dc[l]);
+            }
+            ++cs;
+            if (cs == CH || t == 0) {
+                reduce_chunk(cs);
+                cs = 0;
+                t_chunk = t - 1;
+            }
+        } else {
+            T* grow_t = dzinc + (cx.id.b * L + t) * d;
+            if (use_lds) {
+                if (active) {
+#pragma unroll
+                    for (int a = 0; a < K; ++a)
+                        if (cx.a0 + a < d) lds_add(&acc[cx.a0 + a], dz.da[a]);
+                    if constexpr (TAIL >= 2) {
+#pragma unroll
+                        for (int j = 0; j < Tr::DD; ++j) lds_add(&acc[j], dz.dj[j]);
+                    }
+#pragma unroll
+                    for (int l = 0; l < M; ++l) lds_add(&acc[cx.p[l]], dz.dc[l]);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                for (int e = lane; e < slots * d; e += kWave) {
+                    const T v = wbuf[e];
+                    wbuf[e] = T(0);
+                    const int64_t bb = b_first + e / d;
+                    if (bb < batch) dev_add(&dzinc[(bb * L + t) * d + e % d], v);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_wave_barrier();
+            } else if (active) {
                 if constexpr (TAIL >= 2) {
 #pragma unroll
-                    for (int j = 0; j < Tr::DD; ++j) lds_add(&acc[j], dz.dj[j]);
+                    for (int j = 0; j < Tr::DD; ++j) dev_add(&grow_t[j], dz.dj[j]);
                 }
 #pragma unroll
                 for (int a = 0; a < K; ++a)
-                    if (cx.a0 + a < d) lds_add(&acc[cx.a0 + a], dz.da[a]);
+                    if (cx.a0 + a < d) dev_add(&grow_t[cx.a0 + a], dz.da[a]);
 #pragma unroll
-                for (int l = 0; l < M; ++l) lds_add(&acc[cx.p[l]], dz.dc[l]);
+                for (int l = 0; l < M; ++l) dev_add(&grow_t[cx.p[l]], dz.dc[l]);
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            for (int e = lane; e < slots * d; e += kWave) {
-                const T v = wacc[e];
-                wacc[e] = T(0);
-                const int64_t bb = b_first + e / d;
-                if (bb < batch) dev_add(&dzinc[(bb * L + t) * d + e % d], v);
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_wave_barrier();
-        } else if (active) {
-            if constexpr (TAIL >= 2) {
-#pragma unroll
-                for (int j = 0; j < Tr::DD; ++j) dev_add(&grow_t[j], dz.dj[j]);
-            }
-#pragma unroll
-            for (int a = 0; a < K; ++a)
-                if (cx.a0 + a < d) dev_add(&grow_t[cx.a0 + a], dz.da[a]);
-#pragma unroll
-            for (int l = 0; l < M; ++l) dev_add(&grow_t[cx.p[l]], dz.dc[l]);
         }
-        cur = nxt;
-        row = nrow;
+    };
+
+    // reverse sweep with two alternating increment buffers (see the forward kernel)
+    const T* base = inc + cx.id.b * L * d;
+    typename Tr::Inc za, zb;
+    cx.load_inc(za, base + (L - 1) * d);
+    wait_all_loads();
+    int64_t t = L - 1;
+    for (; t >= 1; t -= 2) {
+        cx.load_inc(zb, base + (t - 1) * d);
+        loads_issued();
+        do_step(za, t);
+        wait_all_loads();
+        cx.load_inc(za, base + ((t >= 2) ? t - 2 : 0) * d);
+        loads_issued();
+        do_step(zb, t - 1);
+        wait_all_loads();
     }
+    if (t == 0) do_step(za, 0);
 }
 
 // ---------------------------------------------------------------------------

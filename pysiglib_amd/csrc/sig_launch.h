@@ -11,7 +11,7 @@ constexpr size_t kMaxDynLds = 64 * 1024;
 template <typename T, int D, int N, int TAIL, int K>
 hipError_t launch_tree_fwd(const FwdParams& p)
 {
-    const TreeGeom g = make_geom(p.d, N - TAIL, K);
+    const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
@@ -24,13 +24,20 @@ hipError_t launch_tree_fwd(const FwdParams& p)
 template <typename T, int D, int N, int TAIL, int K>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
-    const TreeGeom g = make_geom(p.d, N - TAIL, K);
+    const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
-    size_t lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
+    size_t lds;
     int use_lds = 1;
-    if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
+    if (g.wide) {
+        static_assert(D <= 31, "wide-layout reduction tile assumes at most 31 letters");
+        lds = size_t(kWavesPerBlock) * size_t(bwd_chunk(D > 0 ? D : 1)) * size_t(D) * kRedStride * sizeof(T);
+    } else {
+        lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
+        if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
+    }
+    if (lds > kMaxDynLds) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
                        static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,

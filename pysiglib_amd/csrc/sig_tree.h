@@ -57,12 +57,12 @@ struct TreeGeom {
     int64_t wpp;        // waves per path when a path spans waves, else 1
 };
 
-__host__ __device__ inline TreeGeom make_geom(int d, int m, int k)
+__host__ __device__ inline TreeGeom make_geom(int d, int m, int k, bool allow_wide)
 {
     TreeGeom g;
     g.P = ipow64(d, m);
     g.ng = (d + k - 1) / k;
-    g.wide = g.P >= 48;
+    g.wide = allow_wide && g.P >= 48;   // must agree with the kernel's compile-time choice
     if (g.wide) {
         g.p_pad = (g.P + kWave - 1) / kWave * kWave;
         g.lpp = g.ng * g.p_pad;

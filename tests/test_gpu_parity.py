@@ -1,0 +1,323 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle and the golden vectors.
+
+Tolerances: float64 1e-10, float32 1e-4, relative to the per-level (forward) or per-path (backward) max norm,
+as stated for this path; the golden-vector tests use the reference's absolute tolerances
+(tests/conftest.py:34-50 of the reference: 1e-10 / 1e-4; backward fixtures are float32, 1e-5).
+"""
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+from tests import _configs as C
+from tests._mathref import level_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float64: 1e-10, np.float32: 1e-4}
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def P():
+    import pysiglib_amd
+    assert torch.cuda.is_available()
+    return pysiglib_amd
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import sigref
+    return sigref
+
+
+def dev(a):
+    return torch.tensor(np.ascontiguousarray(a), device=DEV)
+
+
+def bwd_rel_err(got, ref):
+    got = got.reshape(ref.shape[0], -1).astype(np.float64)
+    ref2 = ref.reshape(ref.shape[0], -1).astype(np.float64)
+    den = np.maximum(np.abs(ref2).max(axis=1), np.finfo(np.float64).tiny)
+    return float((np.abs(got - ref2).max(axis=1) / den).max())
+
+
+AUGS = {
+    "sig": ({}, "path"),
+    "sig_ta": (dict(time_aug=True), "path"),
+    "sig_ll": (dict(lead_lag=True), "path_dim2"),
+    "sig_ta_ll": (dict(time_aug=True, lead_lag=True), "path_dim2"),
+}
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("key", list(AUGS))
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_forward_golden(P, fixtures, deg, key, dtype):
+    kw, pkey = AUGS[key]
+    expected = fixtures[f"{key}__d{deg}"]
+    x = fixtures[pkey].astype(dtype)
+    got = P.sig(dev(x), deg, **kw)
+    assert got.device.type == "cuda"
+    np.testing.assert_allclose(got.cpu().numpy(), expected, rtol=0, atol=TOL[dtype])
+    single = P.sig(dev(x[0]), deg, horner=False, **kw)          # single path, other value of the horner flag
+    np.testing.assert_allclose(single.cpu().numpy(), expected[0], rtol=0, atol=TOL[dtype])
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_backward_golden(P, fixtures, deg, dtype):
+    x = dev(fixtures["path"].astype(dtype))
+    g = dev(fixtures[f"sig_bp_derivs__d{deg}"].astype(dtype))     # one column wider: carries the scalar slot
+    expected = fixtures[f"sig_bp_expected__d{deg}"]
+    s = P.sig(x, deg)
+    got = P.sig_backprop(x.clone(), s.clone(), g.clone(), deg)
+    np.testing.assert_allclose(got.cpu().numpy(), expected, rtol=0, atol=1e-5 if dtype == np.float64 else 1e-4)
+
+
+def test_kats(P, kats):
+    for k in kats["forward"]:
+        if k["length"] == 0:
+            continue    # zero-length tensors cannot carry the shape through torch
+        dt = np.dtype(k["dtype"]).type
+        x = np.array(k["path"], dtype=dt).reshape(k["batch"], k["length"], k["dimension"])
+        got = P.sig(dev(x), k["degree"], time_aug=k["time_aug"], lead_lag=k["lead_lag"], end_time=k["end_time"],
+                    scalar_term=True).cpu().numpy()
+        tol = 1e-12 if dt == np.float64 else 2e-5
+        np.testing.assert_allclose(got.ravel(), np.array(k["expected"]), rtol=tol, atol=tol, err_msg=k["name"])
+    for k in kats["backward"]:
+        x = np.array(k["path"]).reshape(k["batch"], k["length"], k["dimension"])
+        s = np.array(k["sig"]).reshape(k["batch"], -1)
+        g = np.array(k["derivs"]).reshape(k["batch"], -1)
+        got = P.sig_backprop(dev(x), dev(s), dev(g), k["degree"], time_aug=k["time_aug"], lead_lag=k["lead_lag"],
+                             end_time=k["end_time"]).cpu().numpy()
+        np.testing.assert_allclose(got.ravel(), np.array(k["expected"]), rtol=1e-12, atol=1e-12, err_msg=k["name"])
+
+
+# (batch, length, dim, degree): specialised kernels, run-time-dimension kernel, batch tails, wide/packed geometries
+GRID = [
+    (1, 2, 2, 2), (3, 6, 2, 6), (7, 9, 3, 4), (9, 5, 4, 4), (17, 12, 3, 3), (70, 6, 2, 3), (2, 33, 5, 4),
+    (3, 10, 6, 3), (2, 10, 7, 4), (2, 6, 20, 2), (1, 8, 37, 3), (4, 5, 2, 13), (2, 12, 3, 9), (130, 4, 3, 2),
+    (2, 40, 10, 5), (2, 40, 5, 7), (1, 25, 3, 12), (2, 15, 17, 4), (3, 7, 16, 3), (2, 9, 9, 4), (5, 6, 2, 16),
+]
+
+
+@pytest.mark.parametrize("shape", GRID)
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_grid_vs_oracle(P, oracle, shape, dtype, scalar_term):
+    b, length, d, deg = shape
+    rng = np.random.default_rng(hash(shape) % (2 ** 31))
+    x = (rng.standard_normal((b, length, d)) * (0.5 if deg > 6 else 1.0)).astype(dtype)
+    ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1)
+    got = P.sig(dev(x), deg, scalar_term=scalar_term).cpu().numpy()
+    off = 1 if scalar_term else 0
+    if scalar_term:
+        np.testing.assert_array_equal(got[:, 0], 1.0)
+    assert level_rel_err(got[:, off:], ref[:, off:], d, deg) <= TOL[dtype]
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    ref_b = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
+    xt, st, gt = dev(x), dev(ref), dev(g)
+    keep = (xt.clone(), st.clone(), gt.clone())
+    got_b = P.sig_backprop(xt, st, gt, deg).cpu().numpy()
+    assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
+    for a, bb in zip((xt, st, gt), keep):       # inputs are left bit-identical
+        assert torch.equal(a, bb)
+
+
+@pytest.mark.parametrize("aug", [dict(time_aug=True, end_time=2.5), dict(lead_lag=True),
+                                 dict(time_aug=True, lead_lag=True, end_time=0.5)])
+@pytest.mark.parametrize("shape", [(3, 9, 2, 4), (2, 12, 3, 3), (5, 7, 1, 5), (2, 20, 8, 4), (2, 6, 4, 2), (3, 5, 3, 1)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_augmentations_vs_oracle(P, oracle, aug, shape, dtype):
+    b, length, d, deg = shape
+    rng = np.random.default_rng(17 + d + deg)
+    x = (rng.standard_normal((b, length, d)) * 0.7).astype(dtype)
+    d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    ref = oracle.signature(x, deg, n_jobs=-1, **aug)
+    got = P.sig(dev(x), deg, **aug).cpu().numpy()
+    assert level_rel_err(got, ref, d_aug, deg) <= TOL[dtype]
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    ref_b = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+    got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+    assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
+
+
+def test_closed_forms(P):
+    # straight line: level k = v^(x)k / k!   (tests/test_cuda_horner.py:100-112 of the reference)
+    rng = np.random.default_rng(5)
+    for d, deg in ((2, 12), (3, 8), (5, 5), (10, 4)):
+        v = rng.standard_normal(d) * 0.8
+        ts = np.linspace(0, 1, 9) ** 2
+        got = P.sig(dev(ts[:, None] * v[None, :]), deg).cpu().numpy()
+        lvl, off = np.array(1.0), 0
+        for k in range(1, deg + 1):
+            lvl = np.multiply.outer(lvl, v) / k
+            np.testing.assert_allclose(got[off:off + d ** k], lvl.ravel(), rtol=1e-11, atol=1e-14)
+            off += d ** k
+    # d = 1: Delta^k / k!
+    import math
+    x = np.array([[0.3], [1.0], [-2.0], [0.7]])
+    np.testing.assert_allclose(P.sig(dev(x), 6, scalar_term=True).cpu().numpy(),
+                               [0.4 ** k / math.factorial(k) for k in range(7)], rtol=1e-13)
+    # degree 1 / d = 1: only the endpoints receive gradient, interior exactly zero
+    y = dev(rng.standard_normal((2, 7, 4)))
+    g = dev(rng.standard_normal((2, 4)))
+    grad = P.sig_backprop(y, P.sig(y, 1), g, 1)
+    assert torch.equal(grad[:, 1:-1], torch.zeros_like(grad[:, 1:-1]))
+    torch.testing.assert_close(grad[:, -1], g)
+    torch.testing.assert_close(grad[:, 0], -g)
+
+
+def test_trivial_cases(P):
+    x = torch.zeros(2, 1, 3, dtype=torch.float64, device=DEV)
+    assert torch.equal(P.sig(x, 2, scalar_term=True).cpu(), torch.tensor([[1.] + [0.] * 12] * 2, dtype=torch.float64))
+    assert torch.equal(P.sig(x, 2).cpu(), torch.zeros(2, 12, dtype=torch.float64))
+    y = torch.randn(2, 4, 3, dtype=torch.float64, device=DEV)
+    assert torch.equal(P.sig(y, 0, scalar_term=True).cpu(), torch.ones(2, 1, dtype=torch.float64))
+    assert P.sig(y, 0).shape == (2, 0)
+    assert torch.equal(P.sig(y, 3, scalar_term=True)[:, 1:], P.sig(y, 3))
+    assert torch.equal(P.sig_backprop(x, torch.zeros(2, 12, dtype=torch.float64, device=DEV),
+                                      torch.ones(2, 12, dtype=torch.float64, device=DEV), 2).cpu(),
+                       torch.zeros(2, 1, 3, dtype=torch.float64))
+    assert P.sig(torch.zeros(0, 5, 3, dtype=torch.float64, device=DEV), 3).shape == (0, 39)
+    two = torch.tensor([[0., 0.], [1., 1.]], device=DEV)
+    torch.testing.assert_close(P.sig(two, 1).cpu(), torch.tensor([1., 1.]))
+
+
+def test_batch_dims_views_and_warnings(P, oracle):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 3, 8, 4))
+    ref = oracle.signature(x.reshape(6, 8, 4), 3).reshape(2, 3, -1)
+    got = P.sig(dev(x), 3)
+    assert got.shape == (2, 3, 84)
+    np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=1e-11, atol=1e-12)
+    g = rng.standard_normal(ref.shape)
+    ref_b = oracle.sig_backprop(x.reshape(6, 8, 4), ref.reshape(6, -1), g.reshape(6, -1), 3).reshape(x.shape)
+    np.testing.assert_allclose(P.sig_backprop(dev(x), dev(ref), dev(g), 3).cpu().numpy(), ref_b, rtol=1e-10, atol=1e-11)
+    # non-contiguous / expanded inputs are cloned (tests/test_signature.py:58-79 of the reference)
+    base = torch.rand(5, 20, dtype=torch.float64, device=DEV)[:, :, None]
+    view = base.expand(-1, -1, 6)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        torch.testing.assert_close(P.sig(view, 3), P.sig(view.clone(), 3))
+        strided = torch.randn(4, 30, 6, dtype=torch.float64, device=DEV)[..., ::2]
+        torch.testing.assert_close(P.sig(strided, 4), P.sig(strided.contiguous(), 4))
+    # overflow in the result warns (pysiglib/sig.py:299-310)
+    with pytest.warns(RuntimeWarning):
+        P.sig(torch.full((1, 3, 2), 1e200, dtype=torch.float64, device=DEV).cumsum(1), 3)
+
+
+def test_error_codes_through_the_abi(P):
+    import ctypes
+    from pysiglib_amd import _loader as L
+    f = L.CUSIG_SIGNATURE["float64"]
+    x = torch.zeros(8, dtype=torch.float64, device=DEV)
+    p = ctypes.cast(x.data_ptr(), ctypes.POINTER(ctypes.c_double))
+    assert f(p, p, 1, 0, 2, 2, False, False, 1.0, True, True, None, 0, 0, 0) == 2          # dimension 0
+    assert "dimension 0" in L.last_error_message()
+    assert f(p, p, 1, 2, 2, 2, False, False, 1.0, True, True, None, 4, 0, 0) == 2          # null correction, len != 0
+    assert f(p, p, 1, 2, 2, 2, False, True, 1.0, True, True, p, 4, 0, 0) == 2              # correction with lead-lag
+    assert f(p, p, 1, 2, 2, 2, False, False, 1.0, True, True, p, 4, 0, 0) == 10            # valid correction: unsupported
+    assert f(p, p, 0, 2, 2, 2, False, False, 1.0, True, True, None, 0, 0, 0) == 0          # empty batch
+    assert f(p, p, 1, 100, 2, 100, False, False, 1.0, True, True, None, 0, 0, 0) == 10     # size overflow
+    assert f(p, p, 1, 2, 2, 40, False, False, 1.0, True, True, None, 0, 0, 0) == 10        # no kernel for this degree
+    assert "no kernel" in L.last_error_message()
+    with pytest.raises(Exception, match="Error in pysiglib.sig"):
+        P.sig(torch.zeros(1, 3, 2, dtype=torch.float64, device=DEV), 17)
+    y = torch.zeros(3, 4, 2, dtype=torch.float64, device=DEV)
+    with pytest.raises(ValueError):                                   # width matches neither convention
+        P.sig_backprop(y, torch.zeros(3, 5, dtype=torch.float64, device=DEV),
+                       torch.zeros(3, 5, dtype=torch.float64, device=DEV), 2)
+    with pytest.raises(ValueError):                                   # dtype mismatch
+        P.sig_backprop(y, torch.zeros(3, 6, dtype=torch.float32, device=DEV),
+                       torch.zeros(3, 6, dtype=torch.float32, device=DEV), 2)
+    with pytest.raises(ValueError):                                   # batch mismatch
+        P.sig_backprop(y, torch.zeros(2, 6, dtype=torch.float64, device=DEV),
+                       torch.zeros(2, 6, dtype=torch.float64, device=DEV), 2)
+
+
+def test_autograd_wrapper(P, oracle):
+    rng = np.random.default_rng(8)
+    for aug in ({}, dict(time_aug=True, lead_lag=True, end_time=2.0)):
+        x = rng.standard_normal((3, 9, 3))
+        ref = oracle.signature(x, 4, **aug)
+        g = rng.standard_normal(ref.shape)
+        ref_b = oracle.sig_backprop(x, ref, g, 4, **aug)
+        xt = dev(x).requires_grad_()
+        out = P.torch_api.sig(xt, 4, **aug)
+        (grad,) = torch.autograd.grad(out, xt, dev(g))
+        np.testing.assert_allclose(out.detach().cpu().numpy(), ref, rtol=1e-11, atol=1e-12)
+        np.testing.assert_allclose(grad.cpu().numpy(), ref_b, rtol=1e-10, atol=1e-11)
+    # finite-difference directional derivative (tests/test_cuda_horner.py:131-146 of the reference)
+    x = dev(rng.standard_normal((2, 6, 3))).requires_grad_()
+    seeds = dev(rng.standard_normal((2, 120)))
+    direction = dev(rng.standard_normal((2, 6, 3)))
+    (grad,) = torch.autograd.grad(P.torch_api.sig(x, 4), x, seeds)
+    eps = 1e-5
+    fd = ((P.sig(x.detach() + eps * direction, 4) - P.sig(x.detach() - eps * direction, 4)) * seeds).sum() / (2 * eps)
+    torch.testing.assert_close((grad * direction).sum(), fd, atol=2e-7, rtol=2e-7)
+
+
+def test_reused_buffers_and_repeatability(P, oracle):
+    # the library keeps internal workspaces between calls: interleave shapes and repeat
+    rng = np.random.default_rng(21)
+    cases = [(4, 65, 2, 4), (2, 30, 10, 5), (16, 9, 3, 4), (4, 65, 2, 4)]
+    for (b, length, d, deg) in cases * 2:
+        x = rng.standard_normal((b, length, d)) * 0.4
+        ref = oracle.signature(x, deg, n_jobs=-1)
+        g = rng.standard_normal(ref.shape)
+        assert level_rel_err(P.sig(dev(x), deg).cpu().numpy(), ref, d, deg) <= 1e-10
+        assert bwd_rel_err(P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy(),
+                           oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)) <= 1e-10
+
+
+# ---- the benchmark workloads at full size -----------------------------------------------------------------
+
+@pytest.mark.parametrize("k", [1, 2, 4])
+def test_config_forward_full_size(P, oracle, k):
+    c = C.CONFIGS[k]
+    x = C.make_path(k)
+    kw = dict(time_aug=c["time_aug"], lead_lag=c["lead_lag"], end_time=1.0)
+    ref = oracle.signature(x, c["degree"], n_jobs=-1, **kw)
+    got = P.sig(dev(x), c["degree"], **kw).cpu().numpy()
+    assert got.shape == ref.shape
+    assert level_rel_err(got, ref, C.aug_dim(c), c["degree"]) <= TOL[np.dtype(c["dtype"]).type]
+
+
+def test_config3_forward(P, oracle):
+    """(64, 4096, 3) degree 12: the oracle checks the first 6 paths; all 64 are checked through
+    size-independent properties (level 1 = total increment, level-2 shuffle identity, batch invariance)."""
+    c = C.CONFIGS[3]
+    x = C.make_path(3)
+    xt = dev(x)
+    got = P.sig(xt, 12)
+    assert got.shape == (64, 797160)
+    ref = oracle.signature(x[:6], 12, n_jobs=-1)
+    assert level_rel_err(got[:6].cpu().numpy(), ref, 3, 12) <= 1e-10
+    l1 = got[:, :3].cpu().numpy()
+    np.testing.assert_allclose(l1, x[:, -1] - x[:, 0], rtol=1e-12, atol=1e-14)
+    l2 = got[:, 3:12].cpu().numpy().reshape(64, 3, 3)
+    np.testing.assert_allclose(l2 + l2.transpose(0, 2, 1), l1[:, :, None] * l1[:, None, :], rtol=1e-10, atol=1e-13)
+    again = P.sig(xt[40:47].clone(), 12)
+    assert torch.equal(again, got[40:47])
+    del got, again
+    torch.cuda.empty_cache()
+
+
+def test_config5_backward_full_size(P, oracle):
+    c = C.CONFIGS[5]
+    x = C.make_path(5)
+    sig = oracle.signature(x, 5, n_jobs=-1)
+    g = np.random.default_rng(2005).standard_normal(sig.shape)
+    ref = oracle.sig_backprop(x, sig, g, 5, n_jobs=-1)
+    got = P.sig_backprop(dev(x), dev(sig), dev(g), 5).cpu().numpy()
+    assert bwd_rel_err(got, ref) <= 1e-10
+    # linearity in the upstream gradient holds at any size
+    got2 = P.sig_backprop(dev(x), dev(sig), dev(2.0 * g), 5).cpu().numpy()
+    assert bwd_rel_err(got2, 2.0 * got) <= 1e-12
+    # the GPU forward feeds the GPU backward (the autograd pairing)
+    sig_gpu = P.sig(dev(x), 5)
+    got3 = P.sig_backprop(dev(x), sig_gpu, dev(g), 5).cpu().numpy()
+    assert bwd_rel_err(got3, ref) <= 1e-10
