@@ -17,6 +17,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <vector>
 
 #include "../../include/cusig_amd.h"
 #include "sig_kernels.h"
@@ -116,7 +117,8 @@ static uint64_t checked_mul(uint64_t a, uint64_t b, const char* what)
 // kernel table
 // ---------------------------------------------------------------------------
 struct Table {
-    std::map<std::tuple<int, int, int>, const KernelEntry*> fwd, bwd;
+    // several partitions (tail, k) of one shape may be compiled; the first listed is the default
+    std::map<std::tuple<int, int, int>, std::vector<const KernelEntry*>> fwd, bwd;
     Table()
     {
         int n = 0;
@@ -125,11 +127,15 @@ struct Table {
             for (int j = 0; j < lists[i].count; ++j) {
                 const KernelEntry* e = &lists[i].entries[j];
                 auto key = std::make_tuple(e->is_f64, e->D, e->N);
-                if (e->fwd) fwd[key] = e;
-                if (e->bwd) bwd[key] = e;
+                auto& slot = e->fwd ? fwd[key] : bwd[key];
+                if (e->preferred) slot.insert(slot.begin(), e);
+                else slot.push_back(e);
             }
     }
 };
+
+// tuning hook: when set (tail > 0), prefer the compiled partition with this (tail, k)
+static int g_force_tail = 0, g_force_k = 0;
 
 static const Table& table()
 {
@@ -142,9 +148,13 @@ static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64
     const auto& m = backward ? table().bwd : table().fwd;
     if (d <= 0x7fffffff && degree <= 0x7fffffff) {
         auto it = m.find(std::make_tuple(int(f64), int(d), int(degree)));
-        if (it != m.end()) return it->second;
-        it = m.find(std::make_tuple(int(f64), 0, int(degree)));
-        if (it != m.end()) return it->second;
+        if (it == m.end()) it = m.find(std::make_tuple(int(f64), 0, int(degree)));
+        if (it != m.end() && !it->second.empty()) {
+            if (g_force_tail > 0)
+                for (const KernelEntry* e : it->second)
+                    if (e->tail == g_force_tail && e->k == g_force_k) return e;
+            return it->second.front();
+        }
     }
     return nullptr;
 }
@@ -472,6 +482,12 @@ CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) noexcept { g_profile = e
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; }
 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
+
+CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
+{
+    g_force_tail = tail;
+    g_force_k = k;
+}
 
 CUSIG_AMD_API int cusig_amd_kernel_choice(int backward, int is_f64, uint64_t dimension, uint64_t degree,
                                           int* tail, int* k, int* specialised) noexcept

@@ -36,6 +36,7 @@ struct KernelEntry {
     FwdFn fwd;
     BwdFn bwd;
     const char* name;
+    int preferred;   // default partition of its shape
 };
 
 // every generated instance file contributes one array
