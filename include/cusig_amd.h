@@ -89,6 +89,8 @@ CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree)
 CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
+/* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
+CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: prefer the compiled lane partition (tail, k) where a shape has several; tail = 0 restores
  * the defaults.  Not thread-safe; meant for offline sweeps. */
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) CUSIG_AMD_NOEXCEPT;

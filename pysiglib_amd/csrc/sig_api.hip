@@ -8,6 +8,7 @@
 // (siglib/shared/last_error.h:22-41).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <charconv>
 #include <cstdio>
 #include <cstring>
@@ -240,6 +241,37 @@ struct MainKernelTimer {
 };
 
 // ---------------------------------------------------------------------------
+// time segmentation of the forward sweep
+// ---------------------------------------------------------------------------
+static int g_force_segments = 0;   // tuning hook (0 = automatic)
+
+static int simd_count()
+{
+    static int cached = 0;
+    if (!cached) {
+        int dev = 0, cus = 0;
+        SIG_HIP(hipGetDevice(&dev));
+        SIG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        cached = 4 * (cus > 0 ? cus : 256);
+    }
+    return cached;
+}
+
+// Splitting costs one extra signature write per segment plus the Chen folds, so it only pays when whole-path
+// sweeps leave more than half of the SIMDs without a wave.  Then aim at two waves per SIMD (never more than the
+// kernel's registers allow), with segments of at least 48 increments and at most 256 MB of segment signatures.
+static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_t sig_bytes_all_paths)
+{
+    const int64_t simds = simd_count();
+    if (waves <= 0 || waves * 2 > simds) return 1;
+    int64_t g = int64_t(std::min(waves_per_simd, 2)) * simds / waves;
+    g = std::min<int64_t>(g, 8);
+    g = std::min<int64_t>(g, L / 48);
+    if (sig_bytes_all_paths > 0) g = std::min<int64_t>(g, int64_t((uint64_t(256) << 20) / sig_bytes_all_paths));
+    return int(std::max<int64_t>(g, 1));
+}
+
+// ---------------------------------------------------------------------------
 // shared argument handling
 // ---------------------------------------------------------------------------
 static void validate_correction(const void* correction, uint64_t correction_len, uint64_t dimension,
@@ -294,7 +326,7 @@ static void compute_increments(const T* path, T* inc, uint64_t batch, uint64_t d
                                bool time_aug, bool lead_lag, T end_time, const Shape& s, hipStream_t stream)
 {
     const T time_step = s.len_aug > 1 ? end_time / T(s.len_aug - 1) : T(0);
-    hipLaunchKernelGGL((increments_kernel<T>), dim3(grid_for(batch * s.L * s.d_aug)), dim3(kBlock), 0, stream,
+    hipLaunchKernelGGL((increments_kernel<T>), dim3(grid_for(batch * (s.L + 2) * s.d_aug)), dim3(kBlock), 0, stream,
                        path, inc, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                        int(lead_lag), time_step);
     SIG_HIP(hipGetLastError());
@@ -342,15 +374,54 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             throw std::runtime_error("signature_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
         std::lock_guard<std::mutex> lk(g_ws_mutex);
-        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+        // Few paths cannot fill the chip with whole-path sweeps: split every path into time segments,
+        // sweep all (path, segment) pairs concurrently and fold the pieces with Chen's identity.
+        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0);
+        int nseg = g_force_segments > 0
+                             ? int(std::min<uint64_t>(uint64_t(g_force_segments), s.L))
+                             : choose_segments(total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
+                                               batch * (s.full_len - 1) * sizeof(T));
+        const uint64_t n_coef = s.full_len - 1;
         FwdParams p;
-        p.inc = inc; p.out = out; p.batch = int64_t(batch); p.L = int64_t(s.L); p.d = int(s.d_aug);
-        p.out_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
+        p.inc = inc; p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
+        p.lseg = (int64_t(s.L) + nseg - 1) / nseg;
+        nseg = int((int64_t(s.L) + p.lseg - 1) / p.lseg);      // drop segments the rounding left empty
+        p.nseg = nseg;
+        p.batch = int64_t(batch) * nseg;
+        T* segs = nullptr;
+        T* tmp[2] = {nullptr, nullptr};
+        if (nseg == 1) {
+            p.out = out; p.out_stride = int64_t(s.stride); p.scalar = sc;
+        } else {
+            const uint64_t row_elems = checked_mul(batch, n_coef, "segment signatures");
+            segs = static_cast<T*>(workspace(2, checked_mul(checked_mul(row_elems, uint64_t(nseg), "segment signatures"), sizeof(T), "segment signatures")));
+            if (nseg > 2) {
+                T* t2 = static_cast<T*>(workspace(3, checked_mul(checked_mul(row_elems, 2, "segment signatures"), sizeof(T), "segment signatures")));
+                tmp[0] = t2; tmp[1] = t2 + row_elems;
+            }
+            p.out = segs; p.out_stride = int64_t(n_coef); p.scalar = 0;
+        }
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->fwd(p));
         timer.stop();
+        if (nseg > 1) {
+            const T* acc = segs;
+            int64_t acc_stride = int64_t(n_coef) * nseg;
+            for (int g = 1; g < nseg; ++g) {
+                const bool last = g == nseg - 1;
+                T* dst = last ? out : tmp[(g - 1) & 1];
+                hipLaunchKernelGGL((sig_combine_kernel<T>), dim3(grid_for(batch * n_coef)), dim3(kBlock), 0, stream,
+                                   acc, segs + uint64_t(g) * n_coef, dst, int64_t(batch), int(s.d_aug), int(degree),
+                                   int64_t(n_coef), acc_stride, int64_t(n_coef) * nseg,
+                                   last ? int64_t(s.stride) : int64_t(n_coef), 0, 0, last ? sc : 0);
+                SIG_HIP(hipGetLastError());
+                acc = dst;
+                acc_stride = int64_t(n_coef);
+            }
+        }
         SIG_HIP(hipStreamSynchronize(stream));
         return;
     }
@@ -392,13 +463,13 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             throw std::runtime_error("sig_backprop_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
         std::lock_guard<std::mutex> lk(g_ws_mutex);
-        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
-        const size_t inc_bytes = checked_mul(inc_elems, sizeof(T), "increments");
-        T* inc = static_cast<T*>(workspace(0, inc_bytes));
-        T* dzinc = static_cast<T*>(workspace(1, inc_bytes));
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+        const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
-        hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(inc_elems)), dim3(kBlock), 0, stream, dzinc,
-                           int64_t(inc_elems));
+        hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(dz_elems)), dim3(kBlock), 0, stream, dzinc,
+                           int64_t(dz_elems));
         SIG_HIP(hipGetLastError());
         BwdParams p;
         p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
@@ -482,6 +553,8 @@ CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) noexcept { g_profile = e
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; }
 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
+
+CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {

@@ -29,24 +29,32 @@ __global__ __launch_bounds__(kBlock) void increments_kernel(
     const T* __restrict__ path, T* __restrict__ inc, int64_t batch, int64_t len_raw, int d_raw,
     int time_aug, int lead_lag, T time_step)
 {
+    // Layout [batch][L + 2][d]: row t + 1 holds the increment of step t; rows 0 and L + 1 are zero so
+    // that the sweeps may prefetch one row past either end of a path without a bounds test.
     const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
     const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
-    const int64_t total = batch * L * d;
+    const int64_t rows = L + 2;
+    const int64_t total = batch * rows * d;
     for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
         const int c = int(e % d);
-        const int64_t t = (e / d) % L;
-        const int64_t b = e / (int64_t(d) * L);
+        const int64_t row = (e / d) % rows;
+        const int64_t b = e / (int64_t(d) * rows);
         const T* x = path + b * len_raw * d_raw;
         T v;
-        if (time_aug && c == d - 1) {
-            v = T(t + 1) * time_step - T(t) * time_step;
-        } else if (!lead_lag) {
-            v = x[(t + 1) * d_raw + c] - x[t * d_raw + c];
+        if (row == 0 || row == rows - 1) {
+            v = T(0);
         } else {
-            const int64_t k = t >> 1;
-            const bool odd = t & 1;
-            if (c < d_raw) v = odd ? x[(k + 1) * d_raw + c] - x[k * d_raw + c] : T(0);
-            else v = odd ? T(0) : x[(k + 1) * d_raw + (c - d_raw)] - x[k * d_raw + (c - d_raw)];
+            const int64_t t = row - 1;
+            if (time_aug && c == d - 1) {
+                v = T(t + 1) * time_step - T(t) * time_step;
+            } else if (!lead_lag) {
+                v = x[(t + 1) * d_raw + c] - x[t * d_raw + c];
+            } else {
+                const int64_t k = t >> 1;
+                const bool odd = t & 1;
+                if (c < d_raw) v = odd ? x[(k + 1) * d_raw + c] - x[k * d_raw + c] : T(0);
+                else v = odd ? T(0) : x[(k + 1) * d_raw + (c - d_raw)] - x[k * d_raw + (c - d_raw)];
+            }
         }
         inc[e] = v;
     }
@@ -148,8 +156,11 @@ __device__ __forceinline__ typename Tree<T, D, N, TAIL, K>::Inc negate(const typ
 template <typename T, int D, int N, int TAIL, int K>
 __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d_rt,
-    int64_t out_stride, int scalar)
+    int64_t out_stride, int scalar, int nseg, int64_t lseg)
 {
+    // `batch` counts (path, time segment) pairs: item vb = path * nseg + segment sweeps the
+    // increments [segment * lseg, min(L, (segment + 1) * lseg)) and stores the signature of
+    // that piece in row vb of `out`.  nseg == 1 is the plain whole-path sweep.
     using Tr = Tree<T, D, N, TAIL, K>;
     constexpr int M = Tr::M;
     LaneCtx<T, D, N, TAIL, K> cx;
@@ -168,22 +179,26 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     // Two increment buffers used alternately: the loads of step t+1 are issued
     // before the arithmetic of step t and waited for after it, so neither the
     // scalar-cache nor the vector-memory latency sits on the critical path.
-    const T* base = inc + cx.id.b * L * d;
+    const int64_t seg = cx.id.b % nseg;
+    const int64_t t0 = seg * lseg;
+    const int64_t ns = (L - t0 < lseg) ? L - t0 : lseg;      // steps of this segment (>= 1)
+    const T* row = inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;     // row of the segment's first step
     typename Tr::Inc za, zb;
-    cx.load_inc(za, base);
+    cx.load_inc(za, row);
     wait_all_loads();
     int64_t t = 0;
-    for (; t + 2 <= L; t += 2) {
-        cx.load_inc(zb, base + (t + 1) * d);
+    for (; t + 2 <= ns; t += 2) {
+        cx.load_inc(zb, row + d);
         loads_issued();
         S.fwd_step(za);
         wait_all_loads();
-        cx.load_inc(za, base + ((t + 2 < L) ? t + 2 : t + 1) * d);
+        cx.load_inc(za, row + 2 * d);          // at most one row past the path: the zero guard row
         loads_issued();
         S.fwd_step(zb);
         wait_all_loads();
+        row += 2 * d;
     }
-    if (t < L) S.fwd_step(za);
+    if (t < ns) S.fwd_step(za);
 
     if (!cx.id.active) return;
     T* o = out + cx.id.b * out_stride;
@@ -415,20 +430,21 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     };
 
     // reverse sweep with two alternating increment buffers (see the forward kernel)
-    const T* base = inc + cx.id.b * L * d;
+    const T* row = inc + (cx.id.b * (L + 2) + L) * d;      // row of the last step
     typename Tr::Inc za, zb;
-    cx.load_inc(za, base + (L - 1) * d);
+    cx.load_inc(za, row);
     wait_all_loads();
     int64_t t = L - 1;
     for (; t >= 1; t -= 2) {
-        cx.load_inc(zb, base + (t - 1) * d);
+        cx.load_inc(zb, row - d);
         loads_issued();
         do_step(za, t);
         wait_all_loads();
-        cx.load_inc(za, base + ((t >= 2) ? t - 2 : 0) * d);
+        cx.load_inc(za, row - 2 * d);          // at most the zero guard row in front of the path
         loads_issued();
         do_step(zb, t - 1);
         wait_all_loads();
+        row -= 2 * d;
     }
     if (t == 0) do_step(za, 0);
 }
@@ -549,6 +565,47 @@ __global__ __launch_bounds__(kBlock) void degree_one_bwd_kernel(
         if (i == len_raw - 1) r += v;
         if (i == 0) r -= v;
         out[e] = r;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Chen product C = A (x) B of two signatures per path (scalar terms implicit 1):
+//   C_t[w] = A_t[w] + B_t[w] + sum_{k=1..t-1} A_k[w_1..w_k] * B_{t-k}[w_{k+1}..w_t]
+// (siglib/cpsig/cp_sig_combine.h:35-66).  One thread per output coefficient; rows
+// of A, B, C may have different strides and C may carry a leading scalar slot.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void sig_combine_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int64_t batch, int d, int degree,
+    int64_t sig_len /* sum_{k=1..degree} d^k */, int64_t a_stride, int64_t b_stride, int64_t c_stride,
+    int a_off, int b_off, int c_off)
+{
+    const int64_t total = batch * sig_len;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / sig_len;
+        int64_t r = e % sig_len;
+        // level t and word index w of coefficient r
+        int t = 1;
+        int64_t lvl = d, lo = 0;
+        while (r >= lo + lvl) { lo += lvl; lvl *= d; ++t; }
+        const int64_t w = r - lo;
+        const T* a = A + b * a_stride + a_off;
+        const T* bb = B + b * b_stride + b_off;
+        T acc = a[lo + w] + bb[lo + w];
+        // split w after its first k letters: prefix index w / d^(t-k), suffix index w % d^(t-k)
+        int64_t div = lvl / d;          // d^(t-1)
+        int64_t a_lo = 0, a_sz = d;     // level k of A
+        int64_t b_lo = lo - div;        // start of level t-1 of B
+        int64_t b_sz = div;
+        for (int k = 1; k < t; ++k) {
+            acc = fmadd(a[a_lo + w / div], bb[b_lo + w % div], acc);
+            a_lo += a_sz; a_sz *= d;
+            b_sz /= d; b_lo -= b_sz;
+            div /= d;
+        }
+        T* c = C + b * c_stride;
+        c[c_off + r] = acc;
+        if (c_off && r == 0) c[0] = T(1);
     }
 }
 

@@ -17,8 +17,20 @@ hipError_t launch_tree_fwd(const FwdParams& p)
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), 0, p.stream,
                        static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
-                       p.out_stride, p.scalar);
+                       p.out_stride, p.scalar, p.nseg, p.lseg);
     return hipGetLastError();
+}
+
+// resident waves per SIMD of the forward kernel (register-limited)
+template <typename T, int D, int N, int TAIL, int K>
+int fwd_waves_per_simd()
+{
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, tree_fwd_kernel<T, D, N, TAIL, K>, kBlock, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return 1;
+    }
+    return blocks < 1 ? 1 : blocks;
 }
 
 template <typename T, int D, int N, int TAIL, int K>

@@ -13,6 +13,8 @@ struct FwdParams {
     int64_t out_stride;
     int scalar;
     hipStream_t stream;
+    int nseg;        // time segments per path; batch counts (path, segment) items
+    int64_t lseg;    // increments per segment
 };
 
 struct BwdParams {
@@ -37,6 +39,7 @@ struct KernelEntry {
     BwdFn bwd;
     const char* name;
     int preferred;   // default partition of its shape
+    int (*waves_per_simd)();   // register-limited residency of the kernel
 };
 
 // every generated instance file contributes one array

@@ -273,6 +273,32 @@ def test_reused_buffers_and_repeatability(P, oracle):
                            oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)) <= 1e-10
 
 
+@pytest.mark.parametrize("segments", [1, 2, 3, 5, 8])
+def test_time_segmented_forward(P, oracle, segments):
+    """The forward sweep may split paths into time segments folded with Chen's identity; every split must agree."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    rng = np.random.default_rng(40 + segments)
+    cases = [((3, 17, 3, 4), {}, False), ((2, 64, 10, 5), {}, True), ((2, 9, 2, 6), dict(time_aug=True, lead_lag=True), False),
+             ((5, 4, 6, 3), {}, True), ((1, 100, 5, 7), {}, False), ((70, 23, 2, 3), dict(lead_lag=True), True)]
+    try:
+        L.CUSIG.cusig_amd_force_segments(segments)
+        for (shape, aug, scalar_term) in cases:
+            b, length, d, deg = shape
+            for dtype in (np.float64, np.float32):
+                x = (rng.standard_normal(shape[:3]) * 0.4).astype(dtype)
+                ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+                got = P.sig(dev(x), deg, scalar_term=scalar_term, **aug).cpu().numpy()
+                off = 1 if scalar_term else 0
+                d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+                if scalar_term:
+                    np.testing.assert_array_equal(got[:, 0], 1.0)
+                assert level_rel_err(got[:, off:], ref[:, off:], d_aug, deg) <= TOL[dtype], (shape, aug, dtype)
+    finally:
+        L.CUSIG.cusig_amd_force_segments(0)
+
+
 # ---- the benchmark workloads at full size -----------------------------------------------------------------
 
 @pytest.mark.parametrize("k", [1, 2, 4])
