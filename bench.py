@@ -19,6 +19,17 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 
+# HBM bytes per launch of the sweep kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
+# known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
+# reports null instead of a stale figure.
+TRAFFIC_BYTES = {
+    "fwd_f64_d10_n5_t2_k5": 54.7e6,
+    "bwd_f64_d10_n5_t2_k5": 156.1e6,
+    "fwd_f32_d5_n7_t2_k5": 77.9e6,
+    "fwd_f64_d3_n12_t4_k3": 466.8e6,
+    "fwd_f32_d17_n4_t1_k17": 318.2e6,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -27,6 +38,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-configs", action="store_true", help="also time configs 2-4 (reported under 'configs')")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="only run a plain 256 MiB device copy (calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     return ap.parse_args()
 
 
@@ -132,6 +145,17 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
 
+    if args.copy_calib:
+        n = 256 * 1024 * 1024 // 8
+        src = torch.arange(n, dtype=torch.float64, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calib_bytes_read": n * 8, "copy_calib_bytes_written": n * 8, "copies": 3}))
+        return
+
     r1 = Runner(1, torch, np, loader, cfgmod)
     r5 = Runner(5, torch, np, loader, cfgmod)
     r5.forward()            # the backward consumes the forward's signature
@@ -194,7 +218,8 @@ def main():
         "roofline": {
             "bound": "mfma", "pipe": "vector FP64 FMA (rank-1 updates: no MFMA tile applies; same 78.6 TFLOP/s peak)",
             "kernel": dominant["kernel"], "achieved": dominant["tflops"], "peak": peak, "unit": "TFLOP/s",
-            "frac": dominant["tflops"] / peak, "kernel_ms": dominant["ms"], "traffic": None,
+            "frac": dominant["tflops"] / peak, "kernel_ms": dominant["ms"],
+            "traffic": TRAFFIC_BYTES.get(dominant["kernel"]),
             "fwd_bwd_combined_frac": (r1.flops_fwd + r5.flops_bwd) / ((kms_f + kms_b) * 1e-3) / 1e12 / peak,
         },
         "configs": configs,
