@@ -12,7 +12,7 @@ import os
 from ctypes import POINTER, c_bool, c_char_p, c_double, c_float, c_int, c_uint64
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libcusig.so")
+LIB_PATH = os.environ.get("PYSIGLIB_AMD_LIB") or os.path.join(_HERE, "csrc", "libcusig.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(

@@ -31,6 +31,14 @@ OVERRIDES = {
 }
 
 
+# which twin (scalar-load or LDS-staged increments) a shape launches: 0 decide by occupancy at run time,
+# 1 always staged, 2 never staged.  Measured on MI355X at the benchmark workloads.
+STAGE_POLICY = {
+    ("f32", 5, 7, "fwd"): 1,
+    ("f32", 17, 4, "fwd"): 2,
+    ("f64", 3, 12, "fwd"): 2,
+}
+
 # additional partitions compiled next to the default one (selectable through
 # cusig_amd_force_partition; used for tuning sweeps): (dtype, D, N, dir) -> [(TAIL, K), ...]
 EXTRA = {
@@ -108,17 +116,19 @@ def main():
         for (D, N) in shapes:
             for direction in ("fwd", "bwd"):
                 tail, K = choose(D, N, dtype, direction)
-                insts.append((T, D, N, tail, K, direction, 1))
-                for (tl, kk) in EXTRA.get((dtype, D, N, direction), []):
-                    if (tl, kk) != (tail, K):
-                        insts.append((T, D, N, tl, kk, direction, 0))
+                parts = [(tail, K, 1)] + [(tl, kk, 0) for (tl, kk) in EXTRA.get((dtype, D, N, direction), [])
+                                          if (tl, kk) != (tail, K)]
+                for (tl, kk, pref) in parts:
+                    insts.append((T, D, N, tl, kk, direction, pref, 0))
+                    if D ** (N - tl) >= 48 and D <= 31:       # wide layout: also the LDS-staged variant
+                        insts.append((T, D, N, tl, kk, direction, pref, 1))
         for N in range(2, MAX_GENERIC_N + 1):
             for direction in ("fwd", "bwd"):
-                insts.append((T, 0, N, 1, GENERIC_K, direction, 1))
+                insts.append((T, 0, N, 1, GENERIC_K, direction, 1, 0))
 
     # balance files by a rough compile-cost estimate
     def weight(i):
-        T, D, N, tail, K, direction, pref = i
+        T, D, N, tail, K, direction, pref, zl = i
         w = K * (max(D, 1) ** tail) + N * N
         return w * (3 if direction == "bwd" else 1)
     insts.sort(key=weight, reverse=True)
@@ -137,25 +147,28 @@ def main():
         lines = ["// generated by gen_instances.py -- do not edit", '#include "../sig_launch.h"', "",
                  "namespace sigamd {", ""]
         # explicit kernel instantiations (seen by the device and the host pass)
-        for (T, D, N, tail, K, direction, pref) in bucket:
+        for (T, D, N, tail, K, direction, pref, zl) in bucket:
+            zs = "true" if zl else "false"
             if direction == "fwd":
-                lines.append("template __global__ void tree_fwd_kernel<%s, %d, %d, %d, %d>(const %s*, %s*, int64_t, "
-                             "int64_t, int, int64_t, int, int, int64_t);" % (T, D, N, tail, K, T, T))
+                lines.append("template __global__ void tree_fwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, %s*, int64_t, "
+                             "int64_t, int, int64_t, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T))
             else:
-                lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d>(const %s*, const %s*, "
-                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int);" % (T, D, N, tail, K, T, T, T, T))
+                lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
+                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int);" % (T, D, N, tail, K, zs, T, T, T, T))
         lines.append("")
         lines.append("#if !defined(__HIP_DEVICE_COMPILE__)   // the launcher table is host data")
         lines.append("static const KernelEntry kEntries_%02d[] = {" % fi)
-        for (T, D, N, tail, K, direction, pref) in bucket:
+        for (T, D, N, tail, K, direction, pref, zl) in bucket:
             is64 = 1 if T == "double" else 0
-            name = "%s_%s_d%d_n%d_t%d_k%d" % (direction, "f64" if is64 else "f32", D, N, tail, K)
+            zs = "true" if zl else "false"
+            pol = STAGE_POLICY.get(("f64" if is64 else "f32", D, N, direction), 0)
+            name = "%s_%s_d%d_n%d_t%d_k%d%s" % (direction, "f64" if is64 else "f32", D, N, tail, K, "_lds" if zl else "")
             if direction == "fwd":
-                lines.append('    {%d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d>},'
-                             % (is64, D, N, tail, K, T, D, N, tail, K, name, pref, T, D, N, tail, K))
+                lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
+                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))
             else:
-                lines.append('    {%d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d>, "%s", %d, nullptr},'
-                             % (is64, D, N, tail, K, T, D, N, tail, K, name, pref))
+                lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, nullptr, %d},'
+                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, pol))
         lines.append("};")
         lines.append("extern const EntryList kList_%02d = {kEntries_%02d, %d};" % (fi, fi, len(bucket)))
         lines.append("#endif")
@@ -177,8 +190,8 @@ def main():
     with open(os.path.join(args.out, "registry.cpp"), "w") as fh:
         fh.write("\n".join(reg))
     print("wrote %d instances into %d files under %s" % (len(insts), args.files, args.out))
-    for (T, D, N, tail, K, direction, pref) in sorted(insts, key=lambda i: (i[0], i[1], i[2], i[5])):
-        if (D, N) in ((10, 5), (5, 7), (3, 12), (17, 4)):
+    for (T, D, N, tail, K, direction, pref, zl) in sorted(insts, key=lambda i: (i[0], i[1], i[2], i[5])):
+        if (D, N) in ((10, 5), (5, 7), (3, 12), (17, 4)) and not zl:
             print("  ", T, D, N, direction, "tail", tail, "K", K, "default" if pref else "extra")
 
 

@@ -129,7 +129,7 @@ struct Table {
                 const KernelEntry* e = &lists[i].entries[j];
                 auto key = std::make_tuple(e->is_f64, e->D, e->N);
                 auto& slot = e->fwd ? fwd[key] : bwd[key];
-                if (e->preferred) slot.insert(slot.begin(), e);
+                if (e->preferred && !e->staged) slot.insert(slot.begin(), e);
                 else slot.push_back(e);
             }
     }
@@ -153,10 +153,21 @@ static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64
         if (it != m.end() && !it->second.empty()) {
             if (g_force_tail > 0)
                 for (const KernelEntry* e : it->second)
-                    if (e->tail == g_force_tail && e->k == g_force_k) return e;
+                    if (e->tail == g_force_tail && e->k == g_force_k && !e->staged) return e;
             return it->second.front();
         }
     }
+    return nullptr;
+}
+
+// the LDS-staged twin of a kernel instance (same partition), if one was compiled
+static const KernelEntry* staged_twin(bool backward, const KernelEntry* base)
+{
+    const auto& m = backward ? table().bwd : table().fwd;
+    auto it = m.find(std::make_tuple(base->is_f64, base->D, base->N));
+    if (it == m.end()) return nullptr;
+    for (const KernelEntry* e : it->second)
+        if (e->staged && e->tail == base->tail && e->k == base->k) return e;
     return nullptr;
 }
 
@@ -271,6 +282,21 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
     return int(std::max<int64_t>(g, 1));
 }
 
+// With at most two waves per SIMD the LDS-staged twin (all-VGPR FMAs, HBM latency hidden by a chunk of
+// arithmetic) is the faster way to feed increments; with more resident waves the scalar path costs nothing.
+static int g_force_staged = -1;   // tuning hook: -1 automatic, 0 never, 1 whenever compiled
+
+static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, int64_t waves)
+{
+    const bool want = g_force_staged >= 0 ? g_force_staged != 0
+                      : base->stage_policy == 1 ? true
+                      : base->stage_policy == 2 ? false
+                                                : waves <= 2 * int64_t(simd_count());
+    if (!want) return base;
+    const KernelEntry* twin = staged_twin(backward, base);
+    return twin ? twin : base;
+}
+
 // ---------------------------------------------------------------------------
 // shared argument handling
 // ---------------------------------------------------------------------------
@@ -375,7 +401,8 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                                      ", degree " + std::to_string(degree) + " in this build");
         std::lock_guard<std::mutex> lk(g_ws_mutex);
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
-        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;    // staged sweeps read whole chunks past either end
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
         // Few paths cannot fill the chip with whole-path sweeps: split every path into time segments,
         // sweep all (path, segment) pairs concurrently and fold the pieces with Chen's identity.
@@ -404,6 +431,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             }
             p.out = segs; p.out_stride = int64_t(n_coef); p.scalar = 0;
         }
+        e = pick_variant(false, e, total_waves(geom, p.batch));
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->fwd(p));
         timer.stop();
@@ -465,7 +493,8 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         std::lock_guard<std::mutex> lk(g_ws_mutex);
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
-        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
         T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
         hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(dz_elems)), dim3(kBlock), 0, stream, dzinc,
@@ -474,6 +503,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         BwdParams p;
         p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
         p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
+        e = pick_variant(true, e, total_waves(make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0), int64_t(batch)));
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->bwd(p));
         timer.stop();
@@ -555,6 +585,8 @@ CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
 
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
+
+CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {

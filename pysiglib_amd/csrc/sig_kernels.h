@@ -150,10 +150,153 @@ __device__ __forceinline__ typename Tree<T, D, N, TAIL, K>::Inc negate(const typ
     return o;
 }
 
+
+// ---------------------------------------------------------------------------
+// Sweep drivers: feed the increments of steps first, first + DIR, ... (count
+// steps) to step(z, t).  Two ways of getting an increment row to a wave:
+//
+//  * scalar path (any layout): the row is read where it lies in HBM/L2 with two
+//    alternating register sets; the loads of the next step are issued before the
+//    arithmetic of the current one.  In the wide layout the row address is
+//    wave-uniform, so the row arrives in SGPRs through the scalar cache.
+//
+//  * staged path (wide layout only): every wave copies chunks of kStageSteps
+//    rows into a private LDS ring two chunks ahead of use (ordinary vector loads,
+//    so HBM latency is hidden by a whole chunk of arithmetic) and reads each row
+//    back with broadcast LDS reads one step ahead.  The row then sits in VGPRs:
+//    an FMA whose operands are all VGPRs issues faster than one reading an SGPR
+//    when a SIMD holds only one or two waves, which is the regime of small batches.
+// ---------------------------------------------------------------------------
+constexpr int kStageSteps = 16;
+
+template <typename T, int D, int DIR>
+struct IncRing {
+    static constexpr int CS = kStageSteps;
+    static constexpr int CHUNK = CS * D;                       // elements per chunk
+    static constexpr int NREG = (CHUNK + kWave - 1) / kWave;   // elements per lane per chunk
+    static constexpr int ELEMS = 2 * CHUNK + D;                // two chunks and one wrap row
+    // DIR > 0: [even chunk][odd chunk][copy of row 0 of the even chunk]
+    // DIR < 0: [copy of the last row of the even chunk][odd chunk][even chunk]
+    __host__ __device__ static constexpr int base(int parity)
+    {
+        return DIR > 0 ? parity * CHUNK : D + (1 - parity) * CHUNK;
+    }
+    T* lds;
+    int lane;
+    T regs[NREG];
+
+    __device__ __forceinline__ void issue(const T* __restrict__ g)
+    {
+#pragma unroll
+        for (int i = 0; i < NREG; ++i) {
+            const int e = lane + kWave * i;
+            regs[i] = ((i + 1) * kWave <= CHUNK || e < CHUNK) ? g[e] : T(0);
+        }
+    }
+    __device__ __forceinline__ void commit(int parity)
+    {
+        T* dst = lds + base(parity);
+#pragma unroll
+        for (int i = 0; i < NREG; ++i) {
+            const int e = lane + kWave * i;
+            if ((i + 1) * kWave <= CHUNK || e < CHUNK) {
+                dst[e] = regs[i];
+                if (parity == 0) {
+                    if (DIR > 0) { if (e < D) lds[2 * CHUNK + e] = regs[i]; }
+                    else { if (e >= CHUNK - D) lds[e - (CHUNK - D)] = regs[i]; }
+                }
+            }
+        }
+    }
+};
+
+// scalar path
+template <int DIR, typename Cx, typename Inc, typename T, typename StepFn>
+__device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
+                                             StepFn&& step)
+{
+    const int d = cx.d;
+    Inc za, zb;
+    cx.load_inc(za, row);
+    wait_all_loads();
+    int64_t i = 0;
+    for (; i + 2 <= count; i += 2) {
+        cx.load_inc(zb, row + DIR * d);
+        loads_issued();
+        step(za, first + DIR * i);
+        wait_all_loads();
+        cx.load_inc(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
+        loads_issued();
+        step(zb, first + DIR * (i + 1));
+        wait_all_loads();
+        row += 2 * DIR * d;
+    }
+    if (i < count) step(za, first + DIR * i);
+}
+
+// staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0
+template <int DIR, int G0, typename Tr, typename Cx, typename T, typename StepFn>
+__device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
+                                             T* lds_wave, StepFn&& step)
+{
+    constexpr int D = Tr::DD;
+    using Ring = IncRing<T, D, DIR>;
+    constexpr int CS = Ring::CS;
+    Ring ring;
+    ring.lds = lds_wave;
+    ring.lane = threadIdx.x & (kWave - 1);
+    // memory start of chunk k: DIR > 0: row + k * CHUNK;  DIR < 0: the CS rows ending with the row of step first - k*CS
+    auto chunk_src = [&](int64_t k) -> const T* {
+        return DIR > 0 ? row + k * Ring::CHUNK : row - (k * CS + (CS - 1)) * D;
+    };
+    const int64_t nchunks = (count + CS - 1) / CS;
+
+    auto load_row = [&](typename Tr::Inc& in, const T* lp) {
+        if constexpr (Tr::TAIL_ >= 2) {
+#pragma unroll
+            for (int j = 0; j < D; ++j) in.z[j] = lp[j];
+        }
+#pragma unroll
+        for (int a = 0; a < Tr::K_; ++a) {
+            if constexpr (G0 >= 0 && Tr::TAIL_ >= 2) in.zs[a] = (G0 + a < D) ? in.z[(G0 + a < D) ? G0 + a : 0] : T(0);
+            else if constexpr (G0 >= 0) in.zs[a] = (G0 + a < D) ? lp[(G0 + a < D) ? G0 + a : 0] : T(0);
+            else in.zs[a] = (cx.a0 + a < D) ? lp[cx.a0 + a] : T(0);
+        }
+#pragma unroll
+        for (int l = 0; l < Tr::M; ++l) in.pz[l] = lp[cx.p[l]];
+    };
+
+    ring.issue(chunk_src(0));
+    ring.commit(0);
+    if (nchunks > 1) ring.issue(chunk_src(1));
+    typename Tr::Inc za, zb;
+    load_row(za, ring.lds + Ring::base(0) + (DIR > 0 ? 0 : (CS - 1) * D));
+    int64_t done = 0;
+    for (int64_t k = 0; k < nchunks; ++k) {
+        const int parity = int(k & 1);
+        if (k + 1 < nchunks) ring.commit(parity ^ 1);            // chunk k+1 becomes readable
+        if (k + 2 < nchunks) ring.issue(chunk_src(k + 2));       // two chunks ahead of use
+        const T* lp = ring.lds + Ring::base(parity) + (DIR > 0 ? 0 : (CS - 1) * D);
+        const int nk = int((count - done < CS) ? count - done : CS);
+        int i = 0;
+        for (; i + 2 <= nk; i += 2) {
+            load_row(zb, lp + DIR * D);
+            loads_issued();
+            step(za, first + DIR * (done + i));
+            load_row(za, lp + 2 * DIR * D);                      // may be row 0 of the next chunk (contiguous or wrap copy)
+            loads_issued();
+            step(zb, first + DIR * (done + i + 1));
+            lp += 2 * DIR * D;
+        }
+        if (i < nk) step(za, first + DIR * (done + i));          // odd tail: only in the last chunk
+        done += nk;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Forward sweep.
 // ---------------------------------------------------------------------------
-template <typename T, int D, int N, int TAIL, int K>
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d_rt,
     int64_t out_stride, int scalar, int nseg, int64_t lseg)
@@ -176,29 +319,27 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
 #pragma unroll
     for (int i = 0; i < Tr::SUB; ++i) S.s[i] = T(0);
 
-    // Two increment buffers used alternately: the loads of step t+1 are issued
-    // before the arithmetic of step t and waited for after it, so neither the
-    // scalar-cache nor the vector-memory latency sits on the critical path.
     const int64_t seg = cx.id.b % nseg;
     const int64_t t0 = seg * lseg;
     const int64_t ns = (L - t0 < lseg) ? L - t0 : lseg;      // steps of this segment (>= 1)
     const T* row = inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;     // row of the segment's first step
-    typename Tr::Inc za, zb;
-    cx.load_inc(za, row);
-    wait_all_loads();
-    int64_t t = 0;
-    for (; t + 2 <= ns; t += 2) {
-        cx.load_inc(zb, row + d);
-        loads_issued();
-        S.fwd_step(za);
-        wait_all_loads();
-        cx.load_inc(za, row + 2 * d);          // at most one row past the path: the zero guard row
-        loads_issued();
-        S.fwd_step(zb);
-        wait_all_loads();
-        row += 2 * d;
+    auto step = [&](const typename Tr::Inc& z, int64_t) { S.fwd_step(z); };
+    if constexpr (ZL) {
+        static_assert(LaneCtx<T, D, N, TAIL, K>::WIDE, "staged increments need the wide layout");
+        extern __shared__ double lds_raw_f[];
+        T* lds_wave = reinterpret_cast<T*>(lds_raw_f) + (threadIdx.x >> 6) * IncRing<T, Tr::DD, 1>::ELEMS;
+        constexpr int NG = (Tr::DD + K - 1) / K;
+        if constexpr (NG <= 3) {
+            static_for<0, NG - 1>([&](auto gc) {
+                if (cx.id.g == decltype(gc)::value)
+                    sweep_staged<1, decltype(gc)::value * K, Tr>(cx, row, t0, ns, lds_wave, step);
+            });
+        } else {
+            sweep_staged<1, -1, Tr>(cx, row, t0, ns, lds_wave, step);
+        }
+    } else {
+        sweep_direct<1, LaneCtx<T, D, N, TAIL, K>, typename Tr::Inc>(cx, row, t0, ns, step);
     }
-    if (t < ns) S.fwd_step(za);
 
     if (!cx.id.active) return;
     T* o = out + cx.id.b * out_stride;
@@ -249,7 +390,7 @@ __device__ __forceinline__ void dev_add(T* p, T v)
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename T, int D, int N, int TAIL, int K>
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
     T* __restrict__ dzinc, int64_t batch, int64_t L, int d_rt, int64_t sig_stride, int scalar,
@@ -429,24 +570,22 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         }
     };
 
-    // reverse sweep with two alternating increment buffers (see the forward kernel)
     const T* row = inc + (cx.id.b * (L + 2) + L) * d;      // row of the last step
-    typename Tr::Inc za, zb;
-    cx.load_inc(za, row);
-    wait_all_loads();
-    int64_t t = L - 1;
-    for (; t >= 1; t -= 2) {
-        cx.load_inc(zb, row - d);
-        loads_issued();
-        do_step(za, t);
-        wait_all_loads();
-        cx.load_inc(za, row - 2 * d);          // at most the zero guard row in front of the path
-        loads_issued();
-        do_step(zb, t - 1);
-        wait_all_loads();
-        row -= 2 * d;
+    if constexpr (ZL) {
+        static_assert(WIDE, "staged increments need the wide layout");
+        T* lds_wave = lds + kWavesPerBlock * (CH * Tr::DD * kRedStride) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
+        constexpr int NG = (Tr::DD + K - 1) / K;
+        if constexpr (NG <= 3) {
+            static_for<0, NG - 1>([&](auto gc) {
+                if (cx.id.g == decltype(gc)::value)
+                    sweep_staged<-1, decltype(gc)::value * K, Tr>(cx, row, L - 1, L, lds_wave, do_step);
+            });
+        } else {
+            sweep_staged<-1, -1, Tr>(cx, row, L - 1, L, lds_wave, do_step);
+        }
+    } else {
+        sweep_direct<-1, Cx, typename Tr::Inc>(cx, row, L - 1, L, do_step);
     }
-    if (t == 0) do_step(za, 0);
 }
 
 // ---------------------------------------------------------------------------

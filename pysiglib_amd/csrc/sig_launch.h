@@ -7,33 +7,50 @@ namespace sigamd {
 
 constexpr int64_t kMaxGridX = 2147483647LL;
 constexpr size_t kMaxDynLds = 64 * 1024;
+constexpr size_t kMaxLdsPerBlock = 160 * 1024;
 
-template <typename T, int D, int N, int TAIL, int K>
+// dynamic LDS above 64 KB has to be requested once per kernel
+template <typename Kern>
+hipError_t allow_lds(Kern kern, size_t bytes)
+{
+    if (bytes <= kMaxDynLds) return hipSuccess;
+    if (bytes > kMaxLdsPerBlock) return hipErrorInvalidConfiguration;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+}
+
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
 hipError_t launch_tree_fwd(const FwdParams& p)
 {
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), 0, p.stream,
+    size_t lds = 0;
+    if (ZL) {
+        if (!g.wide) return hipErrorInvalidConfiguration;
+        lds = size_t(kWavesPerBlock) * IncRing<T, (D > 0 ? D : 1), 1>::ELEMS * sizeof(T);
+        hipError_t e = allow_lds(tree_fwd_kernel<T, D, N, TAIL, K, ZL>, lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
                        p.out_stride, p.scalar, p.nseg, p.lseg);
     return hipGetLastError();
 }
 
 // resident waves per SIMD of the forward kernel (register-limited)
-template <typename T, int D, int N, int TAIL, int K>
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
 int fwd_waves_per_simd()
 {
     int blocks = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, tree_fwd_kernel<T, D, N, TAIL, K>, kBlock, 0) != hipSuccess) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, tree_fwd_kernel<T, D, N, TAIL, K, ZL>, kBlock, 0) != hipSuccess) {
         (void)hipGetLastError();
         return 1;
     }
     return blocks < 1 ? 1 : blocks;
 }
 
-template <typename T, int D, int N, int TAIL, int K>
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
@@ -49,8 +66,15 @@ hipError_t launch_tree_bwd(const BwdParams& p)
         lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
         if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
     }
-    if (lds > kMaxDynLds) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
+    if (ZL) {
+        if (!g.wide) return hipErrorInvalidConfiguration;
+        lds += size_t(kWavesPerBlock) * IncRing<T, (D > 0 ? D : 1), -1>::ELEMS * sizeof(T);
+    }
+    {
+        hipError_t e = allow_lds(tree_bwd_kernel<T, D, N, TAIL, K, ZL>, lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
                        static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,
                        p.sig_stride, p.scalar, use_lds);

@@ -35,11 +35,13 @@ typedef hipError_t (*BwdFn)(const BwdParams&);
 // D == 0: run-time dimension.  Exactly one of fwd / bwd is set.
 struct KernelEntry {
     int is_f64, D, N, tail, k;
+    int staged;      // 1: increments staged through LDS into VGPRs (wide layout, low occupancy)
     FwdFn fwd;
     BwdFn bwd;
     const char* name;
     int preferred;   // default partition of its shape
     int (*waves_per_simd)();   // register-limited residency of the kernel
+    int stage_policy;          // which twin to launch: 0 by occupancy, 1 always the staged one, 2 never
 };
 
 // every generated instance file contributes one array

@@ -136,6 +136,8 @@ struct Tree {
     static_assert(D > 0 || TAIL == 1, "run-time dimension supports depth-1 subtrees only");
     static constexpr int M = N - TAIL;
     static constexpr int DD = D > 0 ? D : 1;
+    static constexpr int TAIL_ = TAIL;
+    static constexpr int K_ = K;
     // subtree depth e (1-based) holds K * D^(e-1) values starting at off(e)
     __host__ __device__ static constexpr int cnt(int e) { return K * int(ipow64(DD, e - 1)); }
     __host__ __device__ static constexpr int off(int e)
