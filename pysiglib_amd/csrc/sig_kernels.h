@@ -210,6 +210,15 @@ struct IncRing {
     }
 };
 
+template <typename T>
+__device__ __forceinline__ const T* opaque_lds(const T* p)
+{
+    typedef const T __attribute__((address_space(3))) * LdsPtr;
+    uint32_t a = uint32_t(reinterpret_cast<uintptr_t>((LdsPtr)p));
+    asm volatile("" : "+v"(a));
+    return (const T*)reinterpret_cast<LdsPtr>(uintptr_t(a));
+}
+
 // scalar path
 template <int DIR, typename Cx, typename Inc, typename T, typename StepFn>
 __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
@@ -276,7 +285,8 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
         const int parity = int(k & 1);
         if (k + 1 < nchunks) ring.commit(parity ^ 1);            // chunk k+1 becomes readable
         if (k + 2 < nchunks) ring.issue(chunk_src(k + 2));       // two chunks ahead of use
-        const T* lp = ring.lds + Ring::base(parity) + (DIR > 0 ? 0 : (CS - 1) * D);
+        // the row pointer is made opaque so that row reads use small immediate offsets from one VGPR
+        const T* lp = opaque_lds(ring.lds + Ring::base(parity) + (DIR > 0 ? 0 : (CS - 1) * D));
         const int nk = int((count - done < CS) ? count - done : CS);
         int i = 0;
         for (; i + 2 <= nk; i += 2) {

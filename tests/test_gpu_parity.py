@@ -299,6 +299,37 @@ def test_time_segmented_forward(P, oracle, segments):
         L.CUSIG.cusig_amd_force_segments(0)
 
 
+@pytest.mark.parametrize("shape,dtype", [
+    ((2, 5, 98, 2), np.float64), ((2, 4, 350, 2), np.float32), ((1, 3, 1000, 2), np.float64),     # wide paths, low degree
+    ((70000, 3, 2, 2), np.float32), ((66000, 4, 3, 3), np.float64),                                # batch beyond 65535
+    ((3, 2000, 2, 4), np.float64), ((1, 20001, 3, 3), np.float64),                                 # long paths
+    ((2, 6, 2, 16), np.float64), ((1, 4, 3, 11), np.float64),                                      # highest compiled degrees
+])
+def test_extreme_shapes(P, oracle, shape, dtype):
+    """Shapes the reference's GPU suite probes for its launch and memory limits
+    (tests/test_signature_cuda_shared_memory.py, tests/test_cuda_grid_limits.py of the reference)."""
+    b, length, d, deg = shape
+    rng = np.random.default_rng(b + length + d + deg)
+    scale = 1.0 / np.sqrt(length) if length > 100 else 0.5
+    x = np.cumsum(rng.standard_normal((b, length, d)) * scale, axis=1).astype(dtype)
+    ref = oracle.signature(x, deg, n_jobs=-1)
+    got = P.sig(dev(x), deg).cpu().numpy()
+    assert level_rel_err(got, ref, d, deg) <= TOL[dtype]
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    ref_b = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
+    got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+    assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
+
+
+def test_wide_degree_one(P):
+    x = torch.randn(3, 2, 200000, dtype=torch.float32, device=DEV)
+    torch.testing.assert_close(P.sig(x, 1), x[:, 1] - x[:, 0])
+    g = torch.randn(3, 200000, dtype=torch.float32, device=DEV)
+    grad = P.sig_backprop(x, P.sig(x, 1), g, 1)
+    torch.testing.assert_close(grad[:, 1], g)
+    torch.testing.assert_close(grad[:, 0], -g)
+
+
 # ---- the benchmark workloads at full size -----------------------------------------------------------------
 
 @pytest.mark.parametrize("k", [1, 2, 4])
