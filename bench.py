@@ -23,10 +23,10 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 # known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
 # reports null instead of a stale figure.
 TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5": 54.7e6,
-    "bwd_f64_d10_n5_t2_k5": 156.1e6,
-    "fwd_f32_d5_n7_t2_k5": 77.9e6,
-    "fwd_f64_d3_n12_t4_k3": 466.8e6,
+    "fwd_f64_d10_n5_t2_k5_lds": 53.0e6,
+    "bwd_f64_d10_n5_t2_k5_lds": 152.0e6,
+    "fwd_f32_d5_n7_t2_k5_lds": 71.4e6,
+    "fwd_f64_d3_n12_t4_k3": 466.7e6,
     "fwd_f32_d17_n4_t1_k17": 318.2e6,
 }
 

@@ -525,16 +525,15 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         if constexpr (WIDE) {
             T* tile = wbuf + cs * (Tr::DD * kRedStride) + woff;
 #pragma unroll
-            for (int j = 0; j < Tr::DD; ++j) tile[j * kRedStride] = (active && TAIL >= 2) ? dz.dj[j] : T(0);
-            if (active) {
-                // depth-1 letters (wave-uniform rows) and chain letters (per-lane rows) are
-                // added into the lane's own column; LDS executes a wave's operations in order
+            for (int j = 0; j < Tr::DD; ++j) tile[j * kRedStride] = (TAIL >= 2) ? dz.dj[j] : T(0);
+            // depth-1 letters (wave-uniform rows) and chain letters (per-lane rows) are added into the
+            // lane's own column; LDS executes a wave's operations in order.  Idle lanes need no
+            // predicate: their adjoints were loaded as zero, so every piece they produce is zero.
 #pragma unroll
-                for (int a = 0; a < K; ++a)
-                    if (cx.a0 + a < Tr::DD) lds_add(&tile[(cx.a0 + a) * kRedStride], dz.da[a]);
+            for (int a = 0; a < K; ++a)
+                if (cx.a0 + a < Tr::DD) lds_add(&tile[(cx.a0 + a) * kRedStride], dz.da[a]);
 #pragma unroll
-                for (int l = 0; l < M; ++l) lds_add(&tile[cx.p[l] * kRedStride], dz.dc[l]);
-            }
+            for (int l = 0; l < M; ++l) lds_add(&tile[cx.p[l] * kRedStride], dz.dc[l]);
             ++cs;
             if (cs == CH || t == 0) {
                 reduce_chunk(cs);
