@@ -144,6 +144,24 @@ static const Table& table()
     return t;
 }
 
+static int simd_count();
+static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64_t degree);
+static double sweep_estimate(const KernelEntry* e, int d, int64_t batch);
+
+// The specialised partition of a shape is tuned for a full chip; with few paths its few, heavy lanes make every
+// one of the L dependent steps slow.  Then the run-time-dimension kernel (one word prefix per lane, many light
+// lanes) finishes sooner even though it issues more instructions in total.
+static const KernelEntry* choose_entry(bool backward, bool f64, uint64_t d, uint64_t degree, uint64_t batch)
+{
+    const KernelEntry* spec = find_entry(backward, f64, d, degree);
+    if (!spec || spec->D == 0 || g_force_tail > 0) return spec;
+    const auto& m = backward ? table().bwd : table().fwd;
+    auto it = m.find(std::make_tuple(int(f64), 0, int(degree)));
+    if (it == m.end() || it->second.empty()) return spec;
+    const KernelEntry* gen = it->second.front();
+    return sweep_estimate(gen, int(d), int64_t(batch)) < 0.7 * sweep_estimate(spec, int(d), int64_t(batch)) ? gen : spec;
+}
+
 static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64_t degree)
 {
     const auto& m = backward ? table().bwd : table().fwd;
@@ -158,6 +176,37 @@ static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64
         }
     }
     return nullptr;
+}
+
+// Rough VALU instruction count of one forward step of one lane for partition (tail, k); the backward costs a
+// near-constant multiple of it, so the same figure ranks partitions for both sweeps.
+static double lane_step_cost(int d, int n, int tail, int k)
+{
+    const int m = n - tail;
+    double cost = m;
+    for (int t = 1; t <= n; ++t) {
+        if (t == 1) cost += 1;
+        else if (t <= m) cost += 2.0 * (t - 1);
+        else {
+            cost += 1 + 2.0 * (m - 1);
+            double nodes = k;
+            for (int e = 1; e <= t - m; ++e) {
+                cost += (e == t - m) ? nodes : 2.0 * nodes + nodes / (e == 1 ? k : d);
+                nodes *= d;
+            }
+        }
+    }
+    return cost;
+}
+
+// A sweep is a chain of L dependent steps: its duration is L times the longer of one lane-step (latency of a
+// lone wave) and the chip-wide issue time of all waves' steps.  Returns a relative figure.
+static double sweep_estimate(const KernelEntry* e, int d, int64_t batch)
+{
+    const TreeGeom g = make_geom(d, e->N - e->tail, e->k, e->D > 0);
+    const double rounds = double(total_waves(g, batch)) / double(simd_count());
+    const double per_step = lane_step_cost(d, e->N, e->tail, e->k) * (e->D > 0 ? 1.0 : 1.15);
+    return per_step * std::max(1.0, rounds * 0.8);
 }
 
 // the LDS-staged twin of a kernel instance (same partition), if one was compiled
@@ -395,7 +444,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                            path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), time_step, sc);
     } else {
-        const KernelEntry* e = find_entry(false, sizeof(T) == 8, s.d_aug, degree);
+        const KernelEntry* e = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch);
         if (!e)
             throw std::runtime_error("signature_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
@@ -486,7 +535,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                            sig_derivs, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), sc);
     } else {
-        const KernelEntry* e = find_entry(true, sizeof(T) == 8, s.d_aug, degree);
+        const KernelEntry* e = choose_entry(true, sizeof(T) == 8, s.d_aug, degree, batch);
         if (!e)
             throw std::runtime_error("sig_backprop_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");

@@ -219,25 +219,26 @@ __device__ __forceinline__ const T* opaque_lds(const T* p)
     return (const T*)reinterpret_cast<LdsPtr>(uintptr_t(a));
 }
 
-// scalar path
-template <int DIR, typename Cx, typename Inc, typename T, typename StepFn>
+// scalar path.  WAIT_ALL: end every step with a full wait for outstanding loads (cheapest schedule when the
+// step issues no stores); the backward must not do that, because a full wait would also wait for the
+// acknowledgement of the global atomics it fires, so there the compiler's per-register waits are used.
+template <int DIR, bool WAIT_ALL, typename Cx, typename Inc, typename T, typename StepFn>
 __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
                                              StepFn&& step)
 {
     const int d = cx.d;
     Inc za, zb;
     cx.load_inc(za, row);
-    wait_all_loads();
     int64_t i = 0;
     for (; i + 2 <= count; i += 2) {
         cx.load_inc(zb, row + DIR * d);
         loads_issued();
         step(za, first + DIR * i);
-        wait_all_loads();
+        if constexpr (WAIT_ALL) wait_all_loads();
         cx.load_inc(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
         loads_issued();
         step(zb, first + DIR * (i + 1));
-        wait_all_loads();
+        if constexpr (WAIT_ALL) wait_all_loads();
         row += 2 * DIR * d;
     }
     if (i < count) step(za, first + DIR * i);
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
             sweep_staged<1, -1, Tr>(cx, row, t0, ns, lds_wave, step);
         }
     } else {
-        sweep_direct<1, LaneCtx<T, D, N, TAIL, K>, typename Tr::Inc>(cx, row, t0, ns, step);
+        sweep_direct<1, true, LaneCtx<T, D, N, TAIL, K>, typename Tr::Inc>(cx, row, t0, ns, step);
     }
 
     if (!cx.id.active) return;
@@ -383,11 +384,25 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
 // back through the step, emit the increment gradient.
 // (siglib/cpsig/cp_signature.h:1137-1187)
 // ---------------------------------------------------------------------------
-// LDS tile of the wide-layout reduction: one row per (step-in-chunk, letter), two
-// half-rows of 32 lanes padded to 33 so that writers and the summing lanes both
-// hit distinct banks.
-constexpr int kRedStride = 66;
-__host__ __device__ constexpr int bwd_chunk(int d) { return (31 / d) < 1 ? 1 : ((31 / d) > 8 ? 8 : (31 / d)); }
+// LDS tile of the increment-gradient reduction: one row per (step-in-chunk, letter), one column per lane.
+constexpr int kRedStride = 65;
+// steps per chunk of the reduction tile (at most 16 KB of LDS per wave); 0: the path is too wide for the tile
+template <typename T>
+__host__ __device__ constexpr int red_chunk(int d)
+{
+    const int rows = int(16384 / (kRedStride * sizeof(T)));     // 31 (f64) / 63 (f32)
+    return d > rows ? 0 : (rows / d > 8 ? 8 : rows / d);
+}
+
+// Orders the LDS traffic of ONE wave: the hardware executes a wave's LDS operations in issue order, so lanes
+// see each other's earlier writes and atomics without any wait; only the compiler has to be kept from moving
+// memory operations across this point.  (A memory fence would also wait for the global atomics in flight.)
+__device__ __forceinline__ void wave_lds_sync()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+}
 
 template <typename T>
 __device__ __forceinline__ void lds_add(T* p, T v)
@@ -454,61 +469,71 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     });
 
     // ---- reduction of the per-lane increment-gradient pieces ------------
-    // wide layout: every lane writes its D partial sums of a step into a
-    // [row = step-in-chunk * D + letter][lane] tile in LDS (chain pieces are added
-    // into the lane's own column); once the chunk is full each row is summed by
-    // a pair of lanes and added to dz[b][t][letter] in HBM.  packed layout:
-    // per-wave accumulator [path-in-wave][letter] updated with LDS atomics.
+    // Every lane adds its pieces of a step into its own column of an LDS tile
+    // [row = step-in-chunk * d + letter][lane] (row stride 65: writers and summing lanes both hit distinct
+    // banks; own column: no atomic ever collides).  When the chunk is full each (row, column segment) is
+    // summed by one lane and added to dz[path][step][letter] in HBM.  Column segments: the lanes of one path
+    // when several whole paths share the wave, else two halves of the wave.  Paths too wide for the tile
+    // (d > 31 in f64, d > 63 in f32) fall back to a per-wave accumulator updated with LDS atomics, whose
+    // collisions are rare exactly because d is large.
     const int lane = threadIdx.x & (kWave - 1);
     const int wave_in_block = threadIdx.x >> 6;
     constexpr bool WIDE = Cx::WIDE;
-    constexpr int CH = bwd_chunk(Tr::DD);
-    const int slots = cx.G.ppw;
-    T* wbuf;
-    if constexpr (WIDE) wbuf = lds + wave_in_block * (CH * Tr::DD * kRedStride);
-    else wbuf = lds + int64_t(wave_in_block) * slots * d;
+    const int CH = red_chunk<T>(d);
+    const bool tiled = CH > 0;
+    const int slots = WIDE ? 1 : cx.G.ppw;
+    T* wbuf = lds + int64_t(wave_in_block) * (tiled ? int64_t(CH) * d * kRedStride : int64_t(slots) * d);
     T* acc = wbuf + int64_t(cx.id.slot) * d;
-    const int woff = (lane >> 5) * 33 + (lane & 31);
-    if constexpr (!WIDE) {
-        if (use_lds) {
-            for (int e = lane; e < slots * d; e += kWave) wbuf[e] = T(0);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_wave_barrier();
-        }
+    const int nsg = slots > 1 ? slots : 2;                    // column segments per row
+    const int seg_cnt = slots > 1 ? int(cx.G.lpp) : kWave / 2; // lanes per segment
+    if (!tiled && use_lds) {
+        for (int e = lane; e < slots * d; e += kWave) wbuf[e] = T(0);
+        wave_lds_sync();
     }
     int64_t b_first;
     {
         const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + wave_in_block;
-        b_first = (cx.G.ppw > 1) ? wave * cx.G.ppw : (wave / cx.G.wpp);
+        b_first = (slots > 1) ? wave * slots : (wave / cx.G.wpp);
     }
-    int cs = 0;                 // rows of the current chunk already filled (in steps)
+    int cs = 0;                 // steps already written into the current chunk
     int64_t t_chunk = L - 1;    // step held by chunk slot 0
 
     auto reduce_chunk = [&](int n_slots) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        const int n_rows = n_slots * Tr::DD;
-        for (int h = lane; h < 2 * n_rows; h += kWave) {
-            const int rowi = h >> 1, half = h & 1;
-            const T* src = wbuf + rowi * kRedStride + half * 33;
+        wave_lds_sync();
+        const int items = n_slots * d * nsg;
+        for (int it = lane; it < items; it += kWave) {
+            const int sg = it % nsg, r = it / nsg;
+            const T* src = wbuf + r * kRedStride + sg * seg_cnt;
             T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
+            if (seg_cnt == kWave / 2) {
 #pragma unroll
-            for (int i = 0; i < 32; i += 4) {
-                s0 += src[i];
-                s1 += src[i + 1];
-                s2 += src[i + 2];
-                s3 += src[i + 3];
+                for (int i = 0; i < kWave / 2; i += 4) {
+                    s0 += src[i];
+                    s1 += src[i + 1];
+                    s2 += src[i + 2];
+                    s3 += src[i + 3];
+                }
+            } else {
+                int i = 0;
+                for (; i + 4 <= seg_cnt; i += 4) {
+                    s0 += src[i];
+                    s1 += src[i + 1];
+                    s2 += src[i + 2];
+                    s3 += src[i + 3];
+                }
+                for (; i < seg_cnt; ++i) s0 += src[i];
             }
             T sum = (s0 + s1) + (s2 + s3);
-            sum += __shfl_xor(sum, 1);
-            if (half == 0) {
-                const int slot = rowi / Tr::DD, j = rowi % Tr::DD;
-                dev_add(&dzinc[(cx.id.b * L + (t_chunk - slot)) * d + j], sum);
+            const int slot = r / d, j = r % d;
+            if (slots > 1) {
+                const int64_t bb = b_first + sg;
+                if (bb < batch) dev_add(&dzinc[(bb * L + (t_chunk - slot)) * d + j], sum);
+            } else {
+                sum += __shfl_xor(sum, 1);      // the two halves of a row sit in neighbouring lanes
+                if (sg == 0 && b_first < batch) dev_add(&dzinc[(b_first * L + (t_chunk - slot)) * d + j], sum);
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
+        wave_lds_sync();
     };
 
     auto do_step = [&](const typename Tr::Inc& z, int64_t t) {
@@ -522,18 +547,21 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
         A.pullback(S, z, dz);
 
-        if constexpr (WIDE) {
-            T* tile = wbuf + cs * (Tr::DD * kRedStride) + woff;
+        if (tiled) {
+            // Idle lanes need no predicate: their adjoints were loaded as zero, so every piece they produce is zero.
+            T* col = wbuf + cs * (d * kRedStride) + lane;
+            if constexpr (TAIL >= 2) {
 #pragma unroll
-            for (int j = 0; j < Tr::DD; ++j) tile[j * kRedStride] = (TAIL >= 2) ? dz.dj[j] : T(0);
-            // depth-1 letters (wave-uniform rows) and chain letters (per-lane rows) are added into the
-            // lane's own column; LDS executes a wave's operations in order.  Idle lanes need no
-            // predicate: their adjoints were loaded as zero, so every piece they produce is zero.
+                for (int j = 0; j < Tr::DD; ++j) col[j * kRedStride] = dz.dj[j];
+            } else {
+                for (int j = 0; j < d; ++j) col[j * kRedStride] = T(0);
+            }
+            // depth-1 letters and chain letters go into the lane's own column; LDS executes a wave's operations in order
 #pragma unroll
             for (int a = 0; a < K; ++a)
-                if (cx.a0 + a < Tr::DD) lds_add(&tile[(cx.a0 + a) * kRedStride], dz.da[a]);
+                if (cx.a0 + a < d) lds_add(&col[(cx.a0 + a) * kRedStride], dz.da[a]);
 #pragma unroll
-            for (int l = 0; l < M; ++l) lds_add(&tile[cx.p[l] * kRedStride], dz.dc[l]);
+            for (int l = 0; l < M; ++l) lds_add(&col[cx.p[l] * kRedStride], dz.dc[l]);
             ++cs;
             if (cs == CH || t == 0) {
                 reduce_chunk(cs);
@@ -554,17 +582,14 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
 #pragma unroll
                     for (int l = 0; l < M; ++l) lds_add(&acc[cx.p[l]], dz.dc[l]);
                 }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                wave_lds_sync();
                 for (int e = lane; e < slots * d; e += kWave) {
                     const T v = wbuf[e];
                     wbuf[e] = T(0);
                     const int64_t bb = b_first + e / d;
                     if (bb < batch) dev_add(&dzinc[(bb * L + t) * d + e % d], v);
                 }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                __builtin_amdgcn_wave_barrier();
+                wave_lds_sync();
             } else if (active) {
                 if constexpr (TAIL >= 2) {
 #pragma unroll
@@ -582,7 +607,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* row = inc + (cx.id.b * (L + 2) + L) * d;      // row of the last step
     if constexpr (ZL) {
         static_assert(WIDE, "staged increments need the wide layout");
-        T* lds_wave = lds + kWavesPerBlock * (CH * Tr::DD * kRedStride) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
+        T* lds_wave = lds + kWavesPerBlock * (red_chunk<T>(Tr::DD) * Tr::DD * kRedStride) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
         constexpr int NG = (Tr::DD + K - 1) / K;
         if constexpr (NG <= 3) {
             static_for<0, NG - 1>([&](auto gc) {
@@ -593,7 +618,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
             sweep_staged<-1, -1, Tr>(cx, row, L - 1, L, lds_wave, do_step);
         }
     } else {
-        sweep_direct<-1, Cx, typename Tr::Inc>(cx, row, L - 1, L, do_step);
+        sweep_direct<-1, false, Cx, typename Tr::Inc>(cx, row, L - 1, L, do_step);
     }
 }
 

@@ -59,9 +59,9 @@ hipError_t launch_tree_bwd(const BwdParams& p)
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
     size_t lds;
     int use_lds = 1;
-    if (g.wide) {
-        static_assert(D <= 31, "wide-layout reduction tile assumes at most 31 letters");
-        lds = size_t(kWavesPerBlock) * size_t(bwd_chunk(D > 0 ? D : 1)) * size_t(D) * kRedStride * sizeof(T);
+    const int ch = red_chunk<T>(p.d);
+    if (ch > 0) {
+        lds = size_t(kWavesPerBlock) * size_t(ch) * size_t(p.d) * kRedStride * sizeof(T);
     } else {
         lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
         if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
