@@ -404,11 +404,17 @@ __device__ __forceinline__ void wave_lds_sync()
     asm volatile("" ::: "memory");
 }
 
+// Add into an LDS word that only the calling lane touches between two wave_lds_sync() points (its own column
+// of the reduction tile) or that several lanes may hit (the shared accumulator of the wide-path fallback).
+// ds_add_f64 is fast; ds_add_f32 was measured several times slower than a plain read-add-write on gfx950, so
+// the own-column case uses the latter for float.
 template <typename T>
-__device__ __forceinline__ void lds_add(T* p, T v)
+__device__ __forceinline__ void lds_add_shared(T* p, T v)
 {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
+__device__ __forceinline__ void lds_add(double* p, double v) { lds_add_shared(p, v); }
+__device__ __forceinline__ void lds_add(float* p, float v) { *p += v; }
 template <typename T>
 __device__ __forceinline__ void dev_add(T* p, T v)
 {
@@ -574,13 +580,13 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 if (active) {
 #pragma unroll
                     for (int a = 0; a < K; ++a)
-                        if (cx.a0 + a < d) lds_add(&acc[cx.a0 + a], dz.da[a]);
+                        if (cx.a0 + a < d) lds_add_shared(&acc[cx.a0 + a], dz.da[a]);
                     if constexpr (TAIL >= 2) {
 #pragma unroll
-                        for (int j = 0; j < Tr::DD; ++j) lds_add(&acc[j], dz.dj[j]);
+                        for (int j = 0; j < Tr::DD; ++j) lds_add_shared(&acc[j], dz.dj[j]);
                     }
 #pragma unroll
-                    for (int l = 0; l < M; ++l) lds_add(&acc[cx.p[l]], dz.dc[l]);
+                    for (int l = 0; l < M; ++l) lds_add_shared(&acc[cx.p[l]], dz.dc[l]);
                 }
                 wave_lds_sync();
                 for (int e = lane; e < slots * d; e += kWave) {
