@@ -68,6 +68,43 @@ CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const dou
                                       uint64_t correction_len, uint64_t correction_batch_stride,
                                       uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
 
+/* Chen product of two signatures per batch item: out = sig1 (x) sig2, all [batch, S(+1)].
+ * Replaces: siglib/cusig/cu_sig_combine.cu:157-169 (decl siglib/cusig/cusig.h:364-365),
+ * bound by pysiglib/load_siglib.py:450-454, called from pysiglib/sig.py:113-121. */
+CUSIG_AMD_API int sig_combine_cuda_f(const float* sig1, const float* sig2, float* out, uint64_t batch_size,
+                                     uint64_t dimension, uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_combine_cuda_d(const double* sig1, const double* sig2, double* out, uint64_t batch_size,
+                                     uint64_t dimension, uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
+/* Gradients of a loss w.r.t. sig1 and sig2 given its gradient w.r.t. sig1 (x) sig2 (scalar slots get 0).
+ * Replaces: siglib/cusig/cu_sig_combine.cu:323-337 (decl siglib/cusig/cusig.h:387-388),
+ * bound by pysiglib/load_siglib.py:466-471. */
+CUSIG_AMD_API int sig_combine_backprop_cuda_f(const float* sig_combined_deriv, float* sig1_deriv, float* sig2_deriv,
+                                              const float* sig1, const float* sig2, uint64_t batch_size,
+                                              uint64_t dimension, uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_combine_backprop_cuda_d(const double* sig_combined_deriv, double* sig1_deriv, double* sig2_deriv,
+                                              const double* sig1, const double* sig2, uint64_t batch_size,
+                                              uint64_t dimension, uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
+/* Materialises the lead-lag / time augmentation: data_in [batch, length, dimension] ->
+ * data_out [batch, len_eff, d_eff].
+ * Replaces: siglib/cusig/cu_path_transforms.cu:48-127 (decl siglib/cusig/cusig.h:66-67),
+ * bound by pysiglib/load_siglib.py:420-424, called from pysiglib/transform_path.py. */
+CUSIG_AMD_API int transform_path_cuda_f(const float* data_in, float* data_out, uint64_t batch_size, uint64_t dimension,
+                                        uint64_t length, bool time_aug, bool lead_lag, float end_time) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int transform_path_cuda_d(const double* data_in, double* data_out, uint64_t batch_size, uint64_t dimension,
+                                        uint64_t length, bool time_aug, bool lead_lag, double end_time) CUSIG_AMD_NOEXCEPT;
+
+/* Adjoint of the augmentation: derivs [batch, len_eff, d_eff] -> data_out [batch, length, dimension].
+ * Replaces: siglib/cusig/cu_path_transforms.cu:129-205 (decl siglib/cusig/cusig.h:91-92),
+ * bound by pysiglib/load_siglib.py:425-429. */
+CUSIG_AMD_API int transform_path_backprop_cuda_f(const float* derivs, float* data_out, uint64_t batch_size,
+                                                 uint64_t dimension, uint64_t length, bool time_aug, bool lead_lag,
+                                                 float end_time) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int transform_path_backprop_cuda_d(const double* derivs, double* data_out, uint64_t batch_size,
+                                                 uint64_t dimension, uint64_t length, bool time_aug, bool lead_lag,
+                                                 double end_time) CUSIG_AMD_NOEXCEPT;
+
 /* Message of the last failing call made by the calling thread ("" if none).
  * Replaces: cusig_last_error_message, probed by pysiglib/load_siglib.py:108-110
  * and read by pysiglib/error_codes.py:28-42. */

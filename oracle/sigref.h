@@ -36,6 +36,25 @@ int sigref_sig_backprop_f(const float *path, float *out, const float *sig_derivs
 int sigref_sig_backprop_d(const double *path, double *out, const double *sig_derivs, const double *sig,
                           uint64_t batch, uint64_t dimension, uint64_t length, uint64_t degree,
                           int time_aug, int lead_lag, double end_time, int scalar_term, int n_jobs);
+/* Operators either side of the signature path, same argument meaning as the reference's
+ * sig_combine_{f,d}, sig_combine_backprop_{f,d}, transform_path_{f,d}, transform_path_backprop_{f,d}
+ * (siglib/cpsig/cpsig.h) without n_jobs. */
+int sigref_sig_combine_f(const float *sig1, const float *sig2, float *out, uint64_t batch, uint64_t dimension,
+                         uint64_t degree, int scalar_term);
+int sigref_sig_combine_d(const double *sig1, const double *sig2, double *out, uint64_t batch, uint64_t dimension,
+                         uint64_t degree, int scalar_term);
+int sigref_sig_combine_backprop_f(const float *dout, float *d1, float *d2, const float *sig1, const float *sig2,
+                                  uint64_t batch, uint64_t dimension, uint64_t degree, int scalar_term);
+int sigref_sig_combine_backprop_d(const double *dout, double *d1, double *d2, const double *sig1, const double *sig2,
+                                  uint64_t batch, uint64_t dimension, uint64_t degree, int scalar_term);
+int sigref_transform_path_f(const float *in, float *out, uint64_t batch, uint64_t dimension, uint64_t length,
+                            int time_aug, int lead_lag, float end_time);
+int sigref_transform_path_d(const double *in, double *out, uint64_t batch, uint64_t dimension, uint64_t length,
+                            int time_aug, int lead_lag, double end_time);
+int sigref_transform_path_backprop_f(const float *derivs, float *out, uint64_t batch, uint64_t dimension,
+                                     uint64_t length, int time_aug, int lead_lag);
+int sigref_transform_path_backprop_d(const double *derivs, double *out, uint64_t batch, uint64_t dimension,
+                                     uint64_t length, int time_aug, int lead_lag);
 #ifdef __cplusplus
 }
 #endif

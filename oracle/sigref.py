@@ -36,6 +36,18 @@ def _load():
         g = getattr(lib, "sigref_sig_backprop_" + suf)
         g.restype = i32
         g.argtypes = (ptr, ptr, ptr, ptr, u64, u64, u64, u64, i32, i32, real, i32, i32)
+        f = getattr(lib, "sigref_sig_combine_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, u64, u64, u64, i32)
+        f = getattr(lib, "sigref_sig_combine_backprop_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, ptr, ptr, u64, u64, u64, i32)
+        f = getattr(lib, "sigref_transform_path_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, u64, u64, u64, i32, i32, real)
+        f = getattr(lib, "sigref_transform_path_backprop_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, u64, u64, u64, i32, i32)
     return lib
 
 
@@ -110,4 +122,71 @@ def sig_backprop(path, sig, sig_derivs, degree, time_aug=False, lead_lag=False, 
         float(end_time), int(scalar_term), n_jobs)
     if rc:
         raise RuntimeError("sigref_sig_backprop returned %d" % rc)
+    return out[0] if single else out
+
+
+def _rows(arr, dtype):
+    a = np.ascontiguousarray(arr, dtype=dtype)
+    return a.reshape(-1, a.shape[-1])
+
+
+def sig_combine(sig1, sig2, dimension, degree):
+    """Oracle Chen product; scalar_term is inferred from the width."""
+    sig1 = np.asarray(sig1)
+    suf, real = _suffix(sig1.dtype)
+    a, b = _rows(sig1, sig1.dtype), _rows(sig2, sig1.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    out = np.empty_like(a)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_combine_" + suf)(a.ctypes.data_as(ptr), b.ctypes.data_as(ptr), out.ctypes.data_as(ptr),
+                                                   a.shape[0], dimension, degree, int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_combine returned %d" % rc)
+    return out.reshape(sig1.shape)
+
+
+def sig_combine_backprop(derivs, sig1, sig2, dimension, degree):
+    sig1 = np.asarray(sig1)
+    suf, real = _suffix(sig1.dtype)
+    a, b, g = _rows(sig1, sig1.dtype), _rows(sig2, sig1.dtype), _rows(derivs, sig1.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    d1, d2 = np.empty_like(a), np.empty_like(a)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_combine_backprop_" + suf)(
+        g.ctypes.data_as(ptr), d1.ctypes.data_as(ptr), d2.ctypes.data_as(ptr), a.ctypes.data_as(ptr),
+        b.ctypes.data_as(ptr), a.shape[0], dimension, degree, int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_combine_backprop returned %d" % rc)
+    return d1.reshape(sig1.shape), d2.reshape(sig1.shape)
+
+
+def transform_path(path, time_aug=False, lead_lag=False, end_time=1.0):
+    path = np.ascontiguousarray(path)
+    single = path.ndim == 2
+    if single:
+        path = path[None]
+    batch, length, dim = path.shape
+    suf, real = _suffix(path.dtype)
+    out = np.empty((batch, 2 * length - 1 if lead_lag else length, _aug_dim(dim, time_aug, lead_lag)), dtype=path.dtype)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_transform_path_" + suf)(path.ctypes.data_as(ptr), out.ctypes.data_as(ptr), batch, dim,
+                                                      length, int(time_aug), int(lead_lag), float(end_time))
+    if rc:
+        raise RuntimeError("sigref_transform_path returned %d" % rc)
+    return out[0] if single else out
+
+
+def transform_path_backprop(derivs, dimension, length, time_aug=False, lead_lag=False):
+    derivs = np.ascontiguousarray(derivs)
+    single = derivs.ndim == 2
+    if single:
+        derivs = derivs[None]
+    suf, real = _suffix(derivs.dtype)
+    out = np.empty((derivs.shape[0], length, dimension), dtype=derivs.dtype)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_transform_path_backprop_" + suf)(derivs.ctypes.data_as(ptr), out.ctypes.data_as(ptr),
+                                                               derivs.shape[0], dimension, length, int(time_aug),
+                                                               int(lead_lag))
+    if rc:
+        raise RuntimeError("sigref_transform_path_backprop returned %d" % rc)
     return out[0] if single else out

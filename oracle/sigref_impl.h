@@ -384,6 +384,132 @@ int FN(sigref_sig_backprop)(const REAL *path, REAL *out, const REAL *sig_derivs,
     return J.status;
 }
 
+
+/* ---- operators either side of the signature path -------------------------- */
+
+/* siglib/cpsig/cp_sig_combine.h:126-176 uncombine_sig_deriv (full layout):
+ * given dF/d(a (x) b) in `da` (overwritten with dF/da) computes dF/db into `db`. */
+static void FN(chen_pullback)(const REAL *a, const REAL *b, REAL *da, REAL *db, uint64_t degree, const uint64_t *lvl)
+{
+    const uint64_t full = lvl[degree + 1];
+    memcpy(db, da, full * sizeof(REAL));
+    for (uint64_t t = degree; t > 0; --t) {
+        for (uint64_t left = t - 1; left > 0; --left) {
+            const uint64_t right = t - left;
+            const uint64_t nl = lvl[left + 1] - lvl[left], nr = lvl[right + 1] - lvl[right];
+            const REAL *res = da + lvl[t];
+            REAL *dbr = db + lvl[right];
+            for (uint64_t i = 0; i < nl; ++i)
+                for (uint64_t j = 0; j < nr; ++j) dbr[j] += res[i * nr + j] * a[lvl[left] + i];
+        }
+    }
+    for (uint64_t left = 1; left < degree; ++left) {
+        for (uint64_t t = left + 1; t <= degree; ++t) {
+            const uint64_t right = t - left;
+            const uint64_t nl = lvl[left + 1] - lvl[left], nr = lvl[right + 1] - lvl[right];
+            const REAL *res = da + lvl[t];
+            for (uint64_t i = 0; i < nl; ++i) {
+                REAL acc = (REAL)0;
+                for (uint64_t j = 0; j < nr; ++j) acc += res[i * nr + j] * b[lvl[right] + j];
+                da[lvl[left] + i] += acc;
+            }
+        }
+    }
+}
+
+/* siglib/cpsig/cp_sig_combine.h:266-316 sig_combine_ / batch_sig_combine_ */
+int FN(sigref_sig_combine)(const REAL *sig1, const REAL *sig2, REAL *out, uint64_t batch, uint64_t d,
+                           uint64_t degree, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *a = (REAL *)malloc(2 * full * sizeof(REAL));
+    if (!lvl || !a) { free(lvl); free(a); return 1; }
+    REAL *b = a + full;
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t off = scalar_term ? 0 : 1;
+    for (uint64_t i = 0; i < batch; ++i) {
+        a[0] = b[0] = (REAL)1;
+        memcpy(a + off, sig1 + i * stride, stride * sizeof(REAL));
+        memcpy(b + off, sig2 + i * stride, stride * sizeof(REAL));
+        FN(chen_inplace)(a, b, degree, lvl);
+        memcpy(out + i * stride, a + off, stride * sizeof(REAL));
+    }
+    free(lvl); free(a);
+    return 0;
+}
+
+/* siglib/cpsig/cp_sig_combine.h:318-400 sig_combine_backprop_ / batch_sig_combine_backprop_:
+ * scalar slots of both gradients are 0. */
+int FN(sigref_sig_combine_backprop)(const REAL *dout, REAL *d1, REAL *d2, const REAL *sig1, const REAL *sig2,
+                                    uint64_t batch, uint64_t d, uint64_t degree, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *a = (REAL *)malloc(4 * full * sizeof(REAL));
+    if (!lvl || !a) { free(lvl); free(a); return 1; }
+    REAL *b = a + full, *da = a + 2 * full, *db = a + 3 * full;
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t off = scalar_term ? 0 : 1;
+    for (uint64_t i = 0; i < batch; ++i) {
+        a[0] = b[0] = (REAL)1; da[0] = (REAL)0;
+        memcpy(a + off, sig1 + i * stride, stride * sizeof(REAL));
+        memcpy(b + off, sig2 + i * stride, stride * sizeof(REAL));
+        memcpy(da + off, dout + i * stride, stride * sizeof(REAL));
+        FN(chen_pullback)(a, b, da, db, degree, lvl);
+        da[0] = db[0] = (REAL)0;
+        memcpy(d1 + i * stride, da + off, stride * sizeof(REAL));
+        memcpy(d2 + i * stride, db + off, stride * sizeof(REAL));
+    }
+    free(lvl); free(a);
+    return 0;
+}
+
+/* siglib/cpsig/cp_path_transforms.h:36-142 transform_path_ (materialised augmentation) */
+int FN(sigref_transform_path)(const REAL *in, REAL *out, uint64_t batch, uint64_t d, uint64_t len,
+                              int time_aug, int lead_lag, REAL end_time)
+{
+    if (d == 0) return 2;
+    FN(vpath) p;
+    for (uint64_t b = 0; b < batch; ++b) {
+        FN(vpath_init)(&p, in + b * d * len, d, len, time_aug, lead_lag, end_time);
+        REAL *o = out + b * p.d * p.len;
+        const REAL scale = p.len > 1 ? end_time / (REAL)(p.len - 1) : (REAL)0;
+        for (uint64_t i = 0; i < p.len; ++i)
+            for (uint64_t c = 0; c < p.d; ++c) o[i * p.d + c] = FN(vpath_at)(&p, i, c, (REAL)i * scale);
+    }
+    return 0;
+}
+
+/* siglib/cpsig/cp_path_transforms.h:182-243 transform_path_backprop_ */
+int FN(sigref_transform_path_backprop)(const REAL *derivs, REAL *out, uint64_t batch, uint64_t d, uint64_t len,
+                                       int time_aug, int lead_lag)
+{
+    if (d == 0) return 2;
+    const uint64_t td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
+    const uint64_t tl = lead_lag ? 2 * len - 1 : len;
+    for (uint64_t b = 0; b < batch; ++b) {
+        const REAL *g = derivs + b * td * tl;
+        REAL *o = out + b * d * len;
+        for (uint64_t k = 0; k < len; ++k)
+            for (uint64_t j = 0; j < d; ++j) {
+                if (!lead_lag) { o[k * d + j] = g[k * td + j]; continue; }
+                REAL v = g[(2 * k) * td + j];
+                if (k + 1 < len) v += g[(2 * k + 1) * td + j];
+                v += g[(2 * k) * td + d + j];
+                if (k >= 1) v += g[(2 * k - 1) * td + d + j];
+                o[k * d + j] = v;
+            }
+    }
+    return 0;
+}
+
 #undef FN
 #undef CAT
 #undef CAT_

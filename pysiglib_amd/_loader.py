@@ -59,6 +59,19 @@ CUSIG_SIG_BACKPROP = _table("sig_backprop_cuda", lambda r: (
     c_bool, POINTER(r), c_uint64, c_uint64, c_uint64))
 
 
+CUSIG_SIG_COMBINE = _table("sig_combine_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool))
+
+CUSIG_SIG_COMBINE_BACKPROP = _table("sig_combine_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool))
+
+CUSIG_TRANSFORM_PATH = _table("transform_path_cuda", lambda r: (
+    POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool, r))
+
+CUSIG_TRANSFORM_PATH_BACKPROP = _table("transform_path_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool, r))
+
+
 def last_error_message():
     msg = CUSIG.cusig_last_error_message()
     return msg.decode("utf-8", errors="replace") if msg else ""

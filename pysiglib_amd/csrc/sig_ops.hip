@@ -1,0 +1,276 @@
+// Operators either side of the signature sweep, behind the reference's entry points:
+//   sig_combine_cuda_{f,d}, sig_combine_backprop_cuda_{f,d}   (siglib/cusig/cu_sig_combine.cu:157-337)
+//   transform_path_cuda_{f,d}, transform_path_backprop_cuda_{f,d} (siglib/cusig/cu_path_transforms.cu:48-205)
+// The Chen product itself is the kernel the time-segmented forward sweep folds its pieces with.
+#include <hip/hip_runtime.h>
+
+#include "../../include/cusig_amd.h"
+#include "sig_host.h"
+#include "sig_kernels.h"
+
+namespace sigamd {
+
+// Adjoint of C = A (x) B (siglib/cpsig/cp_sig_combine.h:126-176).  One thread per coefficient r = (level t, word w):
+//   dA_t[w] = dC_t[w] + sum_{m=1..N-t} sum_{v in d^m} dC_{t+m}[w v] * B_m[v]        (contiguous block of dC)
+//   dB_t[w] = dC_t[w] + sum_{k=1..N-t} sum_{u in d^k} dC_{t+k}[u w] * A_k[u]        (stride d^t in dC)
+// Scalar slots of both gradients are zero.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
+    const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, const T* __restrict__ A,
+    const T* __restrict__ B, int64_t batch, int d, int degree, int64_t sig_len, int64_t stride, int off)
+{
+    const int64_t total = batch * sig_len;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / sig_len;
+        const int64_t r = e % sig_len;
+        int t = 1;
+        int64_t lvl = d, lo = 0;
+        while (r >= lo + lvl) { lo += lvl; lvl *= d; ++t; }
+        const int64_t w = r - lo;
+        const T* g = dC + b * stride + off;
+        const T* a = A + b * stride + off;
+        const T* bb = B + b * stride + off;
+        T ga = g[lo + w], gb = ga;
+        int64_t up_lo = lo + lvl;      // start of level t + m in dC
+        int64_t up_sz = lvl * d;       // its size d^(t+m)
+        int64_t lo_m = 0, sz_m = d;    // level m of A / B
+        for (int m = 1; t + m <= degree; ++m) {
+            const T* blockp = g + up_lo + w * sz_m;        // words w v, v in d^m
+            T s0 = T(0), s1 = T(0);
+            int64_t v = 0;
+            for (; v + 2 <= sz_m; v += 2) {
+                s0 = fmadd(blockp[v], bb[lo_m + v], s0);
+                s1 = fmadd(blockp[v + 1], bb[lo_m + v + 1], s1);
+            }
+            for (; v < sz_m; ++v) s0 = fmadd(blockp[v], bb[lo_m + v], s0);
+            ga += s0 + s1;
+            const T* strided = g + up_lo + w;               // words u w, u in d^m: index u * d^t + w
+            T q0 = T(0), q1 = T(0);
+            int64_t u = 0;
+            for (; u + 2 <= sz_m; u += 2) {
+                q0 = fmadd(strided[u * lvl], a[lo_m + u], q0);
+                q1 = fmadd(strided[(u + 1) * lvl], a[lo_m + u + 1], q1);
+            }
+            for (; u < sz_m; ++u) q0 = fmadd(strided[u * lvl], a[lo_m + u], q0);
+            gb += q0 + q1;
+            up_lo += up_sz;
+            up_sz *= d;
+            lo_m += sz_m;
+            sz_m *= d;
+        }
+        dA[b * stride + off + r] = ga;
+        dB[b * stride + off + r] = gb;
+        if (off && r == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
+    }
+}
+
+// Materialised lead-lag / time augmentation: point i of the lead-lag path has lag = x[i/2] and
+// lead = x[i/2 + (i odd)]; time is the last channel, i * end_time / (len_eff - 1)
+// (siglib/cpsig/cp_path_transforms.h:36-142).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transform_path_kernel(
+    const T* __restrict__ in, T* __restrict__ out, int64_t batch, int64_t len, int d, int time_aug, int lead_lag, T scale)
+{
+    const int td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
+    const int64_t tl = lead_lag ? 2 * len - 1 : len;
+    const int64_t total = batch * tl * td;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int c = int(e % td);
+        const int64_t i = (e / td) % tl;
+        const int64_t b = e / (int64_t(td) * tl);
+        const T* x = in + b * len * d;
+        T v;
+        if (time_aug && c == td - 1) v = T(i) * scale;
+        else if (!lead_lag) v = x[i * d + c];
+        else if (c < d) v = x[(i >> 1) * d + c];
+        else v = x[((i >> 1) + (i & 1)) * d + (c - d)];
+        out[e] = v;
+    }
+}
+
+// Adjoint of the augmentation: a raw point collects the gradient of every transformed point that copies it;
+// the time channel has no raw counterpart (siglib/cpsig/cp_path_transforms.h:182-243).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transform_path_bwd_kernel(
+    const T* __restrict__ derivs, T* __restrict__ out, int64_t batch, int64_t len, int d, int time_aug, int lead_lag)
+{
+    const int td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
+    const int64_t tl = lead_lag ? 2 * len - 1 : len;
+    const int64_t total = batch * len * d;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int j = int(e % d);
+        const int64_t k = (e / d) % len;
+        const int64_t b = e / (int64_t(d) * len);
+        const T* g = derivs + b * tl * td;
+        T v;
+        if (!lead_lag) {
+            v = g[k * td + j];
+        } else {
+            v = g[(2 * k) * td + j] + g[(2 * k) * td + d + j];
+            if (k + 1 < len) v += g[(2 * k + 1) * td + j];
+            if (k >= 1) v += g[(2 * k - 1) * td + d + j];
+        }
+        out[e] = v;
+    }
+}
+
+struct SigShape {
+    uint64_t n_coef, stride;
+    int off;
+};
+
+static SigShape sig_shape(uint64_t dimension, uint64_t degree, bool scalar_term, const char* who)
+{
+    if (dimension == 0) throw std::invalid_argument(std::string(who) + " received dimension 0");
+    if (dimension > 0x3fffffff || degree > 0x7fffffff) throw std::invalid_argument(std::string(who) + ": shape out of range");
+    const uint64_t full = sig_length_u64(dimension, degree);
+    if (full == 0) throw std::overflow_error("signature length overflows 64 bits");
+    SigShape s;
+    s.n_coef = full - 1;
+    s.stride = scalar_term ? full : full - 1;
+    s.off = scalar_term ? 1 : 0;
+    return s;
+}
+
+template <typename T>
+static void sig_combine_impl(const T* sig1, const T* sig2, T* out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                             bool scalar_term)
+{
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_combine_cuda");
+    if (batch == 0) return;
+    checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    if (s.n_coef == 0) {        // degree 0: only the scalar slot exists
+        if (scalar_term)
+            hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
+                               int64_t(1), 1);
+    } else {
+        hipLaunchKernelGGL((sig_combine_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, sig1, sig2,
+                           out, int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride),
+                           int64_t(s.stride), int64_t(s.stride), s.off, s.off, s.off);
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+template <typename T>
+static void sig_combine_backprop_impl(const T* derivs, T* d1, T* d2, const T* sig1, const T* sig2, uint64_t batch,
+                                      uint64_t dimension, uint64_t degree, bool scalar_term)
+{
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_combine_backprop_cuda");
+    if (batch == 0) return;
+    checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    if (s.n_coef == 0) {
+        if (scalar_term) {
+            hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, d1, int64_t(batch));
+            hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, d2, int64_t(batch));
+        }
+    } else {
+        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, derivs,
+                           d1, d2, sig1, sig2, int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef),
+                           int64_t(s.stride), s.off);
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+static void path_shape_check(uint64_t dimension, uint64_t length, const char* who)
+{
+    if (dimension == 0) throw std::invalid_argument(std::string(who) + " received path of dimension 0");
+    if (dimension > 0x3fffffff || length > (uint64_t(1) << 40)) throw std::invalid_argument(std::string(who) + ": shape out of range");
+}
+
+template <typename T>
+static void transform_path_impl(const T* in, T* out, uint64_t batch, uint64_t dimension, uint64_t length, bool time_aug,
+                                bool lead_lag, T end_time)
+{
+    path_shape_check(dimension, length, "transform_path_cuda");
+    if (batch == 0 || length == 0) return;
+    const uint64_t td = (lead_lag ? 2 * dimension : dimension) + (time_aug ? 1 : 0);
+    const uint64_t tl = lead_lag ? 2 * length - 1 : length;
+    const uint64_t total = checked_mul(checked_mul(batch, tl, "transformed path"), td, "transformed path");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    const T scale = tl > 1 ? end_time / T(tl - 1) : T(0);
+    hipLaunchKernelGGL((transform_path_kernel<T>), dim3(grid_for(total)), dim3(kBlock), 0, stream, in, out, int64_t(batch),
+                       int64_t(length), int(dimension), int(time_aug), int(lead_lag), scale);
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+template <typename T>
+static void transform_path_backprop_impl(const T* derivs, T* out, uint64_t batch, uint64_t dimension, uint64_t length,
+                                         bool time_aug, bool lead_lag)
+{
+    path_shape_check(dimension, length, "transform_path_backprop_cuda");
+    if (batch == 0 || length == 0) return;
+    const uint64_t total = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    hipLaunchKernelGGL((transform_path_bwd_kernel<T>), dim3(grid_for(total)), dim3(kBlock), 0, stream, derivs, out,
+                       int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+}  // namespace sigamd
+
+using namespace sigamd;
+
+extern "C" {
+
+CUSIG_AMD_API int sig_combine_cuda_f(const float* sig1, const float* sig2, float* out, uint64_t batch_size,
+                                     uint64_t dimension, uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] { sig_combine_impl<float>(sig1, sig2, out, batch_size, dimension, degree, scalar_term); });
+}
+CUSIG_AMD_API int sig_combine_cuda_d(const double* sig1, const double* sig2, double* out, uint64_t batch_size,
+                                     uint64_t dimension, uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] { sig_combine_impl<double>(sig1, sig2, out, batch_size, dimension, degree, scalar_term); });
+}
+CUSIG_AMD_API int sig_combine_backprop_cuda_f(const float* sig_combined_deriv, float* sig1_deriv, float* sig2_deriv,
+                                              const float* sig1, const float* sig2, uint64_t batch_size,
+                                              uint64_t dimension, uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] {
+        sig_combine_backprop_impl<float>(sig_combined_deriv, sig1_deriv, sig2_deriv, sig1, sig2, batch_size, dimension,
+                                         degree, scalar_term);
+    });
+}
+CUSIG_AMD_API int sig_combine_backprop_cuda_d(const double* sig_combined_deriv, double* sig1_deriv, double* sig2_deriv,
+                                              const double* sig1, const double* sig2, uint64_t batch_size,
+                                              uint64_t dimension, uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] {
+        sig_combine_backprop_impl<double>(sig_combined_deriv, sig1_deriv, sig2_deriv, sig1, sig2, batch_size, dimension,
+                                          degree, scalar_term);
+    });
+}
+CUSIG_AMD_API int transform_path_cuda_f(const float* data_in, float* data_out, uint64_t batch_size, uint64_t dimension,
+                                        uint64_t length, bool time_aug, bool lead_lag, float end_time) noexcept
+{
+    return guarded([&] { transform_path_impl<float>(data_in, data_out, batch_size, dimension, length, time_aug, lead_lag, end_time); });
+}
+CUSIG_AMD_API int transform_path_cuda_d(const double* data_in, double* data_out, uint64_t batch_size, uint64_t dimension,
+                                        uint64_t length, bool time_aug, bool lead_lag, double end_time) noexcept
+{
+    return guarded([&] { transform_path_impl<double>(data_in, data_out, batch_size, dimension, length, time_aug, lead_lag, end_time); });
+}
+CUSIG_AMD_API int transform_path_backprop_cuda_f(const float* derivs, float* data_out, uint64_t batch_size,
+                                                 uint64_t dimension, uint64_t length, bool time_aug, bool lead_lag,
+                                                 float) noexcept
+{
+    return guarded([&] { transform_path_backprop_impl<float>(derivs, data_out, batch_size, dimension, length, time_aug, lead_lag); });
+}
+CUSIG_AMD_API int transform_path_backprop_cuda_d(const double* derivs, double* data_out, uint64_t batch_size,
+                                                 uint64_t dimension, uint64_t length, bool time_aug, bool lead_lag,
+                                                 double) noexcept
+{
+    return guarded([&] { transform_path_backprop_impl<double>(derivs, data_out, batch_size, dimension, length, time_aug, lead_lag); });
+}
+
+}  // extern "C"

@@ -24,16 +24,12 @@ int not_implemented(const char* name) noexcept
 #define STUB_ONE(name) \
     extern "C" __attribute__((visibility("default"))) int name(...) noexcept { return not_implemented(#name); }
 
-STUB_PAIR(transform_path_cuda)
-STUB_PAIR(transform_path_backprop_cuda)
 STUB_PAIR(log_sig_combine_cuda)
 STUB_PAIR(log_sig_from_path_cuda)
 STUB_PAIR(log_sig_from_path_backprop_cuda)
 STUB_PAIR(log_sig_combine_backprop_cuda)
-STUB_PAIR(sig_combine_cuda)
 STUB_PAIR(sig_join_cuda)
 STUB_PAIR(sig_join_backprop_cuda)
-STUB_PAIR(sig_combine_backprop_cuda)
 STUB_PAIR(sig_coef_cuda)
 STUB_PAIR(sig_coef_backprop_cuda)
 STUB_PAIR(sig_to_log_sig_cuda)

@@ -30,3 +30,47 @@ def sig(path, degree, *, time_aug=False, lead_lag=False, end_time=1., horner=Tru
 
 
 signature = sig
+
+
+class SigCombine(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, sig1, sig2, dimension, degree, time_aug, lead_lag):
+        from .ops import sig_combine as _combine
+        out = _combine(sig1, sig2, dimension, degree, time_aug=time_aug, lead_lag=lead_lag)
+        ctx.save_for_backward(sig1, sig2)
+        ctx.args = (dimension, degree, time_aug, lead_lag)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .ops import sig_combine_backprop as _combine_backprop
+        sig1, sig2 = ctx.saved_tensors
+        dimension, degree, time_aug, lead_lag = ctx.args
+        d1, d2 = _combine_backprop(grad_output, sig1, sig2, dimension, degree, time_aug=time_aug, lead_lag=lead_lag)
+        return d1, d2, None, None, None, None
+
+
+def sig_combine(sig1, sig2, dimension, degree, *, time_aug=False, lead_lag=False, n_jobs=1):
+    """Differentiable ``sig_combine``."""
+    return SigCombine.apply(sig1, sig2, dimension, degree, time_aug, lead_lag)
+
+
+class TransformPath(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, path, time_aug, lead_lag, end_time):
+        from .ops import transform_path as _transform
+        ctx.args = (time_aug, lead_lag, end_time)
+        return _transform(path, time_aug=time_aug, lead_lag=lead_lag, end_time=end_time)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .ops import transform_path_backprop as _transform_backprop
+        time_aug, lead_lag, end_time = ctx.args
+        return _transform_backprop(grad_output, time_aug=time_aug, lead_lag=lead_lag, end_time=end_time), None, None, None
+
+
+def transform_path(path, *, time_aug=False, lead_lag=False, end_time=1., n_jobs=1):
+    """Differentiable ``transform_path``."""
+    if (not time_aug) and (not lead_lag):
+        return path
+    return TransformPath.apply(path, time_aug, lead_lag, end_time)

@@ -1,0 +1,243 @@
+"""Parity of sig_combine / transform_path and their backward passes (HIP, through the C ABI) with the CPU oracle,
+the reference's hand-computed vectors and its golden float32 gradients.
+
+Tolerances: float64 1e-10, float32 1e-4 (relative to the per-level / per-row max norm); exact for the pure copies
+of transform_path; golden float32 gradients at the reference's 1e-5 (tests/test_sig_combine_backprop.py:24).
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests import _ops_kats as K
+from tests._mathref import level_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float64: 1e-10, np.float32: 1e-4}
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def P():
+    import pysiglib_amd
+    assert torch.cuda.is_available()
+    return pysiglib_amd
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import sigref
+    return sigref
+
+
+def dev(a, dtype=None):
+    return torch.tensor(np.ascontiguousarray(a, dtype=dtype), device=DEV)
+
+
+def row_rel_err(got, ref):
+    got = got.reshape(-1, ref.shape[-1]).astype(np.float64)
+    ref = ref.reshape(-1, ref.shape[-1]).astype(np.float64)
+    den = np.maximum(np.abs(ref).max(axis=1), np.finfo(np.float64).tiny)
+    return float((np.abs(got - ref).max(axis=1) / den).max())
+
+
+def test_combine_kats(P):
+    for s1, s2, want, d, deg in K.COMBINE:
+        got = P.sig_combine(dev(s1), dev(s2), d, deg)
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=0, atol=1e-14)
+        got = P.sig_combine(dev(s1[1:]), dev(s2[1:]), d, deg)
+        np.testing.assert_allclose(got.cpu().numpy(), want[1:], rtol=0, atol=1e-14)
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 5, 7), (5, 4, 33), (3, 1, 4), (1, 6, 3), (7, 3, 130), (10, 5, 32),
+                                         (37, 2, 5), (2, 14, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_combine_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+    rng = np.random.default_rng(100 * d + deg)
+    n = oracle.sig_length(d, deg) - 1
+    scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
+    a = (rng.standard_normal((batch, n)) * scale).astype(dtype)
+    b = (rng.standard_normal((batch, n)) * scale).astype(dtype)
+    if scalar_term:
+        one = np.ones((batch, 1), dtype=dtype)
+        a, b = np.hstack([one, a]), np.hstack([one, b])
+    want = oracle.sig_combine(a, b, d, deg)
+    got = P.sig_combine(dev(a), dev(b), d, deg).cpu().numpy()
+    assert got.shape == want.shape and got.dtype == dtype
+    off = 1 if scalar_term else 0
+    if scalar_term:
+        assert np.all(got[:, 0] == 1)
+    assert np.max(level_rel_err(got[:, off:], want[:, off:], d, deg)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+def test_combine_chen_identity(P, deg):
+    # the reference's own test of sig_combine (tests/test_sig_combine.py:27-54)
+    rng = np.random.default_rng(42 + deg)
+    x1 = rng.uniform(size=(32, 100, 5))
+    x2 = rng.uniform(size=(32, 100, 5))
+    whole = P.sig(dev(np.concatenate([x1, x2], axis=1)), deg)
+    s1 = P.sig(dev(x1), deg)
+    s2 = P.sig(dev(np.concatenate([x1[:, -1:], x2], axis=1)), deg)
+    got = P.sig_combine(s1, s2, 5, deg)
+    assert got.device.type == "cuda"
+    np.testing.assert_allclose(got.cpu().numpy(), whole.cpu().numpy(), rtol=0, atol=1e-10)
+
+
+def test_combine_batch_shapes_views_and_errors(P, oracle):
+    d, deg = 10, 3
+    n = P.sig_length(d, deg)
+    col = torch.rand((32, 1), dtype=torch.float64, device=DEV)
+    view = col.expand(-1, n)                      # stride-0 view, as in the reference's non-contiguous test
+    np.testing.assert_array_equal(P.sig_combine(view, view, d, deg).cpu().numpy(),
+                                  P.sig_combine(view.clone(), view.clone(), d, deg).cpu().numpy())
+    a = torch.rand((2, 3, n), dtype=torch.float64, device=DEV)
+    b = torch.rand((2, 3, n), dtype=torch.float64, device=DEV)
+    got = P.sig_combine(a, b, d, deg)
+    assert got.shape == (2, 3, n)
+    np.testing.assert_allclose(got.cpu().numpy(), oracle.sig_combine(a.cpu().numpy(), b.cpu().numpy(), d, deg),
+                               rtol=1e-12, atol=1e-12)
+    assert P.sig_combine(a[0, 0], b[0, 0], d, deg).shape == (n,)
+    empty = torch.empty((0, n), dtype=torch.float64, device=DEV)
+    assert P.sig_combine(empty, empty, d, deg).shape == (0, n)
+    with pytest.raises(ValueError):
+        P.sig_combine(a, b[..., :-1], d, deg)
+    with pytest.raises(ValueError):
+        P.sig_combine(a, b[0], d, deg)
+    with pytest.raises(ValueError):
+        P.sig_combine(a, b.float(), d, deg)
+    with pytest.raises(RuntimeError):
+        P.sig_combine(a.cpu(), b.cpu(), d, deg)
+    with pytest.raises(TypeError):
+        P.sig_combine(a, b, 10.0, deg)
+
+
+def test_combine_backprop_kats(P):
+    for g, s1, s2, w1, w2, d, deg in K.COMBINE_BACKPROP:
+        d1, d2 = P.sig_combine_backprop(dev(g), dev(s1), dev(s2), d, deg)
+        np.testing.assert_allclose(d1.cpu().numpy(), w1, rtol=0, atol=1e-14)
+        np.testing.assert_allclose(d2.cpu().numpy(), w2, rtol=0, atol=1e-14)
+    g, s1, s2, w1, w2 = (np.array([k[i] for k in K.COMBINE_BACKPROP]) for i in range(5))
+    d1, d2 = P.sig_combine_backprop(dev(g), dev(s1), dev(s2), 2, 2)
+    np.testing.assert_allclose(d1.cpu().numpy(), w1, rtol=0, atol=1e-14)
+    np.testing.assert_allclose(d2.cpu().numpy(), w2, rtol=0, atol=1e-14)
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_combine_backprop_golden(P, fixtures, deg, dtype):
+    s1, s2, g = (dev(fixtures["sig_comb_bp_%s__d%d" % (k, deg)], dtype) for k in ("sig1", "sig2", "derivs"))
+    d1, d2 = P.sig_combine_backprop(g, s1, s2, 3, deg)
+    atol = 1e-5 if dtype == np.float64 else 1e-4
+    np.testing.assert_allclose(d1.cpu().numpy()[:, 1:], fixtures["sig_comb_bp_d1__d%d" % deg], rtol=0, atol=atol)
+    np.testing.assert_allclose(d2.cpu().numpy()[:, 1:], fixtures["sig_comb_bp_d2__d%d" % deg], rtol=0, atol=atol)
+    assert torch.all(d1[:, 0] == 0) and torch.all(d2[:, 0] == 0)
+    one1, one2 = P.sig_combine_backprop(g[0], s1[0], s2[0], 3, deg)
+    np.testing.assert_array_equal(one1.cpu().numpy(), d1[0].cpu().numpy())
+    np.testing.assert_array_equal(one2.cpu().numpy(), d2[0].cpu().numpy())
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 5, 7), (5, 4, 33), (3, 1, 4), (1, 6, 3), (7, 3, 130), (10, 5, 32),
+                                         (37, 2, 5), (2, 14, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_combine_backprop_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+    rng = np.random.default_rng(7 * d + deg)
+    n = oracle.sig_length(d, deg) - (0 if scalar_term else 1)
+    a, b, g = (rng.standard_normal((batch, n)).astype(dtype) for _ in range(3))
+    if scalar_term:
+        a[:, 0] = 1
+        b[:, 0] = 1
+    w1, w2 = oracle.sig_combine_backprop(g, a, b, d, deg)
+    d1, d2 = P.sig_combine_backprop(dev(g), dev(a), dev(b), d, deg)
+    assert d1.shape == w1.shape and d2.shape == w2.shape
+    assert row_rel_err(d1.cpu().numpy(), w1) < TOL[dtype]
+    assert row_rel_err(d2.cpu().numpy(), w2) < TOL[dtype]
+
+
+def test_combine_autograd(P):
+    d, deg = 3, 4
+    n = P.sig_length(d, deg)
+    a = torch.rand((5, n), dtype=torch.float64, device=DEV, requires_grad=True)
+    b = torch.rand((5, n), dtype=torch.float64, device=DEV, requires_grad=True)
+    w = torch.rand((5, n), dtype=torch.float64, device=DEV)
+    (P.torch_api.sig_combine(a, b, d, deg) * w).sum().backward()
+    d1, d2 = P.sig_combine_backprop(w, a.detach(), b.detach(), d, deg)
+    np.testing.assert_array_equal(a.grad.cpu().numpy(), d1.cpu().numpy())
+    np.testing.assert_array_equal(b.grad.cpu().numpy(), d2.cpu().numpy())
+    # directional derivative: <w, C(a + h u, b) - C(a - h u, b)> / 2h == <dA, u>  (the product is bilinear: exact up to rounding)
+    u = torch.rand_like(w)
+    h = 1e-3
+    num = ((P.sig_combine(a.detach() + h * u, b.detach(), d, deg) - P.sig_combine(a.detach() - h * u, b.detach(), d, deg))
+           * w).sum() / (2 * h)
+    assert abs(float(num) - float((d1 * u).sum())) < 1e-8 * max(1.0, abs(float(num)))
+
+
+def test_transform_kats(P):
+    for path, kw, want in K.TRANSFORM:
+        got = P.transform_path(dev(path), **kw)
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=0, atol=1e-15)
+    for g, kw, want in K.TRANSFORM_BACKPROP:
+        got = P.transform_path_backprop(dev(g), **kw)
+        assert got.shape == want.shape
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=0, atol=1e-14)
+
+
+@pytest.mark.parametrize("kw", [dict(time_aug=True), dict(lead_lag=True), dict(time_aug=True, lead_lag=True),
+                                dict(time_aug=True, end_time=2.5), dict(time_aug=True, lead_lag=True, end_time=.3)])
+@pytest.mark.parametrize("shape", [(3, 2, 1), (2, 9, 4), (10, 100, 5), (1, 3, 70), (300, 33, 3)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_transform_vs_oracle(P, oracle, kw, shape, dtype):
+    rng = np.random.default_rng(shape[1])
+    x = rng.uniform(size=shape).astype(dtype)
+    want = oracle.transform_path(x, **kw)
+    got = P.transform_path(dev(x), **kw).cpu().numpy()
+    assert got.shape == want.shape and got.dtype == dtype
+    nt = -1 if kw.get("time_aug") else None
+    np.testing.assert_array_equal(got[..., :nt], want[..., :nt])                 # copied channels: bit-exact
+    if nt:
+        np.testing.assert_allclose(got[..., -1], want[..., -1], rtol=0, atol=TOL[dtype] * kw.get("end_time", 1.0))
+    g = rng.standard_normal(want.shape).astype(dtype)
+    wantg = oracle.transform_path_backprop(g, shape[2], shape[1], time_aug=kw.get("time_aug", False),
+                                           lead_lag=kw.get("lead_lag", False))
+    gotg = P.transform_path_backprop(dev(g), **kw).cpu().numpy()
+    assert gotg.shape == wantg.shape
+    np.testing.assert_allclose(gotg, wantg, rtol=0, atol=TOL[dtype] * 4)
+
+
+def test_transform_feeds_signature_and_autograd(P):
+    rng = np.random.default_rng(5)
+    x = dev(rng.uniform(size=(6, 20, 3)))
+    for kw in (dict(time_aug=True, end_time=1.5), dict(lead_lag=True), dict(time_aug=True, lead_lag=True)):
+        a = P.sig(P.transform_path(x, **kw), 4)
+        b = P.sig(x, 4, **kw)
+        np.testing.assert_allclose(a.cpu().numpy(), b.cpu().numpy(), rtol=1e-11, atol=1e-11)
+        xr = x.clone().requires_grad_(True)
+        y = P.torch_api.transform_path(xr, **kw)
+        w = torch.rand_like(y)
+        (y * w).sum().backward()
+        np.testing.assert_array_equal(xr.grad.cpu().numpy(), P.transform_path_backprop(w, **kw).cpu().numpy())
+
+
+def test_transform_identity_batch_shapes_and_errors(P):
+    x = torch.rand((2, 3, 8, 4), dtype=torch.float64, device=DEV)
+    assert P.transform_path(x) is x
+    assert P.transform_path_backprop(x) is x
+    y = P.transform_path(x, time_aug=True, lead_lag=True)
+    assert y.shape == (2, 3, 15, 9)
+    np.testing.assert_array_equal(y[1, 2].cpu().numpy(), P.transform_path(x[1, 2], time_aug=True, lead_lag=True).cpu().numpy())
+    assert P.transform_path_backprop(y, time_aug=True, lead_lag=True).shape == x.shape
+    assert P.transform_path(x[:, :, ::2], lead_lag=True).shape == (2, 3, 7, 8)          # strided view
+    empty = torch.empty((0, 8, 4), dtype=torch.float64, device=DEV)
+    assert P.transform_path(empty, time_aug=True).shape == (0, 8, 5)
+    one = torch.rand((1, 4), dtype=torch.float64, device=DEV)
+    assert P.transform_path(one, lead_lag=True).shape == (1, 8)
+    with pytest.raises(ValueError):
+        P.transform_path(one, time_aug=True)
+    with pytest.raises(ValueError):
+        P.transform_path_backprop(torch.rand((4, 6), dtype=torch.float64, device=DEV), lead_lag=True)
+    with pytest.raises(TypeError):
+        P.transform_path(x, time_aug=True, end_time=1)
+    with pytest.raises(RuntimeError):
+        P.transform_path(x.cpu(), time_aug=True)
