@@ -159,15 +159,35 @@ struct Tree {
         T pz[M];
     };
 
-    // U_t at chain depth `depth` (1 <= depth <= min(t-1, M)):
-    //   U(1) = z[p_1]/t + S_1[p_1];  U(l+1) = U(l) * z[p_{l+1}] / (t-l) + S_{l+1}[..]
-    // All intermediate values are returned in u[0..depth).
-    template <int t, int depth>
-    __device__ __forceinline__ void chain_u(const Inc& in, T (&u)[M > 0 ? M : 1]) const
+    // Horner values along the prefix: for target level t (2 <= t <= N) and chain depth l + 1 (l < depth(t))
+    //   u[t][0] = z[p_1]/t + S_1[p_1];   u[t][l] = u[t][l-1] * z[p_{l+1}] / (t-l) + S_{l+1}[p_1..p_{l+1}]
+    // (siglib/cpsig/cp_signature.h:464-499 regrouped per word).
+    __host__ __device__ static constexpr int depth(int t) { return t - 1 < M ? t - 1 : M; }
+    struct Chain {
+        T u[N + 1][M];
+    };
+
+    // Keeps the instruction scheduler from re-serialising what the source interleaves: the compiler's machine
+    // model lets dependent FP64 FMAs issue back to back, the hardware stalls them for about two issue slots when
+    // a SIMD holds a single wave.
+    __device__ __forceinline__ static void pin() { __builtin_amdgcn_sched_barrier(0); }
+
+    // All chains of one step, evaluated in lockstep over the depth so that consecutive instructions belong to
+    // different target levels.  Every value is computed from the state before the step.
+    __device__ __forceinline__ void chain_all(const Inc& in, Chain& ch) const
     {
-        u[0] = fmadd(in.pz[0], rcp<T>(t), c[0]);
+        T q[N + 1];     // q[t] = z[p_{l+1}] / (t - l) of the current row
 #pragma unroll
-        for (int l = 1; l < depth; ++l) u[l] = fmadd(u[l - 1] * rcp<T>(t - l), in.pz[l], c[l]);
+        for (int l = 0; l < M; ++l) {
+#pragma unroll
+            for (int t = l + 2; t <= N; ++t)
+                ch.u[t][l] = (l == 0) ? fmadd(in.pz[0], rcp<T>(t), c[0]) : fmadd(ch.u[t][l - 1], q[t], c[l]);
+            if (l + 1 < M) {
+#pragma unroll
+                for (int t = l + 3; t <= N; ++t) q[t] = in.pz[l + 1] * rcp<T>(t - l - 1);
+            }
+            pin();
+        }
     }
 
     template <int E>
@@ -188,36 +208,40 @@ struct Tree {
             for (int ch = 0; ch < NCH; ++ch)
                 s[off(E) + pidx * NCH + ch] = fmadd(upar, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
         } else {
+            // the children's Horner values first, their consumers afterwards: no FMA directly follows its producer
             const T ur = upar * rcp<T>(I - E + 1);
+            T uc[NCH];
 #pragma unroll
-            for (int ch = 0; ch < NCH; ++ch) {
-                const T uc = fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
-                fwd_desc<E + 1, I>(in, uc, pidx * NCH + ch);
-            }
+            for (int ch = 0; ch < NCH; ++ch) uc[ch] = fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+            if constexpr (NCH >= 4) pin();      // narrow fans: the regions between pins would be too small to fill
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) fwd_desc<E + 1, I>(in, uc[ch], pidx * NCH + ch);
         }
     }
 
+    // subtree target levels t, t-1, ..., M+1: descending, so that every read of a shallower depth still sees the
+    // value from before the step
     template <int t>
-    __device__ __forceinline__ void fwd_level(const Inc& in)
+    __device__ __forceinline__ void fwd_subtree(const Inc& in, const Chain& ch)
     {
-        if constexpr (t == 1) {
-            c[0] += in.pz[0];
-        } else if constexpr (t <= M) {
-            T u[M > 0 ? M : 1];
-            chain_u<t, t - 1>(in, u);
-            c[t - 1] = fmadd(u[t - 2], in.pz[t - 1], c[t - 1]);
-        } else {
-            T u[M > 0 ? M : 1];
-            chain_u<t, M>(in, u);
-            fwd_desc<1, t - M>(in, u[M - 1], 0);
+        if constexpr (t > M) {
+            fwd_desc<1, t - M>(in, ch.u[t][M - 1], 0);
+            fwd_subtree<t - 1>(in, ch);
         }
-        if constexpr (t > 1) fwd_level<t - 1>(in);
     }
 
     // S <- S (x) exp(z): target levels in descending order so that every read of
     // a lower level still sees the value from before the step
     // (siglib/cpsig/cp_signature.h:464-499).
-    __device__ __forceinline__ void fwd_step(const Inc& in) { fwd_level<N>(in); }
+    __device__ __forceinline__ void fwd_step(const Inc& in)
+    {
+        Chain ch;
+        chain_all(in, ch);
+        fwd_subtree<N>(in, ch);
+#pragma unroll
+        for (int t = M; t >= 2; --t) c[t - 1] = fmadd(ch.u[t][t - 2], in.pz[t - 1], c[t - 1]);
+        c[0] += in.pz[0];
+    }
 };
 
 // Adjoint state of one lane: partial adjoints of the shared chain (seeded in one
@@ -252,6 +276,13 @@ struct TreeAdj {
         constexpr T sc = rcp<T>(I - E + 1);
         const T v = (I - E + 1 == 1) ? upar : upar * sc;
         T red = T(0);
+        T uc[NCH];
+        if constexpr (E < I) {
+            // the children's Horner values first, their consumers afterwards
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) uc[ch] = fmadd(v, Tr::template zc<E>(in, ch), S.s[Tr::off(E) + pidx * NCH + ch]);
+            if constexpr (NCH >= 4) Tr::pin();
+        }
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
             const int ci = Tr::off(E) + pidx * NCH + ch;
@@ -259,8 +290,7 @@ struct TreeAdj {
             if constexpr (E == I) {
                 adj = gs[ci];
             } else {
-                const T uc = fmadd(v, Tr::template zc<E>(in, ch), S.s[ci]);
-                adj = bwd_desc<E + 1, I>(S, in, dz, uc, pidx * NCH + ch);
+                adj = bwd_desc<E + 1, I>(S, in, dz, uc[ch], pidx * NCH + ch);
                 gs[ci] += adj;
             }
             if constexpr (E == 1) dz.da[ch] = fmadd(adj, v, dz.da[ch]);
@@ -270,39 +300,16 @@ struct TreeAdj {
         return (I - E + 1 == 1) ? red : red * sc;
     }
 
-    // Walk the adjoint `adj` of chain node `from` (1-based depth) up to the root.
-    template <int t, int from>
-    __device__ __forceinline__ void chain_up(const typename Tr::Inc& in, DInc& dz, const T (&u)[M > 0 ? M : 1], T adj)
-    {
-#pragma unroll
-        for (int l = from - 1; l >= 1; --l) {
-            // node p_1..p_l, child letter p_{l+1}
-            const T sc = rcp<T>(t - l);
-            const T v = u[l - 1] * sc;
-            dz.dc[l] = fmadd(adj, v, dz.dc[l]);
-            adj = adj * in.pz[l] * sc;
-            gc[l - 1] += adj;
-        }
-        dz.dc[0] = fmadd(adj, rcp<T>(t), dz.dc[0]);
-    }
-
+    // subtree target levels M+1 .. N in ascending order: the upstream adjoint of depth I is consumed before
+    // deeper targets add into it.  a[t] receives the adjoint flowing into the prefix node's Horner value.
     template <int t>
-    __device__ __forceinline__ void bwd_level(const Tr& S, const typename Tr::Inc& in, DInc& dz)
+    __device__ __forceinline__ void bwd_subtree(const Tr& S, const typename Tr::Inc& in, DInc& dz,
+                                                const typename Tr::Chain& ch, T (&a)[N + 1])
     {
-        if constexpr (t == 1) {
-            dz.dc[0] += gc[0];
-        } else if constexpr (t <= M) {
-            T u[M > 0 ? M : 1];
-            S.template chain_u<t, t - 1>(in, u);
-            chain_up<t, t>(in, dz, u, gc[t - 1]);
-        } else {
-            T u[M > 0 ? M : 1];
-            S.template chain_u<t, M>(in, u);
-            const T red = bwd_desc<1, t - M>(S, in, dz, u[M - 1], 0);
-            gc[M - 1] += red;
-            chain_up<t, M>(in, dz, u, red);
+        if constexpr (t <= N) {
+            a[t] = bwd_desc<1, t - M>(S, in, dz, ch.u[t][M - 1], 0);
+            bwd_subtree<t + 1>(S, in, dz, ch, a);
         }
-        if constexpr (t < N) bwd_level<t + 1>(S, in, dz);
     }
 
     // Pull the adjoint back through one step S_after = S (x) exp(z), where S is
@@ -311,7 +318,34 @@ struct TreeAdj {
     // (siglib/cpsig/cp_signature.h:1147-1187).
     __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
-        bwd_level<1>(S, in, dz);
+        typename Tr::Chain ch;
+        S.chain_all(in, ch);
+        // Every target level t reads the adjoint of its own chain node as it was before the step and adds into
+        // shallower nodes only, so all starting adjoints are taken first and the walks to the root run in
+        // lockstep over the depth (consecutive instructions belong to different levels).
+        T a[N + 1];
+        const T g1 = gc[0];
+#pragma unroll
+        for (int t = 2; t <= M; ++t) a[t] = gc[t - 1];
+        bwd_subtree<M + 1>(S, in, dz, ch, a);
+#pragma unroll
+        for (int t = M + 1; t <= N; ++t) gc[M - 1] += a[t];
+#pragma unroll
+        for (int l = M - 1; l >= 1; --l) {
+            // node p_1..p_l, child letter p_{l+1}; levels t > l pass through it
+#pragma unroll
+            for (int t = l + 1; t <= N; ++t) {
+                const T v = ch.u[t][l - 1] * rcp<T>(t - l);
+                dz.dc[l] = fmadd(a[t], v, dz.dc[l]);
+                a[t] = a[t] * (in.pz[l] * rcp<T>(t - l));
+            }
+#pragma unroll
+            for (int t = l + 1; t <= N; ++t) gc[l - 1] += a[t];
+            Tr::pin();
+        }
+        dz.dc[0] += g1;
+#pragma unroll
+        for (int t = 2; t <= N; ++t) dz.dc[0] = fmadd(a[t], rcp<T>(t), dz.dc[0]);
     }
 };
 
