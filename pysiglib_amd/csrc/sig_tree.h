@@ -163,17 +163,21 @@ struct Tree {
     //   u[t][0] = z[p_1]/t + S_1[p_1];   u[t][l] = u[t][l-1] * z[p_{l+1}] / (t-l) + S_{l+1}[p_1..p_{l+1}]
     // (siglib/cpsig/cp_signature.h:464-499 regrouped per word).
     __host__ __device__ static constexpr int depth(int t) { return t - 1 < M ? t - 1 : M; }
+    // Short prefixes: the chains of all target levels are evaluated first, in lockstep over the depth, so that
+    // consecutive instructions belong to different levels.  Long prefixes have enough levels in flight for the
+    // scheduler to overlap one level's chain with another level's subtree by itself; they go level by level,
+    // which keeps fewer values alive.
+    static constexpr bool kLockstep = M <= 4;
     struct Chain {
         T u[N + 1][M];
     };
 
     // Keeps the instruction scheduler from re-serialising what the source interleaves: the compiler's machine
-    // model lets dependent FP64 FMAs issue back to back, the hardware stalls them for about two issue slots when
-    // a SIMD holds a single wave.
+    // model lets dependent FP64 FMAs issue back to back, while the hardware stalls them when a SIMD holds a
+    // single wave (measured: a few percent of a sweep).
     __device__ __forceinline__ static void pin() { __builtin_amdgcn_sched_barrier(0); }
 
-    // All chains of one step, evaluated in lockstep over the depth so that consecutive instructions belong to
-    // different target levels.  Every value is computed from the state before the step.
+    // All chains of one step in lockstep over the depth; every value is computed from the state before the step.
     __device__ __forceinline__ void chain_all(const Inc& in, Chain& ch) const
     {
         T q[N + 1];     // q[t] = z[p_{l+1}] / (t - l) of the current row
@@ -188,6 +192,17 @@ struct Tree {
             }
             pin();
         }
+    }
+
+    // Level-by-level form, used for long prefixes: U_t at chain depth `depth` (1 <= depth <= min(t-1, M)):
+    //   U(1) = z[p_1]/t + S_1[p_1];  U(l+1) = U(l) * z[p_{l+1}] / (t-l) + S_{l+1}[..]
+    // All intermediate values are returned in u[0..depth).
+    template <int t, int depth>
+    __device__ __forceinline__ void chain_u(const Inc& in, T (&u)[M > 0 ? M : 1]) const
+    {
+        u[0] = fmadd(in.pz[0], rcp<T>(t), c[0]);
+#pragma unroll
+        for (int l = 1; l < depth; ++l) u[l] = fmadd(u[l - 1] * rcp<T>(t - l), in.pz[l], c[l]);
     }
 
     template <int E>
@@ -230,11 +245,32 @@ struct Tree {
         }
     }
 
+    template <int t>
+    __device__ __forceinline__ void fwd_level(const Inc& in)
+    {
+        if constexpr (t == 1) {
+            c[0] += in.pz[0];
+        } else if constexpr (t <= M) {
+            T u[M > 0 ? M : 1];
+            chain_u<t, t - 1>(in, u);
+            c[t - 1] = fmadd(u[t - 2], in.pz[t - 1], c[t - 1]);
+        } else {
+            T u[M > 0 ? M : 1];
+            chain_u<t, M>(in, u);
+            fwd_desc<1, t - M>(in, u[M - 1], 0);
+        }
+        if constexpr (t > 1) fwd_level<t - 1>(in);
+    }
+
     // S <- S (x) exp(z): target levels in descending order so that every read of
     // a lower level still sees the value from before the step
     // (siglib/cpsig/cp_signature.h:464-499).
     __device__ __forceinline__ void fwd_step(const Inc& in)
     {
+        if constexpr (!kLockstep) {
+            fwd_level<N>(in);
+            return;
+        }
         Chain ch;
         chain_all(in, ch);
         fwd_subtree<N>(in, ch);
@@ -300,6 +336,41 @@ struct TreeAdj {
         return (I - E + 1 == 1) ? red : red * sc;
     }
 
+    // Walk the adjoint `adj` of chain node `from` (1-based depth) up to the root.
+    template <int t, int from>
+    __device__ __forceinline__ void chain_up(const typename Tr::Inc& in, DInc& dz, const T (&u)[M > 0 ? M : 1], T adj)
+    {
+#pragma unroll
+        for (int l = from - 1; l >= 1; --l) {
+            // node p_1..p_l, child letter p_{l+1}
+            const T sc = rcp<T>(t - l);
+            const T v = u[l - 1] * sc;
+            dz.dc[l] = fmadd(adj, v, dz.dc[l]);
+            adj = adj * in.pz[l] * sc;
+            gc[l - 1] += adj;
+        }
+        dz.dc[0] = fmadd(adj, rcp<T>(t), dz.dc[0]);
+    }
+
+    template <int t>
+    __device__ __forceinline__ void bwd_level(const Tr& S, const typename Tr::Inc& in, DInc& dz)
+    {
+        if constexpr (t == 1) {
+            dz.dc[0] += gc[0];
+        } else if constexpr (t <= M) {
+            T u[M > 0 ? M : 1];
+            S.template chain_u<t, t - 1>(in, u);
+            chain_up<t, t>(in, dz, u, gc[t - 1]);
+        } else {
+            T u[M > 0 ? M : 1];
+            S.template chain_u<t, M>(in, u);
+            const T red = bwd_desc<1, t - M>(S, in, dz, u[M - 1], 0);
+            gc[M - 1] += red;
+            chain_up<t, M>(in, dz, u, red);
+        }
+        if constexpr (t < N) bwd_level<t + 1>(S, in, dz);
+    }
+
     // subtree target levels M+1 .. N in ascending order: the upstream adjoint of depth I is consumed before
     // deeper targets add into it.  a[t] receives the adjoint flowing into the prefix node's Horner value.
     template <int t>
@@ -318,6 +389,10 @@ struct TreeAdj {
     // (siglib/cpsig/cp_signature.h:1147-1187).
     __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
+        if constexpr (!Tr::kLockstep) {
+            bwd_level<1>(S, in, dz);
+            return;
+        }
         typename Tr::Chain ch;
         S.chain_all(in, ch);
         // Every target level t reads the adjoint of its own chain node as it was before the step and adds into
