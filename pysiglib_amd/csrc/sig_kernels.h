@@ -233,15 +233,15 @@ __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__
     for (; i + 2 <= count; i += 2) {
         cx.load_inc(zb, row + DIR * d);
         loads_issued();
-        step(za, first + DIR * i);
+        step(za, first + DIR * i, IntC<-1>{});
         if constexpr (WAIT_ALL) wait_all_loads();
         cx.load_inc(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
         loads_issued();
-        step(zb, first + DIR * (i + 1));
+        step(zb, first + DIR * (i + 1), IntC<-1>{});
         if constexpr (WAIT_ALL) wait_all_loads();
         row += 2 * DIR * d;
     }
-    if (i < count) step(za, first + DIR * i);
+    if (i < count) step(za, first + DIR * i, IntC<-1>{});
 }
 
 // staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0
@@ -293,13 +293,13 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
         for (; i + 2 <= nk; i += 2) {
             load_row(zb, lp + DIR * D);
             loads_issued();
-            step(za, first + DIR * (done + i));
+            step(za, first + DIR * (done + i), IntC<G0>{});
             load_row(za, lp + 2 * DIR * D);                      // may be row 0 of the next chunk (contiguous or wrap copy)
             loads_issued();
-            step(zb, first + DIR * (done + i + 1));
+            step(zb, first + DIR * (done + i + 1), IntC<G0>{});
             lp += 2 * DIR * D;
         }
-        if (i < nk) step(za, first + DIR * (done + i));          // odd tail: only in the last chunk
+        if (i < nk) step(za, first + DIR * (done + i), IntC<G0>{});          // odd tail: only in the last chunk
         done += nk;
     }
 }
@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const int64_t t0 = seg * lseg;
     const int64_t ns = (L - t0 < lseg) ? L - t0 : lseg;      // steps of this segment (>= 1)
     const T* row = inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;     // row of the segment's first step
-    auto step = [&](const typename Tr::Inc& z, int64_t) { S.fwd_step(z); };
+    auto step = [&](const typename Tr::Inc& z, int64_t, auto) { S.fwd_step(z); };
     if constexpr (ZL) {
         static_assert(LaneCtx<T, D, N, TAIL, K>::WIDE, "staged increments need the wide layout");
         extern __shared__ double lds_raw_f[];
@@ -542,7 +542,9 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         wave_lds_sync();
     };
 
-    auto do_step = [&](const typename Tr::Inc& z, int64_t t) {
+    auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c) {
+        constexpr int G0 = decltype(g0c)::value;
+        constexpr bool FOLD = Ad::template kFoldDepth1<G0>;     // depth-1 pieces already sit in dz.dj
         S.fwd_step(negate<T, D, N, TAIL, K>(z));     // state before the step
         typename Ad::DInc dz;
 #pragma unroll
@@ -551,7 +553,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         for (int a = 0; a < K; ++a) dz.da[a] = T(0);
 #pragma unroll
         for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
-        A.pullback(S, z, dz);
+        A.template pullback<G0>(S, z, dz);
 
         if (tiled) {
             // Idle lanes need no predicate: their adjoints were loaded as zero, so every piece they produce is zero.
@@ -563,9 +565,11 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 for (int j = 0; j < d; ++j) col[j * kRedStride] = T(0);
             }
             // depth-1 letters and chain letters go into the lane's own column; LDS executes a wave's operations in order
+            if constexpr (!FOLD) {
 #pragma unroll
-            for (int a = 0; a < K; ++a)
-                if (cx.a0 + a < d) lds_add(&col[(cx.a0 + a) * kRedStride], dz.da[a]);
+                for (int a = 0; a < K; ++a)
+                    if (cx.a0 + a < d) lds_add(&col[(cx.a0 + a) * kRedStride], dz.da[a]);
+            }
 #pragma unroll
             for (int l = 0; l < M; ++l) lds_add(&col[cx.p[l] * kRedStride], dz.dc[l]);
             ++cs;

@@ -300,12 +300,17 @@ struct TreeAdj {
         T da[K];
         T dc[M];
     };
+    // depth-1 pieces can join dj in registers when the depth-1 letters are compile-time constants and dj is in use
+    template <int G0>
+    static constexpr bool kFoldDepth1 = G0 >= 0 && TAIL >= 2;
 
     // Post-order pullback through the subtree for target depth I.  Returns the
     // adjoint flowing into the parent's Horner value ("reduced" in
     // siglib/cpsig/cp_signature.h:1158-1180); children adjoints are the upstream
     // gradient at depth I and the recursion's return values above it.
-    template <int E, int I>
+    // G0 >= 0: the lane's depth-1 letters are the compile-time letters G0 .. G0+K-1 and their pieces are added
+    // to dj[G0 + a] straight away (da stays untouched); G0 < 0: the letters are only known at run time -> da.
+    template <int E, int I, int G0>
     __device__ __forceinline__ T bwd_desc(const Tr& S, const typename Tr::Inc& in, DInc& dz, T upar, int pidx)
     {
         constexpr int NCH = (E == 1) ? K : DD;
@@ -326,11 +331,16 @@ struct TreeAdj {
             if constexpr (E == I) {
                 adj = gs[ci];
             } else {
-                adj = bwd_desc<E + 1, I>(S, in, dz, uc[ch], pidx * NCH + ch);
+                adj = bwd_desc<E + 1, I, G0>(S, in, dz, uc[ch], pidx * NCH + ch);
                 gs[ci] += adj;
             }
-            if constexpr (E == 1) dz.da[ch] = fmadd(adj, v, dz.da[ch]);
-            else dz.dj[ch] = fmadd(adj, v, dz.dj[ch]);
+            if constexpr (E == 1 && kFoldDepth1<G0>) {
+                if (G0 + ch < DD) dz.dj[(G0 + ch < DD) ? G0 + ch : 0] = fmadd(adj, v, dz.dj[(G0 + ch < DD) ? G0 + ch : 0]);
+            } else if constexpr (E == 1) {
+                dz.da[ch] = fmadd(adj, v, dz.da[ch]);
+            } else {
+                dz.dj[ch] = fmadd(adj, v, dz.dj[ch]);
+            }
             red = fmadd(adj, Tr::template zc<E>(in, ch), red);
         }
         return (I - E + 1 == 1) ? red : red * sc;
@@ -352,7 +362,7 @@ struct TreeAdj {
         dz.dc[0] = fmadd(adj, rcp<T>(t), dz.dc[0]);
     }
 
-    template <int t>
+    template <int t, int G0>
     __device__ __forceinline__ void bwd_level(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
         if constexpr (t == 1) {
@@ -364,22 +374,22 @@ struct TreeAdj {
         } else {
             T u[M > 0 ? M : 1];
             S.template chain_u<t, M>(in, u);
-            const T red = bwd_desc<1, t - M>(S, in, dz, u[M - 1], 0);
+            const T red = bwd_desc<1, t - M, G0>(S, in, dz, u[M - 1], 0);
             gc[M - 1] += red;
             chain_up<t, M>(in, dz, u, red);
         }
-        if constexpr (t < N) bwd_level<t + 1>(S, in, dz);
+        if constexpr (t < N) bwd_level<t + 1, G0>(S, in, dz);
     }
 
     // subtree target levels M+1 .. N in ascending order: the upstream adjoint of depth I is consumed before
     // deeper targets add into it.  a[t] receives the adjoint flowing into the prefix node's Horner value.
-    template <int t>
+    template <int t, int G0>
     __device__ __forceinline__ void bwd_subtree(const Tr& S, const typename Tr::Inc& in, DInc& dz,
                                                 const typename Tr::Chain& ch, T (&a)[N + 1])
     {
         if constexpr (t <= N) {
-            a[t] = bwd_desc<1, t - M>(S, in, dz, ch.u[t][M - 1], 0);
-            bwd_subtree<t + 1>(S, in, dz, ch, a);
+            a[t] = bwd_desc<1, t - M, G0>(S, in, dz, ch.u[t][M - 1], 0);
+            bwd_subtree<t + 1, G0>(S, in, dz, ch, a);
         }
     }
 
@@ -387,10 +397,11 @@ struct TreeAdj {
     // the state BEFORE the step.  Target levels ascend so that the adjoint of
     // level t is consumed before higher levels add into it
     // (siglib/cpsig/cp_signature.h:1147-1187).
+    template <int G0 = -1>
     __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
         if constexpr (!Tr::kLockstep) {
-            bwd_level<1>(S, in, dz);
+            bwd_level<1, G0>(S, in, dz);
             return;
         }
         typename Tr::Chain ch;
@@ -402,7 +413,7 @@ struct TreeAdj {
         const T g1 = gc[0];
 #pragma unroll
         for (int t = 2; t <= M; ++t) a[t] = gc[t - 1];
-        bwd_subtree<M + 1>(S, in, dz, ch, a);
+        bwd_subtree<M + 1, G0>(S, in, dz, ch, a);
 #pragma unroll
         for (int t = M + 1; t <= N; ++t) gc[M - 1] += a[t];
 #pragma unroll
