@@ -386,13 +386,35 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
 // ---------------------------------------------------------------------------
 // LDS tile of the increment-gradient reduction: one row per (step-in-chunk, letter), one column per lane.
 constexpr int kRedStride = 65;
-// steps per chunk of the reduction tile (at most 16 KB of LDS per wave); 0: the path is too wide for the tile
-template <typename T>
-__host__ __device__ constexpr int red_chunk(int d)
+// Reduction plan of one backward instance.  PAIR: before a step's per-letter sums go to the tile, the two
+// half-waves exchange halves of the letter range (v_permlane32_swap) and add, so that lanes 0-31 hold letters
+// 0 .. H-1 and lanes 32-63 letters H .. 2H-1 (H = ceil(d/2)), each already summed over the lane pair
+// (lane, lane ^ 32).  The tile then has H rows per step instead of d: half the LDS writes and half the reads of
+// the row sums.  Needs compile-time depth-1 letters (their pieces must already sit in the per-letter sums) and
+// an LDS atomic that tolerates two lanes adding to one word (ds_add_f64).
+template <typename T, int D, int TAIL, int K, bool ZL>
+struct RedPlan {
+    static constexpr int NG = D > 0 ? (D + K - 1) / K : 0;
+    static constexpr bool PAIR = ZL && D > 0 && NG <= 3 && TAIL >= 2 && sizeof(T) == 8;
+    static constexpr int kRows = int(16384 / (kRedStride * sizeof(T)));       // 31 (f64) / 63 (f32)
+    __host__ __device__ static constexpr int rows_per_step(int d) { return PAIR ? (d + 1) / 2 : d; }
+    // steps per chunk of the tile; 0: the path is too wide for the tile
+    __host__ __device__ static constexpr int steps(int d)
+    {
+        const int r = rows_per_step(d);
+        return r > kRows ? 0 : (kRows / r > 8 ? 8 : kRows / r);
+    }
+    __host__ __device__ static constexpr int64_t tile_elems(int d) { return int64_t(steps(d)) * rows_per_step(d) * kRedStride; }
+};
+
+// lanes 0-31: lo[lane] + lo[lane + 32];  lanes 32-63: hi[lane - 32] + hi[lane]
+__device__ __forceinline__ double pair_sum32(double lo, double hi)
 {
-    const int rows = int(16384 / (kRedStride * sizeof(T)));     // 31 (f64) / 63 (f32)
-    return d > rows ? 0 : (rows / d > 8 ? 8 : rows / d);
+    const auto r0 = __builtin_amdgcn_permlane32_swap(unsigned(__double2loint(lo)), unsigned(__double2loint(hi)), false, false);
+    const auto r1 = __builtin_amdgcn_permlane32_swap(unsigned(__double2hiint(lo)), unsigned(__double2hiint(hi)), false, false);
+    return __hiloint2double(int(r1[0]), int(r0[0])) + __hiloint2double(int(r1[1]), int(r0[1]));
 }
+__device__ __forceinline__ float pair_sum32(float lo, float) { return lo; }     // never used: PAIR needs 8-byte words
 
 // Orders the LDS traffic of ONE wave: the hardware executes a wave's LDS operations in issue order, so lanes
 // see each other's earlier writes and atomics without any wait; only the compiler has to be kept from moving
@@ -485,10 +507,13 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave_in_block = threadIdx.x >> 6;
     constexpr bool WIDE = Cx::WIDE;
-    const int CH = red_chunk<T>(d);
+    using Plan = RedPlan<T, D, TAIL, K, ZL>;
+    constexpr bool PAIR = Plan::PAIR;
+    const int CH = Plan::steps(d);
+    const int RS = Plan::rows_per_step(d);      // tile rows per step
     const bool tiled = CH > 0;
     const int slots = WIDE ? 1 : cx.G.ppw;
-    T* wbuf = lds + int64_t(wave_in_block) * (tiled ? int64_t(CH) * d * kRedStride : int64_t(slots) * d);
+    T* wbuf = lds + int64_t(wave_in_block) * (tiled ? Plan::tile_elems(d) : int64_t(slots) * d);
     T* acc = wbuf + int64_t(cx.id.slot) * d;
     const int nsg = slots > 1 ? slots : 2;                    // column segments per row
     const int seg_cnt = slots > 1 ? int(cx.G.lpp) : kWave / 2; // lanes per segment
@@ -506,7 +531,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
 
     auto reduce_chunk = [&](int n_slots) {
         wave_lds_sync();
-        const int items = n_slots * d * nsg;
+        const int items = n_slots * RS * nsg;
         for (int it = lane; it < items; it += kWave) {
             const int sg = it % nsg, r = it / nsg;
             const T* src = wbuf + r * kRedStride + sg * seg_cnt;
@@ -530,8 +555,11 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 for (; i < seg_cnt; ++i) s0 += src[i];
             }
             T sum = (s0 + s1) + (s2 + s3);
-            const int slot = r / d, j = r % d;
-            if (slots > 1) {
+            const int slot = r / RS, j = r % RS;
+            if constexpr (PAIR) {
+                const int letter = j + RS * sg;      // the two halves of a row belong to different letters
+                if (letter < d && b_first < batch) dev_add(&dzinc[(b_first * L + (t_chunk - slot)) * d + letter], sum);
+            } else if (slots > 1) {
                 const int64_t bb = b_first + sg;
                 if (bb < batch) dev_add(&dzinc[(bb * L + (t_chunk - slot)) * d + j], sum);
             } else {
@@ -557,21 +585,36 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
 
         if (tiled) {
             // Idle lanes need no predicate: their adjoints were loaded as zero, so every piece they produce is zero.
-            T* col = wbuf + cs * (d * kRedStride) + lane;
-            if constexpr (TAIL >= 2) {
+            T* col = wbuf + cs * (RS * kRedStride) + lane;
+            if constexpr (PAIR) {
+                static_assert(!PAIR || FOLD, "pairing needs the depth-1 pieces folded into the per-letter sums");
+                constexpr int H = (Tr::DD + 1) / 2;
+#pragma unroll
+                for (int r = 0; r < H; ++r)
+                    col[r * kRedStride] = pair_sum32(dz.dj[r], r + H < Tr::DD ? dz.dj[r + H < Tr::DD ? r + H : 0] : T(0));
+                // chain letters: row and half-wave of the letter, column of this lane within that half
+                T* base = wbuf + cs * (RS * kRedStride) + (lane & 31);
+#pragma unroll
+                for (int l = 0; l < M; ++l) {
+                    const int hi = cx.p[l] >= H ? 1 : 0;
+                    lds_add_shared(&base[(cx.p[l] - H * hi) * kRedStride + 32 * hi], dz.dc[l]);
+                }
+            } else if constexpr (TAIL >= 2) {
 #pragma unroll
                 for (int j = 0; j < Tr::DD; ++j) col[j * kRedStride] = dz.dj[j];
             } else {
                 for (int j = 0; j < d; ++j) col[j * kRedStride] = T(0);
             }
             // depth-1 letters and chain letters go into the lane's own column; LDS executes a wave's operations in order
-            if constexpr (!FOLD) {
+            if constexpr (!PAIR) {
+                if constexpr (!FOLD) {
 #pragma unroll
-                for (int a = 0; a < K; ++a)
-                    if (cx.a0 + a < d) lds_add(&col[(cx.a0 + a) * kRedStride], dz.da[a]);
+                    for (int a = 0; a < K; ++a)
+                        if (cx.a0 + a < d) lds_add(&col[(cx.a0 + a) * kRedStride], dz.da[a]);
+                }
+#pragma unroll
+                for (int l = 0; l < M; ++l) lds_add(&col[cx.p[l] * kRedStride], dz.dc[l]);
             }
-#pragma unroll
-            for (int l = 0; l < M; ++l) lds_add(&col[cx.p[l] * kRedStride], dz.dc[l]);
             ++cs;
             if (cs == CH || t == 0) {
                 reduce_chunk(cs);
@@ -617,7 +660,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* row = inc + (cx.id.b * (L + 2) + L) * d;      // row of the last step
     if constexpr (ZL) {
         static_assert(WIDE, "staged increments need the wide layout");
-        T* lds_wave = lds + kWavesPerBlock * (red_chunk<T>(Tr::DD) * Tr::DD * kRedStride) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
+        T* lds_wave = lds + kWavesPerBlock * Plan::tile_elems(Tr::DD) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
         constexpr int NG = (Tr::DD + K - 1) / K;
         if constexpr (NG <= 3) {
             static_for<0, NG - 1>([&](auto gc) {

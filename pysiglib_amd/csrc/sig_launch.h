@@ -59,9 +59,9 @@ hipError_t launch_tree_bwd(const BwdParams& p)
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
     size_t lds;
     int use_lds = 1;
-    const int ch = red_chunk<T>(p.d);
-    if (ch > 0) {
-        lds = size_t(kWavesPerBlock) * size_t(ch) * size_t(p.d) * kRedStride * sizeof(T);
+    using Plan = RedPlan<T, D, TAIL, K, ZL>;
+    if (Plan::steps(p.d) > 0) {
+        lds = size_t(kWavesPerBlock) * size_t(Plan::tile_elems(p.d)) * sizeof(T);
     } else {
         lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
         if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }
