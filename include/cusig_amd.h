@@ -105,6 +105,33 @@ CUSIG_AMD_API int transform_path_backprop_cuda_d(const double* derivs, double* d
                                                  uint64_t dimension, uint64_t length, bool time_aug, bool lead_lag,
                                                  double end_time) CUSIG_AMD_NOEXCEPT;
 
+/* Signature of each straight-line displacement [batch, dimension] -> [batch, sig_length - !scalar_term].
+ * Replaces: linear_sig_cuda_{f,d} (decl siglib/cusig/cusig.h:942-944; arithmetic siglib/cpsig/cp_sig_join.h:36-104),
+ * bound by pysiglib/load_siglib.py (CUSIG_LINEAR_SIG), called from pysiglib/linear_sig.py. */
+CUSIG_AMD_API int linear_sig_cuda_f(const float* displacement, float* out, uint64_t batch_size, uint64_t dimension,
+                                    uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int linear_sig_cuda_d(const double* displacement, double* out, uint64_t batch_size, uint64_t dimension,
+                                    uint64_t degree, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
+/* Appends (or prepends) one straight-line segment to each signature: out = sig (x) exp(z), resp. exp(z) (x) sig.
+ * Replaces: sig_join_cuda_{f,d} (decl siglib/cusig/cusig.h:962-964; arithmetic siglib/cpsig/cp_sig_join.h:107-160),
+ * bound by pysiglib/load_siglib.py:456-460, called from pysiglib/sig_join.py. */
+CUSIG_AMD_API int sig_join_cuda_f(const float* sig, const float* displacement, float* out, uint64_t batch_size,
+                                  uint64_t dimension, uint64_t degree, bool prepend, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_join_cuda_d(const double* sig, const double* displacement, double* out, uint64_t batch_size,
+                                  uint64_t dimension, uint64_t degree, bool prepend, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
+/* Gradients of sig_join w.r.t. the signature (scalar slot zero) and the displacement.
+ * Replaces: sig_join_backprop_cuda_{f,d} (decl siglib/cusig/cusig.h:984-986; arithmetic
+ * siglib/cpsig/cp_sig_join.h:163-238), bound by pysiglib/load_siglib.py:461-465, called from
+ * pysiglib/sig_join_backprop.py. */
+CUSIG_AMD_API int sig_join_backprop_cuda_f(const float* d_out, float* d_sig, float* d_displacement, const float* sig,
+                                           const float* displacement, uint64_t batch_size, uint64_t dimension,
+                                           uint64_t degree, bool prepend, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_join_backprop_cuda_d(const double* d_out, double* d_sig, double* d_displacement, const double* sig,
+                                           const double* displacement, uint64_t batch_size, uint64_t dimension,
+                                           uint64_t degree, bool prepend, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
 /* Message of the last failing call made by the calling thread ("" if none).
  * Replaces: cusig_last_error_message, probed by pysiglib/load_siglib.py:108-110
  * and read by pysiglib/error_codes.py:28-42. */

@@ -55,6 +55,21 @@ int sigref_transform_path_backprop_f(const float *derivs, float *out, uint64_t b
                                      uint64_t length, int time_aug, int lead_lag);
 int sigref_transform_path_backprop_d(const double *derivs, double *out, uint64_t batch, uint64_t dimension,
                                      uint64_t length, int time_aug, int lead_lag);
+/* linear_sig_{f,d}, sig_join_{f,d}, sig_join_backprop_{f,d} of the reference (siglib/cpsig/cpsig.h) without n_jobs. */
+int sigref_linear_sig_f(const float *displacement, float *out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                        int scalar_term);
+int sigref_sig_join_f(const float *sig, const float *displacement, float *out, uint64_t batch, uint64_t dimension,
+                      uint64_t degree, int prepend, int scalar_term);
+int sigref_sig_join_backprop_f(const float *dout, float *dsig, float *ddisplacement, const float *sig,
+                               const float *displacement, uint64_t batch, uint64_t dimension, uint64_t degree,
+                               int prepend, int scalar_term);
+int sigref_linear_sig_d(const double *displacement, double *out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                        int scalar_term);
+int sigref_sig_join_d(const double *sig, const double *displacement, double *out, uint64_t batch, uint64_t dimension,
+                      uint64_t degree, int prepend, int scalar_term);
+int sigref_sig_join_backprop_d(const double *dout, double *dsig, double *ddisplacement, const double *sig,
+                               const double *displacement, uint64_t batch, uint64_t dimension, uint64_t degree,
+                               int prepend, int scalar_term);
 #ifdef __cplusplus
 }
 #endif

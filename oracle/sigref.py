@@ -48,6 +48,15 @@ def _load():
         f = getattr(lib, "sigref_transform_path_backprop_" + suf)
         f.restype = i32
         f.argtypes = (ptr, ptr, u64, u64, u64, i32, i32)
+        f = getattr(lib, "sigref_linear_sig_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, u64, u64, u64, i32)
+        f = getattr(lib, "sigref_sig_join_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, u64, u64, u64, i32, i32)
+        f = getattr(lib, "sigref_sig_join_backprop_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, ptr, ptr, u64, u64, u64, i32, i32)
     return lib
 
 
@@ -190,3 +199,47 @@ def transform_path_backprop(derivs, dimension, length, time_aug=False, lead_lag=
     if rc:
         raise RuntimeError("sigref_transform_path_backprop returned %d" % rc)
     return out[0] if single else out
+
+
+def linear_sig(displacement, dimension, degree, scalar_term=False):
+    """Oracle signature of straight-line displacements (..., dimension)."""
+    disp = np.ascontiguousarray(displacement)
+    suf, real = _suffix(disp.dtype)
+    z = _rows(disp, disp.dtype)
+    n = sig_length(dimension, degree) - (0 if scalar_term else 1)
+    out = np.empty((z.shape[0], n), dtype=disp.dtype)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_linear_sig_" + suf)(z.ctypes.data_as(ptr), out.ctypes.data_as(ptr), z.shape[0], dimension,
+                                                  degree, int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_linear_sig returned %d" % rc)
+    return out.reshape(disp.shape[:-1] + (n,))
+
+
+def sig_join(sig, displacement, dimension, degree, prepend=False):
+    sig = np.asarray(sig)
+    suf, real = _suffix(sig.dtype)
+    a, z = _rows(sig, sig.dtype), _rows(displacement, sig.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    out = np.empty_like(a)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_join_" + suf)(a.ctypes.data_as(ptr), z.ctypes.data_as(ptr), out.ctypes.data_as(ptr),
+                                                a.shape[0], dimension, degree, int(prepend), int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_join returned %d" % rc)
+    return out.reshape(sig.shape)
+
+
+def sig_join_backprop(derivs, sig, displacement, dimension, degree, prepend=False):
+    sig = np.asarray(sig)
+    suf, real = _suffix(sig.dtype)
+    a, z, g = _rows(sig, sig.dtype), _rows(displacement, sig.dtype), _rows(derivs, sig.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    dsig, dz = np.empty_like(a), np.empty_like(z)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_join_backprop_" + suf)(
+        g.ctypes.data_as(ptr), dsig.ctypes.data_as(ptr), dz.ctypes.data_as(ptr), a.ctypes.data_as(ptr),
+        z.ctypes.data_as(ptr), a.shape[0], dimension, degree, int(prepend), int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_join_backprop returned %d" % rc)
+    return dsig.reshape(sig.shape), dz.reshape(np.shape(displacement))

@@ -510,6 +510,114 @@ int FN(sigref_transform_path_backprop)(const REAL *derivs, REAL *out, uint64_t b
     return 0;
 }
 
+/* siglib/cpsig/cp_sig_combine.h:232-263 linear_sig_deriv_to_increment_deriv: e = exp(z) (full layout),
+ * de = dF/de (destroyed), dz = dF/dz.  Level k = level (k-1) (x) z / k, pulled back from the top level down. */
+static void FN(exp_pullback)(const REAL *e, REAL *de, REAL *dz, uint64_t d, uint64_t degree, const uint64_t *lvl)
+{
+    for (uint64_t j = 0; j < d; ++j) dz[j] = (REAL)0;
+    for (uint64_t k = degree; k > 1; --k) {
+        const REAL inv = (REAL)1 / (REAL)k;
+        const uint64_t nleft = lvl[k] - lvl[k - 1];
+        for (uint64_t i = 0; i < nleft; ++i) {
+            const REAL *g = de + lvl[k] + i * d;
+            const REAL s = e[lvl[k - 1] + i] * inv;
+            REAL dot = (REAL)0;
+            for (uint64_t j = 0; j < d; ++j) {
+                dot += g[j] * e[1 + j];
+                dz[j] += g[j] * s;
+            }
+            de[lvl[k - 1] + i] += dot * inv;
+        }
+    }
+    if (degree >= 1)
+        for (uint64_t j = 0; j < d; ++j) dz[j] += de[1 + j];
+}
+
+/* siglib/cpsig/cp_sig_join.h:62-104 linear_sig_ / batch_linear_sig_ */
+int FN(sigref_linear_sig)(const REAL *disp, REAL *out, uint64_t batch, uint64_t d, uint64_t degree, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *e = (REAL *)malloc(full * sizeof(REAL));
+    if (!lvl || !e) { free(lvl); free(e); return 1; }
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t off = scalar_term ? 0 : 1;
+    for (uint64_t i = 0; i < batch; ++i) {
+        FN(segment_exp)(disp + i * d, e, d, degree, lvl);
+        memcpy(out + i * stride, e + off, stride * sizeof(REAL));
+    }
+    free(lvl); free(e);
+    return 0;
+}
+
+/* siglib/cpsig/cp_sig_join.h:107-160 sig_join_: out = sig (x) exp(z), or exp(z) (x) sig when prepending */
+int FN(sigref_sig_join)(const REAL *sig, const REAL *disp, REAL *out, uint64_t batch, uint64_t d, uint64_t degree,
+                        int prepend, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *a = (REAL *)malloc(2 * full * sizeof(REAL));
+    if (!lvl || !a) { free(lvl); free(a); return 1; }
+    REAL *e = a + full;
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t off = scalar_term ? 0 : 1;
+    for (uint64_t i = 0; i < batch; ++i) {
+        a[0] = (REAL)1;
+        memcpy(a + off, sig + i * stride, stride * sizeof(REAL));
+        FN(segment_exp)(disp + i * d, e, d, degree, lvl);
+        if (prepend) {
+            FN(chen_inplace)(e, a, degree, lvl);
+            memcpy(out + i * stride, e + off, stride * sizeof(REAL));
+        } else {
+            FN(chen_inplace)(a, e, degree, lvl);
+            memcpy(out + i * stride, a + off, stride * sizeof(REAL));
+        }
+    }
+    free(lvl); free(a);
+    return 0;
+}
+
+/* siglib/cpsig/cp_sig_join.h:163-238 sig_join_backprop_ */
+int FN(sigref_sig_join_backprop)(const REAL *dout, REAL *dsig, REAL *ddisp, const REAL *sig, const REAL *disp,
+                                 uint64_t batch, uint64_t d, uint64_t degree, int prepend, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *a = (REAL *)malloc(4 * full * sizeof(REAL));
+    if (!lvl || !a) { free(lvl); free(a); return 1; }
+    REAL *e = a + full, *da = e + full, *de = da + full;
+    sigref_level_index(lvl, d, degree + 2);
+    const uint64_t off = scalar_term ? 0 : 1;
+    for (uint64_t i = 0; i < batch; ++i) {
+        a[0] = (REAL)1;
+        memcpy(a + off, sig + i * stride, stride * sizeof(REAL));
+        FN(segment_exp)(disp + i * d, e, d, degree, lvl);
+        if (prepend) {      /* out = e (x) a */
+            de[0] = (REAL)0;
+            memcpy(de + off, dout + i * stride, stride * sizeof(REAL));
+            FN(chen_pullback)(e, a, de, da, degree, lvl);
+        } else {            /* out = a (x) e */
+            da[0] = (REAL)0;
+            memcpy(da + off, dout + i * stride, stride * sizeof(REAL));
+            FN(chen_pullback)(a, e, da, de, degree, lvl);
+        }
+        da[0] = de[0] = (REAL)0;
+        memcpy(dsig + i * stride, da + off, stride * sizeof(REAL));
+        FN(exp_pullback)(e, de, ddisp + i * d, d, degree, lvl);
+    }
+    free(lvl); free(a);
+    return 0;
+}
+
 #undef FN
 #undef CAT
 #undef CAT_

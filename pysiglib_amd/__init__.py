@@ -3,9 +3,10 @@
 Drop-in for ``pysiglib.sig`` / ``pysiglib.sig_backprop`` / ``pysiglib.torch_api.sig`` on GPU tensors.
 """
 from . import torch_api
-from .ops import sig_combine, sig_combine_backprop, transform_path, transform_path_backprop
+from .ops import (linear_sig, sig_combine, sig_combine_backprop, sig_join, sig_join_backprop, transform_path,
+                  transform_path_backprop)
 from .sig import sig, sig_backprop, signature
 from .sig_length import sig_length
 
-__all__ = ["sig", "signature", "sig_backprop", "sig_length", "sig_combine", "sig_combine_backprop", "transform_path",
-           "transform_path_backprop", "torch_api"]
+__all__ = ["sig", "signature", "sig_backprop", "sig_length", "sig_combine", "sig_combine_backprop", "sig_join",
+           "sig_join_backprop", "linear_sig", "transform_path", "transform_path_backprop", "torch_api"]

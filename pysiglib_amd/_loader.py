@@ -72,6 +72,15 @@ CUSIG_TRANSFORM_PATH_BACKPROP = _table("transform_path_backprop_cuda", lambda r:
     POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool, r))
 
 
+CUSIG_LINEAR_SIG = _table("linear_sig_cuda", lambda r: (POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool))
+
+CUSIG_SIG_JOIN = _table("sig_join_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool))
+
+CUSIG_SIG_JOIN_BACKPROP = _table("sig_join_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool))
+
+
 def last_error_message():
     msg = CUSIG.cusig_last_error_message()
     return msg.decode("utf-8", errors="replace") if msg else ""

@@ -144,10 +144,10 @@ struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
 };
-static std::mutex g_ws_mutex;
+std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
-static void* workspace(int slot, size_t bytes)
+void* workspace(int slot, size_t bytes)
 {
     int dev = 0;
     SIG_HIP(hipGetDevice(&dev));

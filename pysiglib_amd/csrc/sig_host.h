@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <mutex>
 #include <new>
 #include <stdexcept>
 #include <string>
@@ -11,6 +12,11 @@
 namespace sigamd {
 
 extern thread_local char g_last_error[4096];
+
+// Grow-only device buffers, one per (current device, slot), released by cusig_shutdown(); hold g_ws_mutex while a
+// buffer is in use (defined in sig_api.hip).  Slots 0-3: signature sweeps; 4-5: sig_join_backprop.
+extern std::mutex g_ws_mutex;
+void* workspace(int slot, size_t bytes);
 
 inline void clear_last_error() { g_last_error[0] = 0; }
 inline void set_last_error(const char* msg) { std::snprintf(g_last_error, sizeof g_last_error, "%s", msg ? msg : ""); }

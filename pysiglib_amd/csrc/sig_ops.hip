@@ -1,8 +1,13 @@
 // Operators either side of the signature sweep, behind the reference's entry points:
 //   sig_combine_cuda_{f,d}, sig_combine_backprop_cuda_{f,d}   (siglib/cusig/cu_sig_combine.cu:157-337)
 //   transform_path_cuda_{f,d}, transform_path_backprop_cuda_{f,d} (siglib/cusig/cu_path_transforms.cu:48-205)
+//   linear_sig_cuda_{f,d}, sig_join_cuda_{f,d}, sig_join_backprop_cuda_{f,d} (siglib/cusig/cusig.h:929-987; arithmetic of
+//   siglib/cpsig/cp_sig_join.h:36-238 and linear_sig_deriv_to_increment_deriv, siglib/cpsig/cp_sig_combine.h:232-263)
 // The Chen product itself is the kernel the time-segmented forward sweep folds its pieces with.
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <mutex>
 
 #include "../../include/cusig_amd.h"
 #include "sig_host.h"
@@ -114,6 +119,147 @@ __global__ __launch_bounds__(kBlock) void transform_path_bwd_kernel(
     }
 }
 
+
+// level t (1-based), index w inside the level and start `lo` of the level for coefficient r of a scalar-free row
+struct WordPos {
+    int t;
+    int64_t w, lo, size;
+};
+__device__ __forceinline__ WordPos word_pos(int64_t r, int d)
+{
+    WordPos p{1, 0, 0, d};
+    while (r >= p.lo + p.size) { p.lo += p.size; p.size *= d; ++p.t; }
+    p.w = r - p.lo;
+    return p;
+}
+
+// Signature of a straight line: exp(z)_t[w] = z[w_1] ... z[w_t] / t!   (siglib/cpsig/cp_sig_join.h:36-60)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void linear_sig_kernel(
+    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, int d, int64_t sig_len, int64_t stride, int off)
+{
+    const int64_t total = batch * sig_len;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / sig_len, r = e % sig_len;
+        const WordPos p = word_pos(r, d);
+        const T* z = disp + b * d;
+        T v = T(1);
+        int64_t idx = p.w;
+        for (int k = p.t; k >= 1; --k) {        // letters from the right, dividing by k as the reference's level recursion does
+            v *= z[idx % d] / T(k);
+            idx /= d;
+        }
+        out[b * stride + off + r] = v;
+        if (off && r == 0) out[b * stride] = T(1);
+    }
+}
+
+// out = A (x) exp(z) (append) or exp(z) (x) A (prepend), one thread per output coefficient:
+//   append : out_t[w] = sum_{k=0..t} A_{t-k}[w_1..w_{t-k}] * z[w_{t-k+1}] ... z[w_t] / k!
+//   prepend: out_t[w] = sum_{k=0..t} z[w_1] ... z[w_k] / k! * A_{t-k}[w_{k+1}..w_t]          (A_0 = 1)
+// (siglib/cpsig/cp_sig_join.h:107-160)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void sig_join_kernel(
+    const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, int d, int64_t sig_len,
+    int64_t stride, int off, int prepend)
+{
+    const int64_t total = batch * sig_len;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / sig_len, r = e % sig_len;
+        const WordPos p = word_pos(r, d);
+        const T* a = A + b * stride + off;
+        const T* z = disp + b * d;
+        T acc = a[p.lo + p.w];
+        T ek = T(1);
+        int64_t lo = p.lo, size = p.size;       // level t-k of A
+        if (!prepend) {
+            int64_t idx = p.w;
+            for (int k = 1; k <= p.t; ++k) {
+                ek *= z[idx % d] / T(k);
+                idx /= d;
+                size /= d;
+                lo -= size;
+                acc = fmadd(k < p.t ? a[lo + idx] : T(1), ek, acc);
+            }
+        } else {
+            int64_t rem = p.w;
+            for (int k = 1; k <= p.t; ++k) {
+                size /= d;                       // d^(t-k)
+                ek *= z[rem / size] / T(k);
+                rem %= size;
+                lo -= size;
+                acc = fmadd(k < p.t ? a[lo + rem] : T(1), ek, acc);
+            }
+        }
+        out[b * stride + off + r] = acc;
+        if (off && r == 0) out[b * stride] = T(1);
+    }
+}
+
+// Adjoint of z -> exp(z): dz[j] = sum_t 1/t! sum_{w in d^t} dE_t[w] sum_{i : w_i = j} prod_{m != i} z[w_m]
+// (closed form of the level recursion in siglib/cpsig/cp_sig_combine.h:232-263).  One thread per coefficient,
+// per-block partial sums in LDS (or straight to HBM for very wide paths), dz zeroed beforehand.
+constexpr int kExpMaxDegree = 64;
+constexpr int kExpAccMax = 4096;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
+    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int d, int64_t sig_len, int64_t stride,
+    int off, int blocks_per_item, int use_lds)
+{
+    extern __shared__ double exp_lds_raw[];
+    T* acc = reinterpret_cast<T*>(exp_lds_raw);
+    const int64_t b = blockIdx.x / blocks_per_item;
+    const int chunk = blockIdx.x % blocks_per_item;
+    if (use_lds) {
+        for (int j = threadIdx.x; j < d; j += kBlock) acc[j] = T(0);
+        __syncthreads();
+    }
+    const T* z = disp + b * d;
+    const T* g = dE + b * stride + off;
+    for (int64_t r = int64_t(chunk) * kBlock + threadIdx.x; r < sig_len; r += int64_t(blocks_per_item) * kBlock) {
+        const WordPos p = word_pos(r, d);
+        T suf[kExpMaxDegree];       // suf[i] = z[w_{i+2}] ... z[w_t] / t!   (0-based position i)
+        int let[kExpMaxDegree];
+        int64_t idx = p.w;
+        T run = g[r];
+        for (int k = 1; k <= p.t; ++k) run /= T(k);
+        for (int i = p.t - 1; i >= 0; --i) {
+            let[i] = int(idx % d);
+            idx /= d;
+            suf[i] = run;
+            run *= z[let[i]];
+        }
+        T pre = T(1);
+        for (int i = 0; i < p.t; ++i) {
+            const T c = pre * suf[i];
+            if (use_lds) lds_add_shared(&acc[let[i]], c);
+            else dev_add(&dz[b * d + let[i]], c);
+            pre *= z[let[i]];
+        }
+    }
+    if (use_lds) {
+        __syncthreads();
+        for (int j = threadIdx.x; j < d; j += kBlock) dev_add(&dz[b * d + j], acc[j]);
+    }
+}
+
+// d = 1: exp(z)_k = z^k / k!, so dz = sum_k dE_k z^(k-1) / (k-1)!
+template <typename T>
+__global__ __launch_bounds__(kBlock) void exp_pullback_dim_one_kernel(
+    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int64_t batch, int64_t degree, int64_t stride, int off)
+{
+    for (int64_t b = int64_t(blockIdx.x) * kBlock + threadIdx.x; b < batch; b += int64_t(gridDim.x) * kBlock) {
+        const T z = disp[b];
+        const T* g = dE + b * stride + off;
+        T pw = T(1), sum = T(0);
+        for (int64_t k = 1; k <= degree; ++k) {
+            sum = fmadd(g[k - 1], pw, sum);
+            pw *= z / T(k);
+        }
+        dz[b] = sum;
+    }
+}
+
 struct SigShape {
     uint64_t n_coef, stride;
     int off;
@@ -172,6 +318,98 @@ static void sig_combine_backprop_impl(const T* derivs, T* d1, T* d2, const T* si
         hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, derivs,
                            d1, d2, sig1, sig2, int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef),
                            int64_t(s.stride), s.off);
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+
+template <typename T>
+static void linear_sig_impl(const T* disp, T* out, uint64_t batch, uint64_t dimension, uint64_t degree, bool scalar_term)
+{
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "linear_sig_cuda");
+    if (batch == 0) return;
+    checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    if (s.n_coef == 0) {
+        if (scalar_term)
+            hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
+                               int64_t(1), 1);
+    } else {
+        hipLaunchKernelGGL((linear_sig_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, disp, out,
+                           int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off);
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+template <typename T>
+static void sig_join_impl(const T* sig, const T* disp, T* out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                          bool prepend, bool scalar_term)
+{
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_join_cuda");
+    if (batch == 0) return;
+    checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    if (s.n_coef == 0) {
+        if (scalar_term)
+            hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
+                               int64_t(1), 1);
+    } else {
+        hipLaunchKernelGGL((sig_join_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, sig, disp, out,
+                           int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off, int(prepend));
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+template <typename T>
+static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T* sig, const T* disp, uint64_t batch,
+                                   uint64_t dimension, uint64_t degree, bool prepend, bool scalar_term)
+{
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_join_backprop_cuda");
+    if (batch == 0) return;
+    const uint64_t bytes = checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
+    const uint64_t dz_elems = checked_mul(batch, dimension, "displacement gradient");
+    if (dimension >= 2 && degree >= uint64_t(kExpMaxDegree)) throw std::runtime_error("sig_join_backprop_cuda: degree too high");
+    SIG_HIP(hipDeviceSynchronize());
+    hipStream_t stream = nullptr;
+    hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(dz_elems)), dim3(kBlock), 0, stream, d_disp, int64_t(dz_elems));
+    if (s.n_coef == 0) {
+        if (scalar_term) hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, d_sig, int64_t(batch));
+        SIG_HIP(hipGetLastError());
+        SIG_HIP(hipStreamSynchronize(stream));
+        return;
+    }
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    T* E = static_cast<T*>(workspace(4, bytes));
+    T* dE = static_cast<T*>(workspace(5, bytes));
+    hipLaunchKernelGGL((linear_sig_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, disp, E,
+                       int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off);
+    // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
+    const unsigned grid = grid_for(batch * s.n_coef);
+    if (prepend)
+        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, d_out, dE, d_sig, (const T*)E, sig,
+                           int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride), s.off);
+    else
+        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, d_out, d_sig, dE, sig, (const T*)E,
+                           int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride), s.off);
+    if (dimension == 1) {
+        hipLaunchKernelGGL((exp_pullback_dim_one_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, (const T*)dE, disp,
+                           d_disp, int64_t(batch), int64_t(degree), int64_t(s.stride), s.off);
+    } else {
+        const int use_lds = dimension <= uint64_t(kExpAccMax);
+        uint64_t per_item = (s.n_coef + kBlock * 8 - 1) / (kBlock * 8);       // about 8 coefficients per thread
+        if (per_item < 1) per_item = 1;
+        const uint64_t cap = std::max<uint64_t>(1, (65535ull * 16ull) / batch);
+        if (per_item > cap) per_item = cap;
+        const uint64_t blocks = checked_mul(batch, per_item, "grid");
+        if (blocks > 0x7fffffffull) throw std::runtime_error("sig_join_backprop_cuda: batch too large");
+        hipLaunchKernelGGL((exp_pullback_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock),
+                           use_lds ? size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp, d_disp, int(dimension),
+                           int64_t(s.n_coef), int64_t(s.stride), s.off, int(per_item), use_lds);
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -271,6 +509,45 @@ CUSIG_AMD_API int transform_path_backprop_cuda_d(const double* derivs, double* d
                                                  double) noexcept
 {
     return guarded([&] { transform_path_backprop_impl<double>(derivs, data_out, batch_size, dimension, length, time_aug, lead_lag); });
+}
+
+CUSIG_AMD_API int linear_sig_cuda_f(const float* displacement, float* out, uint64_t batch_size, uint64_t dimension,
+                                    uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] { linear_sig_impl<float>(displacement, out, batch_size, dimension, degree, scalar_term); });
+}
+CUSIG_AMD_API int linear_sig_cuda_d(const double* displacement, double* out, uint64_t batch_size, uint64_t dimension,
+                                    uint64_t degree, bool scalar_term) noexcept
+{
+    return guarded([&] { linear_sig_impl<double>(displacement, out, batch_size, dimension, degree, scalar_term); });
+}
+CUSIG_AMD_API int sig_join_cuda_f(const float* sig, const float* displacement, float* out, uint64_t batch_size,
+                                  uint64_t dimension, uint64_t degree, bool prepend, bool scalar_term) noexcept
+{
+    return guarded([&] { sig_join_impl<float>(sig, displacement, out, batch_size, dimension, degree, prepend, scalar_term); });
+}
+CUSIG_AMD_API int sig_join_cuda_d(const double* sig, const double* displacement, double* out, uint64_t batch_size,
+                                  uint64_t dimension, uint64_t degree, bool prepend, bool scalar_term) noexcept
+{
+    return guarded([&] { sig_join_impl<double>(sig, displacement, out, batch_size, dimension, degree, prepend, scalar_term); });
+}
+CUSIG_AMD_API int sig_join_backprop_cuda_f(const float* d_out, float* d_sig, float* d_displacement, const float* sig,
+                                           const float* displacement, uint64_t batch_size, uint64_t dimension,
+                                           uint64_t degree, bool prepend, bool scalar_term) noexcept
+{
+    return guarded([&] {
+        sig_join_backprop_impl<float>(d_out, d_sig, d_displacement, sig, displacement, batch_size, dimension, degree, prepend,
+                                      scalar_term);
+    });
+}
+CUSIG_AMD_API int sig_join_backprop_cuda_d(const double* d_out, double* d_sig, double* d_displacement, const double* sig,
+                                           const double* displacement, uint64_t batch_size, uint64_t dimension,
+                                           uint64_t degree, bool prepend, bool scalar_term) noexcept
+{
+    return guarded([&] {
+        sig_join_backprop_impl<double>(d_out, d_sig, d_displacement, sig, displacement, batch_size, dimension, degree, prepend,
+                                       scalar_term);
+    });
 }
 
 }  // extern "C"

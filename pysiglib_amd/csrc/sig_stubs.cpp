@@ -28,8 +28,6 @@ STUB_PAIR(log_sig_combine_cuda)
 STUB_PAIR(log_sig_from_path_cuda)
 STUB_PAIR(log_sig_from_path_backprop_cuda)
 STUB_PAIR(log_sig_combine_backprop_cuda)
-STUB_PAIR(sig_join_cuda)
-STUB_PAIR(sig_join_backprop_cuda)
 STUB_PAIR(sig_coef_cuda)
 STUB_PAIR(sig_coef_backprop_cuda)
 STUB_PAIR(sig_to_log_sig_cuda)
@@ -54,7 +52,6 @@ STUB_PAIR(branched_log_sig_from_path_cuda)
 STUB_PAIR(branched_log_sig_from_path_backprop_cuda)
 STUB_PAIR(branched_sig_combine_backprop_cuda)
 STUB_PAIR(branched_sig_backprop_cuda)
-STUB_PAIR(linear_sig_cuda)
 STUB_PAIR(log_sig_join_cuda)
 STUB_PAIR(log_sig_join_backprop_cuda)
 STUB_PAIR(logsig_to_sig_cuda)

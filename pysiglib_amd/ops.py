@@ -1,10 +1,11 @@
-"""Operators either side of the signature: ``sig_combine``, ``transform_path`` and their backward passes, with the
-reference's signatures (pysiglib/sig.py:28-126, pysiglib/transform_path.py:28-103,
+"""Operators either side of the signature: ``sig_combine``, ``sig_join``, ``linear_sig``, ``transform_path`` and their
+backward passes, with the reference's signatures (pysiglib/sig.py:28-126, pysiglib/sig_join.py,
+pysiglib/sig_join_backprop.py, pysiglib/linear_sig.py, pysiglib/transform_path.py:28-103,
 pysiglib/transform_path_backprop.py, pysiglib/torch_api/torch_api.py) for GPU tensors."""
 import torch
 
-from ._loader import (CUSIG_SIG_COMBINE, CUSIG_SIG_COMBINE_BACKPROP, CUSIG_TRANSFORM_PATH,
-                      CUSIG_TRANSFORM_PATH_BACKPROP)
+from ._loader import (CUSIG_LINEAR_SIG, CUSIG_SIG_COMBINE, CUSIG_SIG_COMBINE_BACKPROP, CUSIG_SIG_JOIN,
+                      CUSIG_SIG_JOIN_BACKPROP, CUSIG_TRANSFORM_PATH, CUSIG_TRANSFORM_PATH_BACKPROP)
 from .data_handlers import PathInput, SigInput, empty_like_input
 from .error_codes import err_msg
 from .param_checks import check_n_jobs, check_non_neg, check_type
@@ -121,3 +122,68 @@ def transform_path_backprop(derivs, *, time_aug=False, lead_lag=False, end_time=
     if code:
         raise Exception("Error in pysiglib.transform_path_backprop: " + err_msg(code))
     return out
+
+
+def linear_sig(displacement, dimension, degree, *, scalar_term=False, n_jobs=1):
+    """Signature of the straight line with the given displacement(s), shape (..., dimension)."""
+    check_type(dimension, "dimension", int)
+    check_non_neg(dimension, "dimension")
+    check_type(degree, "degree", int)
+    check_non_neg(degree, "degree")
+    check_type(scalar_term, "scalar_term", bool)
+    check_n_jobs(n_jobs)
+    n = sig_length(dimension, degree, scalar_term=scalar_term)
+    z = SigInput(displacement, dimension, "displacement")
+    out, out_ptr = empty_like_input(z, (n,))
+    if z.batch_size == 0:
+        return out
+    with torch.cuda.device(z.device):
+        code = CUSIG_LINEAR_SIG[z.dtype](z.data_ptr, out_ptr, z.batch_size, dimension, degree, scalar_term)
+    if code:
+        raise Exception("Error in pysiglib.linear_sig: " + err_msg(code))
+    return out
+
+
+def sig_join(sig, displacement, dimension, degree, *, prepend=False, n_jobs=1):
+    """Extends each signature by one straight-line segment: S(x * v), or S(v * x) with ``prepend=True``."""
+    check_type(dimension, "dimension", int)
+    check_non_neg(dimension, "dimension")
+    check_type(degree, "degree", int)
+    check_non_neg(degree, "degree")
+    check_n_jobs(n_jobs)
+    scalar_term = infer_scalar_term(sig, dimension, degree)
+    n = sig_length(dimension, degree, scalar_term=scalar_term)
+    a, z = SigInput(sig, n, "sig"), SigInput(displacement, dimension, "displacement")
+    _same([a, z], ["sig", "displacement"])
+    out, out_ptr = empty_like_input(a, (n,))
+    if a.batch_size == 0:
+        return out
+    with torch.cuda.device(a.device):
+        code = CUSIG_SIG_JOIN[a.dtype](a.data_ptr, z.data_ptr, out_ptr, a.batch_size, dimension, degree, bool(prepend),
+                                       scalar_term)
+    if code:
+        raise Exception("Error in pysiglib.sig_join: " + err_msg(code))
+    return out
+
+
+def sig_join_backprop(d_out, sig, displacement, dimension, degree, *, prepend=False, n_jobs=1):
+    """Gradients w.r.t. ``sig`` and ``displacement`` given the gradient w.r.t. ``sig_join(sig, displacement)``."""
+    check_type(dimension, "dimension", int)
+    check_non_neg(dimension, "dimension")
+    check_type(degree, "degree", int)
+    check_non_neg(degree, "degree")
+    check_n_jobs(n_jobs)
+    scalar_term = infer_scalar_term(sig, dimension, degree)
+    n = sig_length(dimension, degree, scalar_term=scalar_term)
+    g, a, z = SigInput(d_out, n, "d_out"), SigInput(sig, n, "sig"), SigInput(displacement, dimension, "displacement")
+    _same([g, a, z], ["d_out", "sig", "displacement"])
+    d_sig, d_sig_ptr = empty_like_input(g, (n,))
+    d_disp, d_disp_ptr = empty_like_input(g, (dimension,))
+    if g.batch_size == 0:
+        return d_sig, d_disp
+    with torch.cuda.device(g.device):
+        code = CUSIG_SIG_JOIN_BACKPROP[g.dtype](g.data_ptr, d_sig_ptr, d_disp_ptr, a.data_ptr, z.data_ptr, g.batch_size,
+                                                dimension, degree, bool(prepend), scalar_term)
+    if code:
+        raise Exception("Error in pysiglib.sig_join_backprop: " + err_msg(code))
+    return d_sig, d_disp

@@ -74,3 +74,25 @@ def transform_path(path, *, time_aug=False, lead_lag=False, end_time=1., n_jobs=
     if (not time_aug) and (not lead_lag):
         return path
     return TransformPath.apply(path, time_aug, lead_lag, end_time)
+
+
+class SigJoin(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, sig, displacement, dimension, degree, prepend):
+        from .ops import sig_join as _join
+        ctx.save_for_backward(sig, displacement)
+        ctx.args = (dimension, degree, prepend)
+        return _join(sig, displacement, dimension, degree, prepend=prepend)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .ops import sig_join_backprop as _join_backprop
+        sig, displacement = ctx.saved_tensors
+        dimension, degree, prepend = ctx.args
+        d_sig, d_disp = _join_backprop(grad_output, sig, displacement, dimension, degree, prepend=prepend)
+        return d_sig, d_disp, None, None, None
+
+
+def sig_join(sig, displacement, dimension, degree, *, prepend=False, n_jobs=1):
+    """Differentiable ``sig_join``."""
+    return SigJoin.apply(sig, displacement, dimension, degree, bool(prepend))

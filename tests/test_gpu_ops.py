@@ -241,3 +241,105 @@ def test_transform_identity_batch_shapes_and_errors(P):
         P.transform_path(x, time_aug=True, end_time=1)
     with pytest.raises(RuntimeError):
         P.transform_path(x.cpu(), time_aug=True)
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 6, 5), (3, 4, 70), (5, 3, 4), (1, 7, 3), (4, 1, 2), (3, 0, 3), (10, 5, 32),
+                                         (40, 2, 3), (2, 14, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_linear_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+    rng = np.random.default_rng(13 * d + deg)
+    z = rng.standard_normal((batch, d)).astype(dtype)
+    want = oracle.linear_sig(z, d, deg, scalar_term=scalar_term)
+    got = P.linear_sig(dev(z), d, deg, scalar_term=scalar_term).cpu().numpy()
+    assert got.shape == want.shape and got.dtype == dtype
+    if want.shape[1]:
+        assert row_rel_err(got, want) < TOL[dtype]
+    if scalar_term:
+        assert np.all(got[:, 0] == 1)
+    if deg >= 1 and not scalar_term:        # equals the signature of the two-point path, computed by the sweep kernels
+        x = np.zeros((batch, 2, d), dtype=dtype)
+        x[:, 1] = z
+        np.testing.assert_allclose(got, P.sig(dev(x), deg).cpu().numpy(), rtol=0, atol=TOL[dtype] * max(1.0, np.abs(want).max()))
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 5, 5), (3, 4, 70), (5, 2, 4), (1, 5, 3), (4, 1, 2), (10, 5, 32), (40, 2, 3),
+                                         (2, 14, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("prepend", [False, True])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_sig_join_vs_oracle(P, oracle, d, deg, batch, dtype, prepend, scalar_term):
+    rng = np.random.default_rng(5 * d + deg)
+    n = oracle.sig_length(d, deg) - 1
+    scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
+    a = (rng.standard_normal((batch, n)) * scale).astype(dtype)
+    z = (rng.standard_normal((batch, d)) * 0.7).astype(dtype)
+    g = rng.standard_normal((batch, n)).astype(dtype)
+    if scalar_term:
+        a = np.hstack([np.ones((batch, 1), dtype=dtype), a])
+        g = np.hstack([np.full((batch, 1), 2.0, dtype=dtype), g])
+    off = 1 if scalar_term else 0
+    want = oracle.sig_join(a, z, d, deg, prepend=prepend)
+    got = P.sig_join(dev(a), dev(z), d, deg, prepend=prepend).cpu().numpy()
+    assert got.shape == want.shape and got.dtype == dtype
+    assert np.max(level_rel_err(got[:, off:], want[:, off:], d, deg)) < TOL[dtype]
+    if scalar_term:
+        assert np.all(got[:, 0] == 1)
+    ws, wz = oracle.sig_join_backprop(g, a, z, d, deg, prepend=prepend)
+    ds, dz = P.sig_join_backprop(dev(g), dev(a), dev(z), d, deg, prepend=prepend)
+    assert ds.shape == ws.shape and dz.shape == wz.shape
+    assert row_rel_err(ds.cpu().numpy(), ws) < TOL[dtype]
+    assert row_rel_err(dz.cpu().numpy(), wz) < (TOL[dtype] if dtype == np.float64 else 5e-4)
+    if scalar_term:
+        assert torch.all(ds[:, 0] == 0)
+
+
+@pytest.mark.parametrize("prepend", [False, True])
+def test_sig_join_extends_the_path_and_autograd(P, prepend):
+    rng = np.random.default_rng(77)
+    d, deg = 4, 4
+    x = rng.uniform(size=(6, 30, d))
+    z = rng.standard_normal((6, d))
+    longer = np.concatenate([x[:, :1] - z[:, None], x], axis=1) if prepend else np.concatenate([x, x[:, -1:] + z[:, None]], axis=1)
+    s = P.sig(dev(x), deg)
+    got = P.sig_join(s, dev(z), d, deg, prepend=prepend)
+    np.testing.assert_allclose(got.cpu().numpy(), P.sig(dev(longer), deg).cpu().numpy(), rtol=1e-10, atol=1e-12)
+    e = P.linear_sig(dev(z), d, deg)
+    comb = P.sig_combine(e, s, d, deg) if prepend else P.sig_combine(s, e, d, deg)
+    np.testing.assert_allclose(got.cpu().numpy(), comb.cpu().numpy(), rtol=1e-12, atol=1e-13)
+    sr, zr = s.clone().requires_grad_(True), dev(z).requires_grad_(True)
+    w = torch.rand_like(s)
+    (P.torch_api.sig_join(sr, zr, d, deg, prepend=prepend) * w).sum().backward()
+    ds, dz = P.sig_join_backprop(w, s, dev(z), d, deg, prepend=prepend)
+    np.testing.assert_array_equal(sr.grad.cpu().numpy(), ds.cpu().numpy())
+    # the displacement gradient is accumulated with atomics: equal up to the order of the additions
+    np.testing.assert_allclose(zr.grad.cpu().numpy(), dz.cpu().numpy(), rtol=1e-13, atol=1e-13)
+
+
+def test_join_linear_batch_shapes_and_errors(P, oracle):
+    d, deg = 3, 3
+    n = P.sig_length(d, deg)
+    s = torch.rand((2, 4, n), dtype=torch.float64, device=DEV)
+    z = torch.rand((2, 4, d), dtype=torch.float64, device=DEV)
+    out = P.sig_join(s, z, d, deg)
+    assert out.shape == (2, 4, n)
+    np.testing.assert_allclose(out.cpu().numpy(), oracle.sig_join(s.cpu().numpy(), z.cpu().numpy(), d, deg), rtol=1e-12, atol=1e-12)
+    assert P.sig_join(s[0, 0], z[0, 0], d, deg).shape == (n,)
+    assert P.linear_sig(z, d, deg).shape == (2, 4, n)
+    assert P.linear_sig(z[1, 2], d, deg, scalar_term=True).shape == (n + 1,)
+    ds, dz = P.sig_join_backprop(out, s, z, d, deg)
+    assert ds.shape == s.shape and dz.shape == z.shape
+    empty_s = torch.empty((0, n), dtype=torch.float64, device=DEV)
+    empty_z = torch.empty((0, d), dtype=torch.float64, device=DEV)
+    assert P.sig_join(empty_s, empty_z, d, deg).shape == (0, n)
+    assert P.linear_sig(empty_z, d, deg).shape == (0, n)
+    with pytest.raises(ValueError):
+        P.sig_join(s, z[0], d, deg)
+    with pytest.raises(ValueError):
+        P.sig_join(s, z.float(), d, deg)
+    with pytest.raises(ValueError):
+        P.sig_join(s, z[..., :2], d, deg)
+    with pytest.raises(ValueError):
+        P.linear_sig(z, d + 1, deg)
+    with pytest.raises(RuntimeError):
+        P.linear_sig(z.cpu(), d, deg)

@@ -3,7 +3,10 @@
 Evidence that does not come from the oracle: the reference's hand-computed vectors (tests/_ops_kats.py), its golden
 float32 gradients of sig_combine (tests/golden/reference_fixture.npz, keys sig_comb_bp_*), Chen's identity against the
 already pinned signature, an independent torch Chen product with autograd, and the textbook lead-lag / time
-augmentation written with repeat / linspace.
+augmentation written with repeat / linspace.  linear_sig / sig_join (the reference holds no vectors for them): the
+signature of the two-point path and of the path with one more point (the already pinned signature), the reference's
+own statement sig_join == sig_combine(sig, linear_sig) (pysiglib/sig_join.py docstring), z^k/k! for one channel, and
+autograd through the independent Chen product and segment exponential.
 """
 import numpy as np
 import pytest
@@ -153,3 +156,92 @@ def test_transform_backprop_vs_autograd(kw, shape):
     np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-13, atol=1e-13)
     gotf = sigref.transform_path_backprop(g.astype(np.float32), shape[2], shape[1], **kw)
     np.testing.assert_allclose(gotf, x.grad.numpy(), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("d,deg", [(2, 6), (3, 4), (5, 3), (1, 7), (4, 1), (3, 0)])
+@pytest.mark.parametrize("dtype,tol", [(np.float64, 1e-13), (np.float32, 1e-5)])
+def test_linear_sig_is_signature_of_a_segment(d, deg, dtype, tol):
+    rng = np.random.default_rng(2 * d + deg)
+    z = rng.standard_normal((4, d)).astype(dtype)
+    got = sigref.linear_sig(z, d, deg, scalar_term=True)
+    assert got.dtype == dtype and np.all(got[:, 0] == 1)
+    np.testing.assert_array_equal(got[:, 1:], sigref.linear_sig(z, d, deg))
+    if deg == 0:
+        assert got.shape == (4, 1)
+        return
+    x = np.zeros((4, 2, d), dtype=dtype)
+    x[:, 0] = rng.standard_normal((4, d)).astype(dtype)
+    x[:, 1] = x[:, 0] + z
+    z_eff = (x[:, 1] - x[:, 0]).astype(dtype)
+    np.testing.assert_allclose(sigref.linear_sig(z_eff, d, deg), sigref.signature(x, deg), rtol=tol, atol=tol)
+    # independent statement: z^(x)k / k!
+    want = torch.cat(M._segment_exp(torch.tensor(z.astype(np.float64)), deg), dim=1).numpy()
+    np.testing.assert_allclose(got[:, 1:], want, rtol=10 * tol, atol=10 * tol)
+    if d == 1:
+        fact = np.cumprod(np.arange(1, deg + 1, dtype=np.float64))
+        np.testing.assert_allclose(got[:, 1:], z.astype(np.float64) ** np.arange(1, deg + 1) / fact, rtol=10 * tol, atol=tol)
+
+
+@pytest.mark.parametrize("d,deg", [(2, 5), (3, 4), (5, 2), (1, 5), (4, 1)])
+@pytest.mark.parametrize("prepend", [False, True])
+def test_sig_join_extends_the_path(d, deg, prepend):
+    rng = np.random.default_rng(d + 10 * deg)
+    x = rng.uniform(size=(5, 9, d))
+    z = rng.standard_normal((5, d))
+    s = sigref.signature(x, deg)
+    longer = np.concatenate([x[:, :1] - z[:, None], x], axis=1) if prepend else np.concatenate([x, x[:, -1:] + z[:, None]], axis=1)
+    got = sigref.sig_join(s, z, d, deg, prepend=prepend)
+    assert np.max(M.level_rel_err(got, sigref.signature(longer, deg), d, deg)) < 1e-11
+    # the reference's own statement of the operator
+    e = sigref.linear_sig(z, d, deg)
+    want = sigref.sig_combine(e, s, d, deg) if prepend else sigref.sig_combine(s, e, d, deg)
+    np.testing.assert_allclose(got, want, rtol=1e-13, atol=1e-13)
+    # scalar-term layout and float32
+    one = np.ones((5, 1))
+    got1 = sigref.sig_join(np.hstack([one, s]), z, d, deg, prepend=prepend)
+    assert np.all(got1[:, 0] == 1)
+    np.testing.assert_array_equal(got1[:, 1:], got)
+    gotf = sigref.sig_join(s.astype(np.float32), z.astype(np.float32), d, deg, prepend=prepend)
+    assert gotf.dtype == np.float32
+    np.testing.assert_allclose(gotf, got, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("d,deg", [(2, 5), (3, 4), (5, 2), (1, 5), (4, 1)])
+@pytest.mark.parametrize("prepend", [False, True])
+def test_sig_join_backprop_vs_autograd(d, deg, prepend):
+    rng = np.random.default_rng(3 * d + deg)
+    n = sigref.sig_length(d, deg) - 1
+    a, g = rng.standard_normal((4, n)), rng.standard_normal((4, n))
+    z = rng.standard_normal((4, d))
+    ta, tz = torch.tensor(a, requires_grad=True), torch.tensor(z, requires_grad=True)
+    e = M._segment_exp(tz, deg)
+    out = M._chen(e, _levels(ta, d, deg), deg) if prepend else M._chen(_levels(ta, d, deg), e, deg)
+    torch.cat(out, dim=1).backward(torch.tensor(g))
+    ds, dz = sigref.sig_join_backprop(g, a, z, d, deg, prepend=prepend)
+    np.testing.assert_allclose(ds, ta.grad.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dz, tz.grad.numpy(), rtol=1e-12, atol=1e-12)
+    # scalar-term layout: same numbers, zero in the scalar slot
+    one, zero = np.ones((4, 1)), np.zeros((4, 1))
+    ds1, dz1 = sigref.sig_join_backprop(np.hstack([zero + 3.0, g]), np.hstack([one, a]), z, d, deg, prepend=prepend)
+    assert np.all(ds1[:, 0] == 0)
+    np.testing.assert_allclose(ds1[:, 1:], ds, rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(dz1, dz, rtol=1e-13, atol=1e-13)
+    dsf, dzf = sigref.sig_join_backprop(g.astype(np.float32), a.astype(np.float32), z.astype(np.float32), d, deg, prepend=prepend)
+    np.testing.assert_allclose(dsf, ds, rtol=5e-4, atol=5e-4)
+    np.testing.assert_allclose(dzf, dz, rtol=5e-4, atol=5e-4)
+
+
+def test_sig_join_backprop_finite_differences():
+    rng = np.random.default_rng(8)
+    d, deg = 3, 4
+    x = rng.uniform(size=(2, 6, d))
+    s, z = sigref.signature(x, deg), rng.standard_normal((2, d))
+    g = rng.standard_normal(s.shape)
+    _, dz = sigref.sig_join_backprop(g, s, z, d, deg)
+    h = 1e-6
+    for j in range(d):
+        zp, zm = z.copy(), z.copy()
+        zp[:, j] += h
+        zm[:, j] -= h
+        num = ((sigref.sig_join(s, zp, d, deg) - sigref.sig_join(s, zm, d, deg)) * g).sum(axis=1) / (2 * h)
+        np.testing.assert_allclose(dz[:, j], num, rtol=1e-6, atol=1e-7)
