@@ -38,6 +38,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-configs", action="store_true", help="also time configs 2-4 (reported under 'configs')")
+    ap.add_argument("--ops", action="store_true",
+                    help="time the operators either side of the sweep (sig_combine, sig_join, linear_sig, transform_path "
+                         "and backward passes) on HBM-bound shapes and print their own JSON line instead")
     ap.add_argument("--copy-calib", action="store_true",
                     help="only run a plain 256 MiB device copy (calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE) and exit")
     return ap.parse_args()
@@ -129,6 +132,59 @@ def cpu_baseline(np, cfgmod):
                       "oracle/sigref.c -O3 -march=native, one path per thread"}
 
 
+def bench_ops(args, torch, loader):
+    """Operators either side of the sweep: HBM-bound element-wise kernels.  Achieved GB/s = algorithmic bytes (every
+    input read once, every output written once) / wall time of the synchronous C-ABI call."""
+    import statistics
+    real = loader.DTYPES["float64"]
+    d, deg, batch = 10, 5, 1024
+    n = int(loader.CUSIG.cusig_amd_sig_length(d, deg)) - 1
+    f64 = dict(dtype=torch.float64, device="cuda:0")
+    a = torch.rand((batch, n), **f64) * 0.1
+    b = torch.rand((batch, n), **f64) * 0.1
+    g = torch.rand((batch, n), **f64)
+    z = torch.rand((batch, d), **f64)
+    o1, o2, oz = torch.empty_like(a), torch.empty_like(a), torch.empty_like(z)
+    pb, plen, pdim = 4096, 1024, 16
+    path = torch.rand((pb, plen, pdim), **f64)
+    tpath = torch.empty((pb, 2 * plen - 1, 2 * pdim + 1), **f64)
+    gpath = torch.empty_like(path)
+
+    def p(t):
+        return ctypes.cast(t.data_ptr(), ctypes.POINTER(real))
+
+    sig_bytes = batch * n * 8
+    cases = [
+        ("sig_combine", lambda: loader.CUSIG_SIG_COMBINE["float64"](p(a), p(b), p(o1), batch, d, deg, False), 3 * sig_bytes),
+        ("sig_combine_backprop", lambda: loader.CUSIG_SIG_COMBINE_BACKPROP["float64"](p(g), p(o1), p(o2), p(a), p(b), batch, d, deg, False), 5 * sig_bytes),
+        ("linear_sig", lambda: loader.CUSIG_LINEAR_SIG["float64"](p(z), p(o1), batch, d, deg, False), sig_bytes),
+        ("sig_join", lambda: loader.CUSIG_SIG_JOIN["float64"](p(a), p(z), p(o1), batch, d, deg, False, False), 2 * sig_bytes),
+        ("sig_join_backprop", lambda: loader.CUSIG_SIG_JOIN_BACKPROP["float64"](p(g), p(o1), p(oz), p(a), p(z), batch, d, deg, False, False), 3 * sig_bytes),
+        ("transform_path", lambda: loader.CUSIG_TRANSFORM_PATH["float64"](p(path), p(tpath), pb, pdim, plen, True, True, 1.0), (path.numel() + tpath.numel()) * 8),
+        ("transform_path_backprop", lambda: loader.CUSIG_TRANSFORM_PATH_BACKPROP["float64"](p(tpath), p(gpath), pb, pdim, plen, True, True, 1.0), (path.numel() + tpath.numel()) * 8),
+    ]
+    out = {}
+    for name, fn, nbytes in cases:
+        for _ in range(args.warmup):
+            rc = fn()
+            if rc:
+                raise RuntimeError("%s failed: %d %s" % (name, rc, loader.last_error_message()))
+        times = []
+        for _ in range(args.steps):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        ms = statistics.median(times) * 1e3
+        out[name] = {"call_ms": ms, "algorithmic_bytes": nbytes, "GB_per_s": nbytes / (ms * 1e-3) / 1e9,
+                     "hbm_frac": nbytes / (ms * 1e-3) / 8e12}
+    print(json.dumps({"metric": "operator kernels, achieved HBM GB/s (algorithmic bytes / synchronous call time)",
+                      "unit": "GB/s", "peak": 8000.0, "dtype": "f64", "data": "synthetic", "steps": args.steps,
+                      "warmup": args.warmup,
+                      "config": {"workload": "signatures: batch %d, dim %d, degree %d (%d coefficients); paths: (%d, %d, %d) "
+                                             "with lead-lag + time" % (batch, d, deg, n, pb, plen, pdim)},
+                      "ops": out}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -154,6 +210,10 @@ def main():
             dst.copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         print(json.dumps({"copy_calib_bytes_read": n * 8, "copy_calib_bytes_written": n * 8, "copies": 3}))
+        return
+
+    if args.ops:
+        bench_ops(args, torch, loader)
         return
 
     r1 = Runner(1, torch, np, loader, cfgmod)

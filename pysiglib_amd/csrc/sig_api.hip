@@ -397,10 +397,14 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             for (int g = 1; g < nseg; ++g) {
                 const bool last = g == nseg - 1;
                 T* dst = last ? out : tmp[(g - 1) & 1];
-                hipLaunchKernelGGL((sig_combine_kernel<T>), dim3(grid_for(batch * n_coef)), dim3(kBlock), 0, stream,
-                                   acc, segs + uint64_t(g) * n_coef, dst, int64_t(batch), int(s.d_aug), int(degree),
-                                   int64_t(n_coef), acc_stride, int64_t(n_coef) * nseg,
-                                   last ? int64_t(s.stride) : int64_t(n_coef), 0, 0, last ? sc : 0);
+                const int64_t b_stride = int64_t(n_coef) * nseg, c_stride = last ? int64_t(s.stride) : int64_t(n_coef);
+                const T* rhs = segs + uint64_t(g) * n_coef;
+                launch_indexed(n_coef, n_coef, batch, [&](auto ix, dim3 grid) {
+                    using I = decltype(ix);
+                    hipLaunchKernelGGL((sig_combine_kernel<T, I>), grid, dim3(kBlock), 0, stream, acc, rhs, dst,
+                                       int64_t(batch), DivBy<I>(s.d_aug), I(n_coef), acc_stride, b_stride, c_stride, 0, 0,
+                                       last ? sc : 0);
+                });
                 SIG_HIP(hipGetLastError());
                 acc = dst;
                 acc_stride = int64_t(n_coef);

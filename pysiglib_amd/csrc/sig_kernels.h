@@ -795,43 +795,101 @@ __global__ __launch_bounds__(kBlock) void degree_one_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Index arithmetic of the coefficient-per-thread kernels.  Word indices are decoded with divisions by the path
+// dimension only; with 32-bit indices (every index below 2^31, the usual case) that division is a multiply-high
+// and a shift by host-computed constants, with 64-bit indices a plain division.
+// ---------------------------------------------------------------------------
+template <typename I>
+struct DivBy;
+template <>
+struct DivBy<uint32_t> {
+    uint32_t d, mul, shr;
+    __host__ explicit DivBy(uint64_t den) : d(uint32_t(den)), mul(0), shr(0)
+    {
+        if (d > 1) {
+            uint32_t lg = 0;
+            while ((uint64_t(1) << lg) < d) ++lg;
+            const uint32_t p = 31 + lg;
+            mul = uint32_t(((uint64_t(1) << p) + d - 1) / d);
+            shr = p - 32;
+        }
+    }
+    __device__ __forceinline__ uint32_t quot(uint32_t n) const { return d == 1 ? n : __umulhi(n, mul) >> shr; }   // n < 2^31
+};
+template <>
+struct DivBy<uint64_t> {
+    uint64_t d;
+    __host__ explicit DivBy(uint64_t den) : d(den) {}
+    __device__ __forceinline__ uint64_t quot(uint64_t n) const { return n / d; }
+};
+
+// calls f(index type tag, 2-D grid): grid.x covers `per_item` work items of one batch entry, grid.y the batch
+template <typename F>
+void launch_indexed(uint64_t max_index, uint64_t per_item, uint64_t batch, F&& f)
+{
+    uint64_t gx = (per_item + kBlock - 1) / kBlock;
+    if (gx < 1) gx = 1;
+    if (gx > (1u << 20)) gx = 1u << 20;
+    const uint64_t gy = batch < 65535 ? (batch < 1 ? 1 : batch) : 65535;
+    const dim3 grid{unsigned(gx), unsigned(gy), 1};
+    if (max_index < (uint64_t(1) << 31)) f(uint32_t{}, grid);
+    else f(uint64_t{}, grid);
+}
+
+// level t (1-based) of coefficient r of a scalar-free signature row, its index w inside the level, the start
+// `lo` and the size of the level
+template <typename I>
+struct WordPos {
+    int t;
+    I w, lo, size;
+};
+template <typename I>
+__device__ __forceinline__ WordPos<I> word_pos(I r, I d)
+{
+    WordPos<I> p{1, 0, 0, d};
+    while (r >= p.lo + p.size) { p.lo += p.size; p.size *= d; ++p.t; }
+    p.w = r - p.lo;
+    return p;
+}
+
+// ---------------------------------------------------------------------------
 // Chen product C = A (x) B of two signatures per path (scalar terms implicit 1):
 //   C_t[w] = A_t[w] + B_t[w] + sum_{k=1..t-1} A_k[w_1..w_k] * B_{t-k}[w_{k+1}..w_t]
 // (siglib/cpsig/cp_sig_combine.h:35-66).  One thread per output coefficient; rows
 // of A, B, C may have different strides and C may carry a leading scalar slot.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_kernel(
-    const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int64_t batch, int d, int degree,
-    int64_t sig_len /* sum_{k=1..degree} d^k */, int64_t a_stride, int64_t b_stride, int64_t c_stride,
+    const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int64_t batch, DivBy<I> dv,
+    I sig_len /* sum_{k=1..degree} d^k */, int64_t a_stride, int64_t b_stride, int64_t c_stride,
     int a_off, int b_off, int c_off)
 {
-    const int64_t total = batch * sig_len;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int64_t b = e / sig_len;
-        int64_t r = e % sig_len;
-        // level t and word index w of coefficient r
-        int t = 1;
-        int64_t lvl = d, lo = 0;
-        while (r >= lo + lvl) { lo += lvl; lvl *= d; ++t; }
-        const int64_t w = r - lo;
+    const I d = I(dv.d);
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * a_stride + a_off;
         const T* bb = B + b * b_stride + b_off;
-        T acc = a[lo + w] + bb[lo + w];
-        // split w after its first k letters: prefix index w / d^(t-k), suffix index w % d^(t-k)
-        int64_t div = lvl / d;          // d^(t-1)
-        int64_t a_lo = 0, a_sz = d;     // level k of A
-        int64_t b_lo = lo - div;        // start of level t-1 of B
-        int64_t b_sz = div;
-        for (int k = 1; k < t; ++k) {
-            acc = fmadd(a[a_lo + w / div], bb[b_lo + w % div], acc);
-            a_lo += a_sz; a_sz *= d;
-            b_sz /= d; b_lo -= b_sz;
-            div /= d;
-        }
         T* c = C + b * c_stride;
-        c[c_off + r] = acc;
-        if (c_off && r == 0) c[0] = T(1);
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            const WordPos<I> p = word_pos<I>(r, d);
+            T acc = a[p.lo + p.w] + bb[p.lo + p.w];
+            // split after k letters, k = t-1 .. 1: the prefix loses its last letter, which becomes the
+            // leading letter of the suffix
+            I pre = p.w, suf = 0, pw = 1;       // pw = d^(t-k-1)
+            I a_lo = p.lo, a_sz = p.size;       // level k+1 of A
+            I b_lo = 0;                         // start of level t-k of B
+            for (int k = p.t - 1; k >= 1; --k) {
+                const I q = dv.quot(pre);
+                suf += (pre - q * d) * pw;
+                pw *= d;
+                pre = q;
+                a_sz = dv.quot(a_sz);
+                a_lo -= a_sz;
+                acc = fmadd(a[a_lo + pre], bb[b_lo + suf], acc);
+                b_lo += pw;
+            }
+            c[c_off + r] = acc;
+            if (c_off && r == 0) c[0] = T(1);
+        }
     }
 }
 

@@ -19,138 +19,141 @@ namespace sigamd {
 //   dA_t[w] = dC_t[w] + sum_{m=1..N-t} sum_{v in d^m} dC_{t+m}[w v] * B_m[v]        (contiguous block of dC)
 //   dB_t[w] = dC_t[w] + sum_{k=1..N-t} sum_{u in d^k} dC_{t+k}[u w] * A_k[u]        (stride d^t in dC)
 // Scalar slots of both gradients are zero.
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, const T* __restrict__ A,
-    const T* __restrict__ B, int64_t batch, int d, int degree, int64_t sig_len, int64_t stride, int off)
+    const T* __restrict__ B, int64_t batch, I d, int degree, I sig_len, int64_t stride, int off)
 {
-    const int64_t total = batch * sig_len;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int64_t b = e / sig_len;
-        const int64_t r = e % sig_len;
-        int t = 1;
-        int64_t lvl = d, lo = 0;
-        while (r >= lo + lvl) { lo += lvl; lvl *= d; ++t; }
-        const int64_t w = r - lo;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* g = dC + b * stride + off;
         const T* a = A + b * stride + off;
         const T* bb = B + b * stride + off;
-        T ga = g[lo + w], gb = ga;
-        int64_t up_lo = lo + lvl;      // start of level t + m in dC
-        int64_t up_sz = lvl * d;       // its size d^(t+m)
-        int64_t lo_m = 0, sz_m = d;    // level m of A / B
-        for (int m = 1; t + m <= degree; ++m) {
-            const T* blockp = g + up_lo + w * sz_m;        // words w v, v in d^m
-            T s0 = T(0), s1 = T(0);
-            int64_t v = 0;
-            for (; v + 2 <= sz_m; v += 2) {
-                s0 = fmadd(blockp[v], bb[lo_m + v], s0);
-                s1 = fmadd(blockp[v + 1], bb[lo_m + v + 1], s1);
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            const WordPos<I> p = word_pos<I>(r, d);
+            T ga = g[r], gb = ga;
+            I up_lo = p.lo + p.size;      // start of level t + m in dC
+            I lo_m = 0, sz_m = d;         // level m of A / B
+            for (int m = 1; p.t + m <= degree; ++m) {
+                const T* blockp = g + up_lo + p.w * sz_m;        // words w v, v in d^m
+                T s0 = T(0), s1 = T(0);
+                I v = 0;
+                for (; v + 2 <= sz_m; v += 2) {
+                    s0 = fmadd(blockp[v], bb[lo_m + v], s0);
+                    s1 = fmadd(blockp[v + 1], bb[lo_m + v + 1], s1);
+                }
+                for (; v < sz_m; ++v) s0 = fmadd(blockp[v], bb[lo_m + v], s0);
+                ga += s0 + s1;
+                const T* strided = g + up_lo + p.w;               // words u w, u in d^m: index u * d^t + w
+                T q0 = T(0), q1 = T(0);
+                I u = 0;
+                for (; u + 2 <= sz_m; u += 2) {
+                    q0 = fmadd(strided[u * p.size], a[lo_m + u], q0);
+                    q1 = fmadd(strided[(u + 1) * p.size], a[lo_m + u + 1], q1);
+                }
+                for (; u < sz_m; ++u) q0 = fmadd(strided[u * p.size], a[lo_m + u], q0);
+                gb += q0 + q1;
+                up_lo += p.size * sz_m;
+                lo_m += sz_m;
+                sz_m *= d;
             }
-            for (; v < sz_m; ++v) s0 = fmadd(blockp[v], bb[lo_m + v], s0);
-            ga += s0 + s1;
-            const T* strided = g + up_lo + w;               // words u w, u in d^m: index u * d^t + w
-            T q0 = T(0), q1 = T(0);
-            int64_t u = 0;
-            for (; u + 2 <= sz_m; u += 2) {
-                q0 = fmadd(strided[u * lvl], a[lo_m + u], q0);
-                q1 = fmadd(strided[(u + 1) * lvl], a[lo_m + u + 1], q1);
-            }
-            for (; u < sz_m; ++u) q0 = fmadd(strided[u * lvl], a[lo_m + u], q0);
-            gb += q0 + q1;
-            up_lo += up_sz;
-            up_sz *= d;
-            lo_m += sz_m;
-            sz_m *= d;
+            dA[b * stride + off + r] = ga;
+            dB[b * stride + off + r] = gb;
+            if (off && r == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
         }
-        dA[b * stride + off + r] = ga;
-        dB[b * stride + off + r] = gb;
-        if (off && r == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
     }
 }
 
 // Materialised lead-lag / time augmentation: point i of the lead-lag path has lag = x[i/2] and
 // lead = x[i/2 + (i odd)]; time is the last channel, i * end_time / (len_eff - 1)
-// (siglib/cpsig/cp_path_transforms.h:36-142).
-template <typename T>
+// (siglib/cpsig/cp_path_transforms.h:36-142).  One thread per output element of a path; `dtd` divides by the
+// transformed dimension.
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void transform_path_kernel(
-    const T* __restrict__ in, T* __restrict__ out, int64_t batch, int64_t len, int d, int time_aug, int lead_lag, T scale)
+    const T* __restrict__ in, T* __restrict__ out, int64_t batch, I len, I d, DivBy<I> dtd, int time_aug, int lead_lag, T scale)
 {
-    const int td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
-    const int64_t tl = lead_lag ? 2 * len - 1 : len;
-    const int64_t total = batch * tl * td;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int c = int(e % td);
-        const int64_t i = (e / td) % tl;
-        const int64_t b = e / (int64_t(td) * tl);
-        const T* x = in + b * len * d;
-        T v;
-        if (time_aug && c == td - 1) v = T(i) * scale;
-        else if (!lead_lag) v = x[i * d + c];
-        else if (c < d) v = x[(i >> 1) * d + c];
-        else v = x[((i >> 1) + (i & 1)) * d + (c - d)];
-        out[e] = v;
+    const I td = I(dtd.d);
+    const I tl = lead_lag ? 2 * len - 1 : len;
+    const I per = tl * td;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* x = in + b * int64_t(len) * int64_t(d);
+        T* o = out + b * int64_t(per);
+        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
+            const I i = dtd.quot(e);
+            const I c = e - i * td;
+            T v;
+            if (time_aug && c == td - 1) v = T(i) * scale;
+            else if (!lead_lag) v = x[i * d + c];
+            else if (c < d) v = x[(i >> 1) * d + c];
+            else v = x[((i >> 1) + (i & 1)) * d + (c - d)];
+            o[e] = v;
+        }
     }
 }
 
 // Adjoint of the augmentation: a raw point collects the gradient of every transformed point that copies it;
-// the time channel has no raw counterpart (siglib/cpsig/cp_path_transforms.h:182-243).
-template <typename T>
+// the time channel has no raw counterpart (siglib/cpsig/cp_path_transforms.h:182-243).  `dd` divides by the raw
+// dimension.
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void transform_path_bwd_kernel(
-    const T* __restrict__ derivs, T* __restrict__ out, int64_t batch, int64_t len, int d, int time_aug, int lead_lag)
+    const T* __restrict__ derivs, T* __restrict__ out, int64_t batch, I len, DivBy<I> dd, int time_aug, int lead_lag)
 {
-    const int td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
-    const int64_t tl = lead_lag ? 2 * len - 1 : len;
-    const int64_t total = batch * len * d;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int j = int(e % d);
-        const int64_t k = (e / d) % len;
-        const int64_t b = e / (int64_t(d) * len);
-        const T* g = derivs + b * tl * td;
-        T v;
-        if (!lead_lag) {
-            v = g[k * td + j];
-        } else {
-            v = g[(2 * k) * td + j] + g[(2 * k) * td + d + j];
-            if (k + 1 < len) v += g[(2 * k + 1) * td + j];
-            if (k >= 1) v += g[(2 * k - 1) * td + d + j];
+    const I d = I(dd.d);
+    const I td = (lead_lag ? 2 * d : d) + (time_aug ? 1 : 0);
+    const I tl = lead_lag ? 2 * len - 1 : len;
+    const I per = len * d;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* g = derivs + b * int64_t(tl) * int64_t(td);
+        T* o = out + b * int64_t(per);
+        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
+            const I k = dd.quot(e);
+            const I j = e - k * d;
+            T v;
+            if (!lead_lag) {
+                v = g[k * td + j];
+            } else {
+                v = g[(2 * k) * td + j] + g[(2 * k) * td + d + j];
+                if (k + 1 < len) v += g[(2 * k + 1) * td + j];
+                if (k >= 1) v += g[(2 * k - 1) * td + d + j];
+            }
+            o[e] = v;
         }
-        out[e] = v;
     }
 }
 
-
-// level t (1-based), index w inside the level and start `lo` of the level for coefficient r of a scalar-free row
-struct WordPos {
-    int t;
-    int64_t w, lo, size;
-};
-__device__ __forceinline__ WordPos word_pos(int64_t r, int d)
-{
-    WordPos p{1, 0, 0, d};
-    while (r >= p.lo + p.size) { p.lo += p.size; p.size *= d; ++p.t; }
-    p.w = r - p.lo;
-    return p;
-}
+// 1/k for k = 0 .. 64 (entry 0 unused): the kernels below divide by small integers once per letter, and an FP64
+// division costs some thirty instructions
+constexpr int kExpMaxDegree = 64;
+__constant__ double kRcp[kExpMaxDegree + 1] = {
+    0.0, 1.0 / 1, 1.0 / 2, 1.0 / 3, 1.0 / 4, 1.0 / 5, 1.0 / 6, 1.0 / 7, 1.0 / 8, 1.0 / 9, 1.0 / 10, 1.0 / 11,
+    1.0 / 12, 1.0 / 13, 1.0 / 14, 1.0 / 15, 1.0 / 16, 1.0 / 17, 1.0 / 18, 1.0 / 19, 1.0 / 20, 1.0 / 21, 1.0 / 22,
+    1.0 / 23, 1.0 / 24, 1.0 / 25, 1.0 / 26, 1.0 / 27, 1.0 / 28, 1.0 / 29, 1.0 / 30, 1.0 / 31, 1.0 / 32, 1.0 / 33,
+    1.0 / 34, 1.0 / 35, 1.0 / 36, 1.0 / 37, 1.0 / 38, 1.0 / 39, 1.0 / 40, 1.0 / 41, 1.0 / 42, 1.0 / 43, 1.0 / 44,
+    1.0 / 45, 1.0 / 46, 1.0 / 47, 1.0 / 48, 1.0 / 49, 1.0 / 50, 1.0 / 51, 1.0 / 52, 1.0 / 53, 1.0 / 54, 1.0 / 55,
+    1.0 / 56, 1.0 / 57, 1.0 / 58, 1.0 / 59, 1.0 / 60, 1.0 / 61, 1.0 / 62, 1.0 / 63, 1.0 / 64};
+template <typename T>
+__device__ __forceinline__ T rcp_of(int k) { return k <= kExpMaxDegree ? T(kRcp[k]) : T(1) / T(k); }
 
 // Signature of a straight line: exp(z)_t[w] = z[w_1] ... z[w_t] / t!   (siglib/cpsig/cp_sig_join.h:36-60)
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void linear_sig_kernel(
-    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, int d, int64_t sig_len, int64_t stride, int off)
+    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I sig_len, int64_t stride, int off)
 {
-    const int64_t total = batch * sig_len;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int64_t b = e / sig_len, r = e % sig_len;
-        const WordPos p = word_pos(r, d);
-        const T* z = disp + b * d;
-        T v = T(1);
-        int64_t idx = p.w;
-        for (int k = p.t; k >= 1; --k) {        // letters from the right, dividing by k as the reference's level recursion does
-            v *= z[idx % d] / T(k);
-            idx /= d;
+    const I d = I(dv.d);
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* z = disp + b * int64_t(d);
+        T* o = out + b * stride;
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            const WordPos<I> p = word_pos<I>(r, d);
+            T v = T(1);
+            I idx = p.w;
+            for (int k = p.t; k >= 1; --k) {        // letters from the right
+                const I q = dv.quot(idx);
+                v *= z[idx - q * d] * rcp_of<T>(k);
+                idx = q;
+            }
+            o[off + r] = v;
+            if (off && r == 0) o[0] = T(1);
         }
-        out[b * stride + off + r] = v;
-        if (off && r == 0) out[b * stride] = T(1);
     }
 }
 
@@ -158,88 +161,104 @@ __global__ __launch_bounds__(kBlock) void linear_sig_kernel(
 //   append : out_t[w] = sum_{k=0..t} A_{t-k}[w_1..w_{t-k}] * z[w_{t-k+1}] ... z[w_t] / k!
 //   prepend: out_t[w] = sum_{k=0..t} z[w_1] ... z[w_k] / k! * A_{t-k}[w_{k+1}..w_t]          (A_0 = 1)
 // (siglib/cpsig/cp_sig_join.h:107-160)
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_join_kernel(
-    const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, int d, int64_t sig_len,
+    const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I sig_len,
     int64_t stride, int off, int prepend)
 {
-    const int64_t total = batch * sig_len;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int64_t b = e / sig_len, r = e % sig_len;
-        const WordPos p = word_pos(r, d);
+    const I d = I(dv.d);
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * stride + off;
-        const T* z = disp + b * d;
-        T acc = a[p.lo + p.w];
-        T ek = T(1);
-        int64_t lo = p.lo, size = p.size;       // level t-k of A
-        if (!prepend) {
-            int64_t idx = p.w;
-            for (int k = 1; k <= p.t; ++k) {
-                ek *= z[idx % d] / T(k);
-                idx /= d;
-                size /= d;
-                lo -= size;
-                acc = fmadd(k < p.t ? a[lo + idx] : T(1), ek, acc);
+        const T* z = disp + b * int64_t(d);
+        T* o = out + b * stride;
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            const WordPos<I> p = word_pos<I>(r, d);
+            T acc = a[p.lo + p.w];
+            T ek = T(1);
+            I lo = p.lo, size = p.size;       // level t-k of A
+            if (!prepend) {
+                I idx = p.w;
+                for (int k = 1; k <= p.t; ++k) {
+                    const I q = dv.quot(idx);
+                    ek *= z[idx - q * d] * rcp_of<T>(k);
+                    idx = q;
+                    size = dv.quot(size);
+                    lo -= size;
+                    acc = fmadd(k < p.t ? a[lo + idx] : T(1), ek, acc);
+                }
+            } else {
+                // letters from the left: reverse the word once (the letters come out of the divisions right to left)
+                I idx = p.w, rev = 0;
+                for (int k = 0; k < p.t; ++k) {
+                    const I q = dv.quot(idx);
+                    rev = rev * d + (idx - q * d);
+                    idx = q;
+                }
+                I rem = p.w;
+                for (int k = 1; k <= p.t; ++k) {
+                    const I q = dv.quot(rev);
+                    const I letter = rev - q * d;      // w_k
+                    rev = q;
+                    size = dv.quot(size);              // d^(t-k)
+                    ek *= z[letter] * rcp_of<T>(k);
+                    rem -= letter * size;              // w_{k+1} .. w_t
+                    lo -= size;
+                    acc = fmadd(k < p.t ? a[lo + rem] : T(1), ek, acc);
+                }
             }
-        } else {
-            int64_t rem = p.w;
-            for (int k = 1; k <= p.t; ++k) {
-                size /= d;                       // d^(t-k)
-                ek *= z[rem / size] / T(k);
-                rem %= size;
-                lo -= size;
-                acc = fmadd(k < p.t ? a[lo + rem] : T(1), ek, acc);
-            }
+            o[off + r] = acc;
+            if (off && r == 0) o[0] = T(1);
         }
-        out[b * stride + off + r] = acc;
-        if (off && r == 0) out[b * stride] = T(1);
     }
 }
 
 // Adjoint of z -> exp(z): dz[j] = sum_t 1/t! sum_{w in d^t} dE_t[w] sum_{i : w_i = j} prod_{m != i} z[w_m]
 // (closed form of the level recursion in siglib/cpsig/cp_sig_combine.h:232-263).  One thread per coefficient,
 // per-block partial sums in LDS (or straight to HBM for very wide paths), dz zeroed beforehand.
-constexpr int kExpMaxDegree = 64;
 constexpr int kExpAccMax = 4096;
-template <typename T>
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
-    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int d, int64_t sig_len, int64_t stride,
-    int off, int blocks_per_item, int use_lds)
+    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int64_t batch, DivBy<I> dv, I sig_len,
+    int64_t stride, int off, int use_lds)
 {
     extern __shared__ double exp_lds_raw[];
     T* acc = reinterpret_cast<T*>(exp_lds_raw);
-    const int64_t b = blockIdx.x / blocks_per_item;
-    const int chunk = blockIdx.x % blocks_per_item;
-    if (use_lds) {
-        for (int j = threadIdx.x; j < d; j += kBlock) acc[j] = T(0);
-        __syncthreads();
-    }
-    const T* z = disp + b * d;
-    const T* g = dE + b * stride + off;
-    for (int64_t r = int64_t(chunk) * kBlock + threadIdx.x; r < sig_len; r += int64_t(blocks_per_item) * kBlock) {
-        const WordPos p = word_pos(r, d);
-        T suf[kExpMaxDegree];       // suf[i] = z[w_{i+2}] ... z[w_t] / t!   (0-based position i)
-        int let[kExpMaxDegree];
-        int64_t idx = p.w;
-        T run = g[r];
-        for (int k = 1; k <= p.t; ++k) run /= T(k);
-        for (int i = p.t - 1; i >= 0; --i) {
-            let[i] = int(idx % d);
-            idx /= d;
-            suf[i] = run;
-            run *= z[let[i]];
+    const I d = I(dv.d);
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        if (use_lds) {
+            __syncthreads();
+            for (I j = threadIdx.x; j < d; j += kBlock) acc[j] = T(0);
+            __syncthreads();
         }
-        T pre = T(1);
-        for (int i = 0; i < p.t; ++i) {
-            const T c = pre * suf[i];
-            if (use_lds) lds_add_shared(&acc[let[i]], c);
-            else dev_add(&dz[b * d + let[i]], c);
-            pre *= z[let[i]];
+        const T* z = disp + b * int64_t(d);
+        const T* g = dE + b * stride + off;
+        T* out = dz + b * int64_t(d);
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            const WordPos<I> p = word_pos<I>(r, d);
+            T suf[kExpMaxDegree];       // suf[i] = dE[w] / t! * z[w_{i+2}] ... z[w_t]   (0-based position i)
+            I let[kExpMaxDegree];
+            I idx = p.w;
+            T run = g[r];
+            for (int k = 1; k <= p.t; ++k) run *= rcp_of<T>(k);
+            for (int i = p.t - 1; i >= 0; --i) {
+                const I q = dv.quot(idx);
+                let[i] = idx - q * d;
+                idx = q;
+                suf[i] = run;
+                run *= z[let[i]];
+            }
+            T pre = T(1);
+            for (int i = 0; i < p.t; ++i) {
+                const T c = pre * suf[i];
+                if (use_lds) lds_add_shared(&acc[let[i]], c);
+                else dev_add(&out[let[i]], c);
+                pre *= z[let[i]];
+            }
         }
-    }
-    if (use_lds) {
-        __syncthreads();
-        for (int j = threadIdx.x; j < d; j += kBlock) dev_add(&dz[b * d + j], acc[j]);
+        if (use_lds) {
+            __syncthreads();
+            for (I j = threadIdx.x; j < d; j += kBlock) dev_add(&out[j], acc[j]);
+        }
     }
 }
 
@@ -292,9 +311,12 @@ static void sig_combine_impl(const T* sig1, const T* sig2, T* out, uint64_t batc
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        hipLaunchKernelGGL((sig_combine_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, sig1, sig2,
-                           out, int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride),
-                           int64_t(s.stride), int64_t(s.stride), s.off, s.off, s.off);
+        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((sig_combine_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig1, sig2, out, int64_t(batch),
+                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), int64_t(s.stride), int64_t(s.stride),
+                               s.off, s.off, s.off);
+        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -315,9 +337,11 @@ static void sig_combine_backprop_impl(const T* derivs, T* d1, T* d2, const T* si
             hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, d2, int64_t(batch));
         }
     } else {
-        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, derivs,
-                           d1, d2, sig1, sig2, int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef),
-                           int64_t(s.stride), s.off);
+        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, derivs, d1, d2, sig1, sig2,
+                               int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
+        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -337,8 +361,11 @@ static void linear_sig_impl(const T* disp, T* out, uint64_t batch, uint64_t dime
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        hipLaunchKernelGGL((linear_sig_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, disp, out,
-                           int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off);
+        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((linear_sig_kernel<T, I>), grid, dim3(kBlock), 0, stream, disp, out, int64_t(batch),
+                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off);
+        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -358,8 +385,11 @@ static void sig_join_impl(const T* sig, const T* disp, T* out, uint64_t batch, u
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        hipLaunchKernelGGL((sig_join_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, sig, disp, out,
-                           int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off, int(prepend));
+        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((sig_join_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig, disp, out, int64_t(batch),
+                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off, int(prepend));
+        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -386,30 +416,30 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     T* E = static_cast<T*>(workspace(4, bytes));
     T* dE = static_cast<T*>(workspace(5, bytes));
-    hipLaunchKernelGGL((linear_sig_kernel<T>), dim3(grid_for(batch * s.n_coef)), dim3(kBlock), 0, stream, disp, E,
-                       int64_t(batch), int(dimension), int64_t(s.n_coef), int64_t(s.stride), s.off);
-    // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
-    const unsigned grid = grid_for(batch * s.n_coef);
-    if (prepend)
-        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, d_out, dE, d_sig, (const T*)E, sig,
-                           int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride), s.off);
-    else
-        hipLaunchKernelGGL((sig_combine_bwd_kernel<T>), dim3(grid), dim3(kBlock), 0, stream, d_out, d_sig, dE, sig, (const T*)E,
-                           int64_t(batch), int(dimension), int(degree), int64_t(s.n_coef), int64_t(s.stride), s.off);
+    launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((linear_sig_kernel<T, I>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
+                           DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off);
+        // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
+        if (prepend)
+            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, d_out, dE, d_sig, (const T*)E,
+                               sig, int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
+        else
+            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, d_out, d_sig, dE, sig,
+                               (const T*)E, int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
+    });
     if (dimension == 1) {
         hipLaunchKernelGGL((exp_pullback_dim_one_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, (const T*)dE, disp,
                            d_disp, int64_t(batch), int64_t(degree), int64_t(s.stride), s.off);
     } else {
         const int use_lds = dimension <= uint64_t(kExpAccMax);
-        uint64_t per_item = (s.n_coef + kBlock * 8 - 1) / (kBlock * 8);       // about 8 coefficients per thread
-        if (per_item < 1) per_item = 1;
-        const uint64_t cap = std::max<uint64_t>(1, (65535ull * 16ull) / batch);
-        if (per_item > cap) per_item = cap;
-        const uint64_t blocks = checked_mul(batch, per_item, "grid");
-        if (blocks > 0x7fffffffull) throw std::runtime_error("sig_join_backprop_cuda: batch too large");
-        hipLaunchKernelGGL((exp_pullback_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock),
-                           use_lds ? size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp, d_disp, int(dimension),
-                           int64_t(s.n_coef), int64_t(s.stride), s.off, int(per_item), use_lds);
+        // about 8 coefficients per thread, so that a block's LDS partial sums amortise their flush
+        launch_indexed(s.n_coef, (s.n_coef + 7) / 8, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((exp_pullback_kernel<T, I>), grid, dim3(kBlock), use_lds ? size_t(dimension) * sizeof(T) : 0,
+                               stream, (const T*)dE, disp, d_disp, int64_t(batch), DivBy<I>(dimension), I(s.n_coef),
+                               int64_t(s.stride), s.off, use_lds);
+        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -433,8 +463,12 @@ static void transform_path_impl(const T* in, T* out, uint64_t batch, uint64_t di
     SIG_HIP(hipDeviceSynchronize());
     hipStream_t stream = nullptr;
     const T scale = tl > 1 ? end_time / T(tl - 1) : T(0);
-    hipLaunchKernelGGL((transform_path_kernel<T>), dim3(grid_for(total)), dim3(kBlock), 0, stream, in, out, int64_t(batch),
-                       int64_t(length), int(dimension), int(time_aug), int(lead_lag), scale);
+    (void)total;
+    launch_indexed(tl * td, (tl * td + 3) / 4, batch, [&](auto ix, dim3 grid) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((transform_path_kernel<T, I>), grid, dim3(kBlock), 0, stream, in, out, int64_t(batch), I(length),
+                           I(dimension), DivBy<I>(td), int(time_aug), int(lead_lag), scale);
+    });
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
 }
@@ -448,8 +482,15 @@ static void transform_path_backprop_impl(const T* derivs, T* out, uint64_t batch
     const uint64_t total = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
     SIG_HIP(hipDeviceSynchronize());
     hipStream_t stream = nullptr;
-    hipLaunchKernelGGL((transform_path_bwd_kernel<T>), dim3(grid_for(total)), dim3(kBlock), 0, stream, derivs, out,
-                       int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+    (void)total;
+    const uint64_t td = (lead_lag ? 2 * dimension : dimension) + (time_aug ? 1 : 0);
+    const uint64_t tl = lead_lag ? 2 * length - 1 : length;
+    checked_mul(checked_mul(batch, tl, "transformed path"), td, "transformed path");
+    launch_indexed(tl * td, length * dimension, batch, [&](auto ix, dim3 grid) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((transform_path_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, derivs, out, int64_t(batch),
+                           I(length), DivBy<I>(dimension), int(time_aug), int(lead_lag));
+    });
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
 }
