@@ -157,6 +157,9 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: how increments reach the waves: -1 automatic, 0 scalar loads, 1 LDS-staged where compiled. */
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
+/* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only
+ * taken for rows of 2^31 coefficients or more) whatever the size. */
+CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: prefer the compiled lane partition (tail, k) where a shape has several; tail = 0 restores
  * the defaults.  Not thread-safe; meant for offline sweeps. */
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) CUSIG_AMD_NOEXCEPT;

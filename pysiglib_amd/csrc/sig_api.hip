@@ -144,6 +144,7 @@ struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
 };
+int g_force_wide_index = 0;
 std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
@@ -547,6 +548,8 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_l
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
 
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
+
+CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {

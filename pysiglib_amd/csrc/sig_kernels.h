@@ -823,6 +823,9 @@ struct DivBy<uint64_t> {
     __device__ __forceinline__ uint64_t quot(uint64_t n) const { return n / d; }
 };
 
+// test hook: nonzero makes launch_indexed pick 64-bit indices whatever the size (defined in sig_api.hip)
+extern int g_force_wide_index;
+
 // calls f(index type tag, 2-D grid): grid.x covers `per_item` work items of one batch entry, grid.y the batch
 template <typename F>
 void launch_indexed(uint64_t max_index, uint64_t per_item, uint64_t batch, F&& f)
@@ -832,7 +835,7 @@ void launch_indexed(uint64_t max_index, uint64_t per_item, uint64_t batch, F&& f
     if (gx > (1u << 20)) gx = 1u << 20;
     const uint64_t gy = batch < 65535 ? (batch < 1 ? 1 : batch) : 65535;
     const dim3 grid{unsigned(gx), unsigned(gy), 1};
-    if (max_index < (uint64_t(1) << 31)) f(uint32_t{}, grid);
+    if (max_index < (uint64_t(1) << 31) && !g_force_wide_index) f(uint32_t{}, grid);
     else f(uint64_t{}, grid);
 }
 

@@ -15,50 +15,114 @@
 
 namespace sigamd {
 
-// Adjoint of C = A (x) B (siglib/cpsig/cp_sig_combine.h:126-176).  One thread per coefficient r = (level t, word w):
+// Adjoint of C = A (x) B (siglib/cpsig/cp_sig_combine.h:126-176), scalar-free rows:
 //   dA_t[w] = dC_t[w] + sum_{m=1..N-t} sum_{v in d^m} dC_{t+m}[w v] * B_m[v]        (contiguous block of dC)
 //   dB_t[w] = dC_t[w] + sum_{k=1..N-t} sum_{u in d^k} dC_{t+k}[u w] * A_k[u]        (stride d^t in dC)
-// Scalar slots of both gradients are zero.
+// Both sums run over the first S_t = d + .. + d^(N-t) entries x of the other factor's row (its levels 1..N-t laid
+// end to end).  Outputs of low levels have long sums, so a sum is cut into parts of kCombChunk entries; a work
+// item is (family, level t, part, word w), words fastest.  Levels with one part are stored directly, the others
+// are set to dC by sig_combine_bwd_init_kernel first and receive their parts through atomics.
+constexpr int kCombChunk = 256;
+constexpr int kCombMaxLevels = 64;
+template <typename I>
+struct CombBwdPlan {
+    int degree;
+    I items;                            // work items of one family
+    I lo[kCombMaxLevels + 2];           // lo[t]: start of level t in a scalar-free row, t = 1 .. degree + 1
+    I item_start[kCombMaxLevels + 2];   // first work item of level t
+    I parts[kCombMaxLevels + 2];        // parts per word of level t (>= 1)
+    I init_len;                         // coefficients (a prefix of the row) whose levels have several parts
+};
+
+template <typename I>
+static CombBwdPlan<I> make_comb_plan(uint64_t d, uint64_t degree)
+{
+    CombBwdPlan<I> p{};
+    p.degree = int(degree);
+    uint64_t lo = 0, sz = d;
+    for (uint64_t t = 1; t <= degree + 1; ++t) {
+        p.lo[t] = I(lo);
+        lo += sz;
+        if (t <= degree) sz *= d;
+    }
+    uint64_t items = 0;
+    p.init_len = 0;
+    for (uint64_t t = 1; t <= degree; ++t) {
+        const uint64_t s_t = uint64_t(p.lo[degree - t + 1]);          // d + .. + d^(degree - t)
+        const uint64_t parts = s_t == 0 ? 1 : (s_t + kCombChunk - 1) / kCombChunk;
+        p.item_start[t] = I(items);
+        p.parts[t] = I(parts);
+        items += parts * (uint64_t(p.lo[t + 1]) - uint64_t(p.lo[t]));
+        if (parts > 1) p.init_len = p.lo[t + 1];
+    }
+    p.item_start[degree + 1] = I(items);
+    p.items = I(items);
+    return p;
+}
+
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void sig_combine_bwd_init_kernel(
+    const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, int64_t batch, I init_len, int64_t stride, int off)
+{
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < init_len; r += I(gridDim.x) * kBlock) {
+            const T v = dC[b * stride + off + r];
+            dA[b * stride + off + r] = v;
+            dB[b * stride + off + r] = v;
+        }
+    }
+}
+
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, const T* __restrict__ A,
-    const T* __restrict__ B, int64_t batch, I d, int degree, I sig_len, int64_t stride, int off)
+    const T* __restrict__ B, int64_t batch, CombBwdPlan<I> plan, int64_t stride, int off)
 {
+    const int N = plan.degree;
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* g = dC + b * stride + off;
-        const T* a = A + b * stride + off;
-        const T* bb = B + b * stride + off;
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T ga = g[r], gb = ga;
-            I up_lo = p.lo + p.size;      // start of level t + m in dC
-            I lo_m = 0, sz_m = d;         // level m of A / B
-            for (int m = 1; p.t + m <= degree; ++m) {
-                const T* blockp = g + up_lo + p.w * sz_m;        // words w v, v in d^m
-                T s0 = T(0), s1 = T(0);
-                I v = 0;
-                for (; v + 2 <= sz_m; v += 2) {
-                    s0 = fmadd(blockp[v], bb[lo_m + v], s0);
-                    s1 = fmadd(blockp[v + 1], bb[lo_m + v + 1], s1);
+        for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < 2 * plan.items; it += I(gridDim.x) * kBlock) {
+            const bool fam_b = it >= plan.items;
+            const I i2 = fam_b ? it - plan.items : it;
+            int t = 1;
+            while (t < N && i2 >= plan.item_start[t + 1]) ++t;
+            const I sz_t = plan.lo[t + 1] - plan.lo[t];
+            const I local = i2 - plan.item_start[t];
+            const I q = local / sz_t;
+            const I w = local - q * sz_t;
+            const I s_t = plan.lo[N - t + 1];
+            const I x0 = q * kCombChunk;
+            const I x1 = x0 + kCombChunk < s_t ? x0 + kCombChunk : s_t;
+            const T* other = (fam_b ? A : B) + b * stride + off;      // the factor the sum runs over
+            T s0 = T(0), s1 = T(0);
+            for (int m = 1; m <= N - t; ++m) {
+                const I seg0 = plan.lo[m] > x0 ? plan.lo[m] : x0;
+                const I seg1 = plan.lo[m + 1] < x1 ? plan.lo[m + 1] : x1;
+                if (seg0 >= seg1) continue;
+                const T* up = g + plan.lo[t + m];                     // level t + m of dC
+                if (!fam_b) {
+                    const T* blockp = up + w * (plan.lo[m + 1] - plan.lo[m]) - plan.lo[m];    // words w v
+                    I x = seg0;
+                    for (; x + 2 <= seg1; x += 2) {
+                        s0 = fmadd(blockp[x], other[x], s0);
+                        s1 = fmadd(blockp[x + 1], other[x + 1], s1);
+                    }
+                    if (x < seg1) s0 = fmadd(blockp[x], other[x], s0);
+                } else {
+                    const T* strided = up + w;                         // words u w: index u * d^t + w
+                    I x = seg0;
+                    for (; x + 2 <= seg1; x += 2) {
+                        s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
+                        s1 = fmadd(strided[(x + 1 - plan.lo[m]) * sz_t], other[x + 1], s1);
+                    }
+                    if (x < seg1) s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
                 }
-                for (; v < sz_m; ++v) s0 = fmadd(blockp[v], bb[lo_m + v], s0);
-                ga += s0 + s1;
-                const T* strided = g + up_lo + p.w;               // words u w, u in d^m: index u * d^t + w
-                T q0 = T(0), q1 = T(0);
-                I u = 0;
-                for (; u + 2 <= sz_m; u += 2) {
-                    q0 = fmadd(strided[u * p.size], a[lo_m + u], q0);
-                    q1 = fmadd(strided[(u + 1) * p.size], a[lo_m + u + 1], q1);
-                }
-                for (; u < sz_m; ++u) q0 = fmadd(strided[u * p.size], a[lo_m + u], q0);
-                gb += q0 + q1;
-                up_lo += p.size * sz_m;
-                lo_m += sz_m;
-                sz_m *= d;
             }
-            dA[b * stride + off + r] = ga;
-            dB[b * stride + off + r] = gb;
-            if (off && r == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
+            const I r = plan.lo[t] + w;
+            T* dst = (fam_b ? dB : dA) + b * stride + off + r;
+            if (plan.parts[t] == 1) *dst = g[r] + (s0 + s1);
+            else dev_add(dst, s0 + s1);
+            if (off && it == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
         }
     }
 }
@@ -219,15 +283,17 @@ constexpr int kExpAccMax = 4096;
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
     const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int64_t batch, DivBy<I> dv, I sig_len,
-    int64_t stride, int off, int use_lds)
+    int64_t stride, int off, int use_lds, int copies)
 {
     extern __shared__ double exp_lds_raw[];
     T* acc = reinterpret_cast<T*>(exp_lds_raw);
     const I d = I(dv.d);
+    // `copies` private sets of d accumulators, chosen by lane: few letters mean many lanes adding to one word
+    T* mine = acc + (threadIdx.x % copies) * d;
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         if (use_lds) {
             __syncthreads();
-            for (I j = threadIdx.x; j < d; j += kBlock) acc[j] = T(0);
+            for (I j = threadIdx.x; j < I(copies) * d; j += kBlock) acc[j] = T(0);
             __syncthreads();
         }
         const T* z = disp + b * int64_t(d);
@@ -250,14 +316,18 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
             T pre = T(1);
             for (int i = 0; i < p.t; ++i) {
                 const T c = pre * suf[i];
-                if (use_lds) lds_add_shared(&acc[let[i]], c);
+                if (use_lds) lds_add_shared(&mine[let[i]], c);
                 else dev_add(&out[let[i]], c);
                 pre *= z[let[i]];
             }
         }
         if (use_lds) {
             __syncthreads();
-            for (I j = threadIdx.x; j < d; j += kBlock) dev_add(&out[j], acc[j]);
+            for (I j = threadIdx.x; j < d; j += kBlock) {
+                T sum = T(0);
+                for (int c = 0; c < copies; ++c) sum += acc[I(c) * d + j];
+                dev_add(&out[j], sum);
+            }
         }
     }
 }
@@ -295,6 +365,27 @@ static SigShape sig_shape(uint64_t dimension, uint64_t degree, bool scalar_term,
     s.stride = scalar_term ? full : full - 1;
     s.off = scalar_term ? 1 : 0;
     return s;
+}
+
+// launches the adjoint of the Chen product (both kernels) on `stream`
+template <typename T>
+static void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint64_t batch, uint64_t dimension,
+                               uint64_t degree, const SigShape& s, hipStream_t stream)
+{
+    if (degree > uint64_t(kCombMaxLevels)) throw std::runtime_error("sig_combine_backprop_cuda: degree too high");
+    launch_indexed(3 * s.n_coef + 1024, 1, batch, [&](auto ix, dim3) {      // 2 * items <= 2 n (1 + degree / kCombChunk)
+        using I = decltype(ix);
+        const CombBwdPlan<I> plan = make_comb_plan<I>(dimension, degree);
+        if (plan.init_len > 0)
+            launch_indexed(0, uint64_t(plan.init_len), batch, [&](auto, dim3 grid) {
+                hipLaunchKernelGGL((sig_combine_bwd_init_kernel<T, I>), grid, dim3(kBlock), 0, stream, dC, dA, dB,
+                                   int64_t(batch), plan.init_len, int64_t(s.stride), s.off);
+            });
+        launch_indexed(0, 2 * uint64_t(plan.items), batch, [&](auto, dim3 grid) {
+            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, dC, dA, dB, A, B, int64_t(batch),
+                               plan, int64_t(s.stride), s.off);
+        });
+    });
 }
 
 template <typename T>
@@ -337,11 +428,7 @@ static void sig_combine_backprop_impl(const T* derivs, T* d1, T* d2, const T* si
             hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, d2, int64_t(batch));
         }
     } else {
-        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, derivs, d1, d2, sig1, sig2,
-                               int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
-        });
+        launch_combine_bwd<T>(derivs, d1, d2, sig1, sig2, batch, dimension, degree, s, stream);
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -420,25 +507,23 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
         using I = decltype(ix);
         hipLaunchKernelGGL((linear_sig_kernel<T, I>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
                            DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off);
-        // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
-        if (prepend)
-            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, d_out, dE, d_sig, (const T*)E,
-                               sig, int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
-        else
-            hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, d_out, d_sig, dE, sig,
-                               (const T*)E, int64_t(batch), I(dimension), int(degree), I(s.n_coef), int64_t(s.stride), s.off);
     });
+    // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
+    if (prepend) launch_combine_bwd<T>(d_out, dE, d_sig, (const T*)E, sig, batch, dimension, degree, s, stream);
+    else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream);
     if (dimension == 1) {
         hipLaunchKernelGGL((exp_pullback_dim_one_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, (const T*)dE, disp,
                            d_disp, int64_t(batch), int64_t(degree), int64_t(s.stride), s.off);
     } else {
         const int use_lds = dimension <= uint64_t(kExpAccMax);
+        const int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(32, uint64_t(kExpAccMax) / dimension))) : 1;
         // about 8 coefficients per thread, so that a block's LDS partial sums amortise their flush
         launch_indexed(s.n_coef, (s.n_coef + 7) / 8, batch, [&](auto ix, dim3 grid) {
             using I = decltype(ix);
-            hipLaunchKernelGGL((exp_pullback_kernel<T, I>), grid, dim3(kBlock), use_lds ? size_t(dimension) * sizeof(T) : 0,
-                               stream, (const T*)dE, disp, d_disp, int64_t(batch), DivBy<I>(dimension), I(s.n_coef),
-                               int64_t(s.stride), s.off, use_lds);
+            hipLaunchKernelGGL((exp_pullback_kernel<T, I>), grid, dim3(kBlock),
+                               use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp,
+                               d_disp, int64_t(batch), DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off, use_lds,
+                               copies);
         });
     }
     SIG_HIP(hipGetLastError());

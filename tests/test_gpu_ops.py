@@ -134,8 +134,9 @@ def test_combine_backprop_golden(P, fixtures, deg, dtype):
     np.testing.assert_allclose(d2.cpu().numpy()[:, 1:], fixtures["sig_comb_bp_d2__d%d" % deg], rtol=0, atol=atol)
     assert torch.all(d1[:, 0] == 0) and torch.all(d2[:, 0] == 0)
     one1, one2 = P.sig_combine_backprop(g[0], s1[0], s2[0], 3, deg)
-    np.testing.assert_array_equal(one1.cpu().numpy(), d1[0].cpu().numpy())
-    np.testing.assert_array_equal(one2.cpu().numpy(), d2[0].cpu().numpy())
+    # long sums are cut into parts that are added with atomics: equal up to the order of the additions
+    np.testing.assert_allclose(one1.cpu().numpy(), d1[0].cpu().numpy(), rtol=1e-6 if dtype == np.float32 else 1e-14, atol=atol * 1e-6)
+    np.testing.assert_allclose(one2.cpu().numpy(), d2[0].cpu().numpy(), rtol=1e-6 if dtype == np.float32 else 1e-14, atol=atol * 1e-6)
 
 
 @pytest.mark.parametrize("d,deg,batch", [(2, 5, 7), (5, 4, 33), (3, 1, 4), (1, 6, 3), (7, 3, 130), (10, 5, 32),
@@ -164,8 +165,8 @@ def test_combine_autograd(P):
     w = torch.rand((5, n), dtype=torch.float64, device=DEV)
     (P.torch_api.sig_combine(a, b, d, deg) * w).sum().backward()
     d1, d2 = P.sig_combine_backprop(w, a.detach(), b.detach(), d, deg)
-    np.testing.assert_array_equal(a.grad.cpu().numpy(), d1.cpu().numpy())
-    np.testing.assert_array_equal(b.grad.cpu().numpy(), d2.cpu().numpy())
+    np.testing.assert_allclose(a.grad.cpu().numpy(), d1.cpu().numpy(), rtol=1e-14, atol=1e-14)
+    np.testing.assert_allclose(b.grad.cpu().numpy(), d2.cpu().numpy(), rtol=1e-14, atol=1e-14)
     # directional derivative: <w, C(a + h u, b) - C(a - h u, b)> / 2h == <dA, u>  (the product is bilinear: exact up to rounding)
     u = torch.rand_like(w)
     h = 1e-3
@@ -311,7 +312,7 @@ def test_sig_join_extends_the_path_and_autograd(P, prepend):
     w = torch.rand_like(s)
     (P.torch_api.sig_join(sr, zr, d, deg, prepend=prepend) * w).sum().backward()
     ds, dz = P.sig_join_backprop(w, s, dev(z), d, deg, prepend=prepend)
-    np.testing.assert_array_equal(sr.grad.cpu().numpy(), ds.cpu().numpy())
+    np.testing.assert_allclose(sr.grad.cpu().numpy(), ds.cpu().numpy(), rtol=1e-14, atol=1e-14)
     # the displacement gradient is accumulated with atomics: equal up to the order of the additions
     np.testing.assert_allclose(zr.grad.cpu().numpy(), dz.cpu().numpy(), rtol=1e-13, atol=1e-13)
 
@@ -343,3 +344,48 @@ def test_join_linear_batch_shapes_and_errors(P, oracle):
         P.linear_sig(z, d + 1, deg)
     with pytest.raises(RuntimeError):
         P.linear_sig(z.cpu(), d, deg)
+
+
+def test_wide_index_arithmetic(P, oracle):
+    """The 64-bit index path of the coefficient-per-thread kernels (rows of 2^31 coefficients or more in production),
+    forced here on small shapes; also covers the time-segmented forward's Chen fold."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_wide_index.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_wide_index.restype = None
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_segments.restype = None
+    rng = np.random.default_rng(31)
+    d, deg, batch = 3, 6, 9
+    n = oracle.sig_length(d, deg) - 1
+    a, b, g = (rng.standard_normal((batch, n)) * 0.3 for _ in range(3))
+    z = rng.standard_normal((batch, d))
+    x = rng.uniform(size=(4, 9, 2))
+    L.CUSIG.cusig_amd_force_wide_index(1)
+    try:
+        np.testing.assert_allclose(P.sig_combine(dev(a), dev(b), d, deg).cpu().numpy(), oracle.sig_combine(a, b, d, deg),
+                                   rtol=1e-12, atol=1e-12)
+        d1, d2 = P.sig_combine_backprop(dev(g), dev(a), dev(b), d, deg)
+        w1, w2 = oracle.sig_combine_backprop(g, a, b, d, deg)
+        np.testing.assert_allclose(d1.cpu().numpy(), w1, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(d2.cpu().numpy(), w2, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(P.linear_sig(dev(z), d, deg).cpu().numpy(), oracle.linear_sig(z, d, deg), rtol=1e-12, atol=1e-12)
+        for prepend in (False, True):
+            np.testing.assert_allclose(P.sig_join(dev(a), dev(z), d, deg, prepend=prepend).cpu().numpy(),
+                                       oracle.sig_join(a, z, d, deg, prepend=prepend), rtol=1e-12, atol=1e-12)
+            ds, dz = P.sig_join_backprop(dev(g), dev(a), dev(z), d, deg, prepend=prepend)
+            ws, wz = oracle.sig_join_backprop(g, a, z, d, deg, prepend=prepend)
+            np.testing.assert_allclose(ds.cpu().numpy(), ws, rtol=1e-12, atol=1e-12)
+            np.testing.assert_allclose(dz.cpu().numpy(), wz, rtol=1e-11, atol=1e-11)
+        kw = dict(time_aug=True, lead_lag=True, end_time=2.0)
+        y = P.transform_path(dev(x), **kw)
+        np.testing.assert_allclose(y.cpu().numpy(), oracle.transform_path(x, **kw), rtol=0, atol=1e-14)
+        gy = rng.standard_normal(tuple(y.shape))
+        np.testing.assert_allclose(P.transform_path_backprop(dev(gy), **kw).cpu().numpy(),
+                                   oracle.transform_path_backprop(gy, 2, 9, time_aug=True, lead_lag=True), rtol=0, atol=1e-13)
+        L.CUSIG.cusig_amd_force_segments(3)
+        xs = rng.uniform(size=(2, 200, 3))
+        np.testing.assert_allclose(P.sig(dev(xs), 4).cpu().numpy(), oracle.signature(xs, 4), rtol=1e-10, atol=1e-12)
+    finally:
+        L.CUSIG.cusig_amd_force_segments(0)
+        L.CUSIG.cusig_amd_force_wide_index(0)
