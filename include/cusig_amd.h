@@ -132,6 +132,30 @@ CUSIG_AMD_API int sig_join_backprop_cuda_d(const double* d_out, double* d_sig, d
                                            const double* displacement, uint64_t batch_size, uint64_t dimension,
                                            uint64_t degree, bool prepend, bool scalar_term) CUSIG_AMD_NOEXCEPT;
 
+/* Coefficients of selected words.  multi_idx: the words' letters end to end, degrees: their lengths (both uint64, on
+ * the device); out [batch, num_multi_idx], or with `prefixes` per word the coefficients of all its non-empty
+ * prefixes (one entry, 1, for the empty word).  Augmentations are applied beforehand (transform_path_cuda).
+ * Replaces: sig_coef_cuda_{f,d} (decl siglib/cusig/cusig.h:468-470; arithmetic
+ * siglib/cpsig/cp_sig_coef_impl.cpp:35-84,138-348), bound by pysiglib/load_siglib.py (CUSIG_SIG_COEF), called from
+ * pysiglib/sig_coef.py. */
+CUSIG_AMD_API int sig_coef_cuda_f(const float* path, float* out, const uint64_t* multi_idx, uint64_t num_multi_idx,
+                                  const uint64_t* degrees, uint64_t batch_size, uint64_t dimension, uint64_t length,
+                                  bool prefixes) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_coef_cuda_d(const double* path, double* out, const uint64_t* multi_idx, uint64_t num_multi_idx,
+                                  const uint64_t* degrees, uint64_t batch_size, uint64_t dimension, uint64_t length,
+                                  bool prefixes) CUSIG_AMD_NOEXCEPT;
+
+/* Path gradient given dF/d(prefix coefficients); coefs and derivs have the `prefixes` layout of sig_coef_cuda.
+ * Replaces: sig_coef_backprop_cuda_{f,d} (decl siglib/cusig/cusig.h:492-494; arithmetic
+ * siglib/cpsig/cp_sig_coef_impl.cpp:360-485), bound by pysiglib/load_siglib.py (CUSIG_SIG_COEF_BACKPROP), called from
+ * pysiglib/sig_coef_backprop.py. */
+CUSIG_AMD_API int sig_coef_backprop_cuda_f(const float* path, float* out, const float* coefs, const float* derivs,
+                                           const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
+                                           uint64_t batch_size, uint64_t dimension, uint64_t length) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_coef_backprop_cuda_d(const double* path, double* out, const double* coefs, const double* derivs,
+                                           const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
+                                           uint64_t batch_size, uint64_t dimension, uint64_t length) CUSIG_AMD_NOEXCEPT;
+
 /* Message of the last failing call made by the calling thread ("" if none).
  * Replaces: cusig_last_error_message, probed by pysiglib/load_siglib.py:108-110
  * and read by pysiglib/error_codes.py:28-42. */

@@ -70,6 +70,19 @@ int sigref_sig_join_d(const double *sig, const double *displacement, double *out
 int sigref_sig_join_backprop_d(const double *dout, double *dsig, double *ddisplacement, const double *sig,
                                const double *displacement, uint64_t batch, uint64_t dimension, uint64_t degree,
                                int prepend, int scalar_term);
+/* sig_coef_{f,d}, sig_coef_backprop_{f,d} of the reference (siglib/cpsig/cpsig.h) without n_jobs. */
+int sigref_sig_coef_f(const float *path, float *out, const uint64_t *multi_idx, uint64_t num_multi_idx,
+                      const uint64_t *degrees, uint64_t batch, uint64_t dimension, uint64_t length, int time_aug,
+                      int lead_lag, float end_time, int prefixes);
+int sigref_sig_coef_backprop_f(const float *path, float *out, const float *coefs, const float *derivs,
+                               const uint64_t *multi_idx, uint64_t num_multi_idx, const uint64_t *degrees, uint64_t batch,
+                               uint64_t dimension, uint64_t length, int time_aug, int lead_lag, float end_time);
+int sigref_sig_coef_d(const double *path, double *out, const uint64_t *multi_idx, uint64_t num_multi_idx,
+                      const uint64_t *degrees, uint64_t batch, uint64_t dimension, uint64_t length, int time_aug,
+                      int lead_lag, double end_time, int prefixes);
+int sigref_sig_coef_backprop_d(const double *path, double *out, const double *coefs, const double *derivs,
+                               const uint64_t *multi_idx, uint64_t num_multi_idx, const uint64_t *degrees, uint64_t batch,
+                               uint64_t dimension, uint64_t length, int time_aug, int lead_lag, double end_time);
 #ifdef __cplusplus
 }
 #endif

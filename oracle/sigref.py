@@ -48,6 +48,13 @@ def _load():
         f = getattr(lib, "sigref_transform_path_backprop_" + suf)
         f.restype = i32
         f.argtypes = (ptr, ptr, u64, u64, u64, i32, i32)
+        pu = ctypes.POINTER(u64)
+        f = getattr(lib, "sigref_sig_coef_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, pu, u64, pu, u64, u64, u64, i32, i32, real, i32)
+        f = getattr(lib, "sigref_sig_coef_backprop_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, ptr, pu, u64, pu, u64, u64, u64, i32, i32, real)
         f = getattr(lib, "sigref_linear_sig_" + suf)
         f.restype = i32
         f.argtypes = (ptr, ptr, u64, u64, u64, i32)
@@ -243,3 +250,53 @@ def sig_join_backprop(derivs, sig, displacement, dimension, degree, prepend=Fals
     if rc:
         raise RuntimeError("sigref_sig_join_backprop returned %d" % rc)
     return dsig.reshape(sig.shape), dz.reshape(np.shape(displacement))
+
+
+def _words(words):
+    flat = np.array([i for w in words for i in w], dtype=np.uint64)
+    degs = np.array([len(w) for w in words], dtype=np.uint64)
+    if flat.size == 0:
+        flat = np.zeros(1, dtype=np.uint64)
+    return flat, degs
+
+
+def sig_coef(path, words, time_aug=False, lead_lag=False, end_time=1.0, prefixes=False):
+    """Oracle coefficients of the given words (list of tuples) for path (length, dim) or (batch, length, dim)."""
+    path = np.ascontiguousarray(path)
+    single = path.ndim == 2
+    if single:
+        path = path[None]
+    batch, length, dim = path.shape
+    suf, real = _suffix(path.dtype)
+    flat, degs = _words(words)
+    row = sum((max(len(w), 1) if prefixes else 1) for w in words)
+    out = np.empty((batch, row), dtype=path.dtype)
+    ptr, pu = ctypes.POINTER(real), ctypes.POINTER(ctypes.c_uint64)
+    rc = getattr(LIB, "sigref_sig_coef_" + suf)(path.ctypes.data_as(ptr), out.ctypes.data_as(ptr), flat.ctypes.data_as(pu),
+                                                len(words), degs.ctypes.data_as(pu), batch, dim, length, int(time_aug),
+                                                int(lead_lag), float(end_time), int(prefixes))
+    if rc:
+        raise RuntimeError("sigref_sig_coef returned %d" % rc)
+    return out[0] if single else out
+
+
+def sig_coef_backprop(path, words, coefs, derivs, time_aug=False, lead_lag=False, end_time=1.0):
+    """coefs / derivs in the prefixes=True layout."""
+    path = np.ascontiguousarray(path)
+    single = path.ndim == 2
+    if single:
+        path = path[None]
+    batch, length, dim = path.shape
+    suf, real = _suffix(path.dtype)
+    flat, degs = _words(words)
+    c = np.ascontiguousarray(coefs, dtype=path.dtype).reshape(batch, -1)
+    g = np.ascontiguousarray(derivs, dtype=path.dtype).reshape(batch, -1)
+    out = np.zeros_like(path)
+    ptr, pu = ctypes.POINTER(real), ctypes.POINTER(ctypes.c_uint64)
+    rc = getattr(LIB, "sigref_sig_coef_backprop_" + suf)(
+        path.ctypes.data_as(ptr), out.ctypes.data_as(ptr), c.ctypes.data_as(ptr), g.ctypes.data_as(ptr),
+        flat.ctypes.data_as(pu), len(words), degs.ctypes.data_as(pu), batch, dim, length, int(time_aug), int(lead_lag),
+        float(end_time))
+    if rc:
+        raise RuntimeError("sigref_sig_coef_backprop returned %d" % rc)
+    return out[0] if single else out

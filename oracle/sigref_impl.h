@@ -618,6 +618,161 @@ int FN(sigref_sig_join_backprop)(const REAL *dout, REAL *dsig, REAL *ddisp, cons
     return 0;
 }
 
+/* siglib/cpsig/cp_sig_coef_impl.cpp:35-84 single_sig_coef_: coefficients of the prefixes of ONE word, swept over the
+ * path with the per-word Horner step (:296-305):  c_i += z_{i-1} * (((1/i!) z_0 + c_1/(i-1)!) z_1 + ...). */
+static void FN(word_sweep)(const FN(vpath) *p, const uint64_t *word, uint64_t k, REAL *c /* k + 1 */, REAL *z /* k */,
+                           const REAL *inv_fact)
+{
+    c[0] = (REAL)1;
+    for (uint64_t i = 1; i <= k; ++i) c[i] = (REAL)0;
+    const REAL step = p->time_step;
+    REAL t_prev = (REAL)0;
+    for (uint64_t s = 0; s + 1 < p->len; ++s) {
+        const REAL t_next = t_prev + step;
+        for (uint64_t i = 0; i < k; ++i) z[i] = FN(vpath_at)(p, s + 1, word[i], t_next) - FN(vpath_at)(p, s, word[i], t_prev);
+        for (uint64_t i = k; i > 0; --i) {
+            REAL acc = inv_fact[i];
+            for (uint64_t j = 0; j + 1 < i; ++j) acc = acc * z[j] + c[j + 1] * inv_fact[i - j - 1];
+            c[i] += acc * z[i - 1];
+        }
+        t_prev = t_next;
+    }
+}
+
+/* siglib/cpsig/cp_sig_coef_impl.cpp:138-348 sig_coef_: out row = per word either its coefficient or, with prefixes,
+ * the coefficients of all its non-empty prefixes (the empty word yields one entry, 1). */
+int FN(sigref_sig_coef)(const REAL *path, REAL *out, const uint64_t *multi_idx, uint64_t num_words, const uint64_t *degrees,
+                        uint64_t batch, uint64_t d_raw, uint64_t len_raw, int time_aug, int lead_lag, REAL end_time,
+                        int prefixes)
+{
+    if (d_raw == 0) return 2;
+    FN(vpath) p0;
+    FN(vpath_init)(&p0, NULL, d_raw, len_raw ? len_raw : 1, time_aug, lead_lag, end_time);
+    uint64_t kmax = 0, total = 0, row = 0;
+    for (uint64_t w = 0; w < num_words; ++w) {
+        if (degrees[w] > kmax) kmax = degrees[w];
+        total += degrees[w];
+        row += prefixes ? (degrees[w] ? degrees[w] : 1) : 1;
+    }
+    if (len_raw == 0) {     /* no points: every non-empty word has coefficient 0 */
+        for (uint64_t b = 0; b < batch; ++b) {
+            REAL *o = out + b * row;
+            for (uint64_t w = 0; w < num_words; ++w) {
+                const uint64_t cnt = prefixes && degrees[w] ? degrees[w] : 1;
+                for (uint64_t i = 0; i < cnt; ++i) *o++ = degrees[w] ? (REAL)0 : (REAL)1;
+            }
+        }
+        return 0;
+    }
+    for (uint64_t i = 0; i < total; ++i) if (multi_idx[i] >= p0.d) return 2;
+    REAL *c = (REAL *)malloc((3 * kmax + 3) * sizeof(REAL));
+    if (!c) return 1;
+    REAL *z = c + kmax + 1, *inv_fact = z + kmax + 1;
+    inv_fact[0] = (REAL)1;
+    for (uint64_t i = 1; i <= kmax; ++i) inv_fact[i] = inv_fact[i - 1] / (REAL)i;
+    for (uint64_t b = 0; b < batch; ++b) {
+        FN(vpath) p;
+        FN(vpath_init)(&p, path + b * d_raw * len_raw, d_raw, len_raw, time_aug, lead_lag, end_time);
+        REAL *o = out + b * row;
+        const uint64_t *word = multi_idx;
+        for (uint64_t w = 0; w < num_words; ++w) {
+            const uint64_t k = degrees[w];
+            if (k == 0) { *o++ = (REAL)1; continue; }
+            FN(word_sweep)(&p, word, k, c, z, inv_fact);
+            if (prefixes) { for (uint64_t i = 1; i <= k; ++i) *o++ = c[i]; }
+            else *o++ = c[k];
+            word += k;
+        }
+    }
+    free(c);
+    return 0;
+}
+
+/* siglib/cpsig/cp_sig_coef_impl.cpp:360-485,546-664 sig_coef_backprop_: reverse sweep per word.  Per step the prefix
+ * coefficients are taken back one step with the increment negated (uncombine_coefs_), then the adjoint goes through the
+ * Horner step (backprop_horner_): `g` (dF/d prefix coefficients) is updated in place and the increment gradient of
+ * every letter is scattered to the two path points of the step.  coefs / derivs have the prefixes layout; words of
+ * degree 0 own one (ignored) entry. */
+int FN(sigref_sig_coef_backprop)(const REAL *path, REAL *out, const REAL *coefs, const REAL *derivs,
+                                 const uint64_t *multi_idx, uint64_t num_words, const uint64_t *degrees, uint64_t batch,
+                                 uint64_t d_raw, uint64_t len_raw, int time_aug, int lead_lag, REAL end_time)
+{
+    if (d_raw == 0) return 2;
+    FN(vpath) p0;
+    FN(vpath_init)(&p0, NULL, d_raw, len_raw, time_aug, lead_lag, end_time);
+    uint64_t kmax = 0, total = 0, row = 0;
+    for (uint64_t w = 0; w < num_words; ++w) {
+        if (degrees[w] > kmax) kmax = degrees[w];
+        total += degrees[w];
+        row += degrees[w] ? degrees[w] : 1;
+    }
+    if (len_raw == 0) return 0;
+    for (uint64_t i = 0; i < total; ++i) if (multi_idx[i] >= p0.d) return 2;
+    REAL *c = (REAL *)malloc((6 * kmax + 6) * sizeof(REAL));
+    REAL *dx = (REAL *)malloc((p0.len ? p0.len : 1) * p0.d * sizeof(REAL));      /* gradient w.r.t. the augmented path */
+    if (!c || !dx) { free(c); free(dx); return 1; }
+    REAL *z = c + kmax + 1, *inv_fact = z + kmax + 1, *g = inv_fact + kmax + 1, *st = g + kmax + 1, *dz = st + kmax + 1;
+    inv_fact[0] = (REAL)1;
+    for (uint64_t i = 1; i <= kmax; ++i) inv_fact[i] = inv_fact[i - 1] / (REAL)i;
+    for (uint64_t b = 0; b < batch; ++b) {
+        FN(vpath) p;
+        FN(vpath_init)(&p, path + b * d_raw * len_raw, d_raw, len_raw, time_aug, lead_lag, end_time);
+        for (uint64_t i = 0; i < p.len * p.d; ++i) dx[i] = (REAL)0;
+        const REAL step = p.time_step;
+        const uint64_t *word = multi_idx;
+        const REAL *crow = coefs + b * row, *grow = derivs + b * row;
+        for (uint64_t w = 0; w < num_words; ++w) {
+            const uint64_t k = degrees[w];
+            if (k == 0) { ++crow; ++grow; continue; }
+            c[0] = (REAL)1;
+            for (uint64_t i = 1; i <= k; ++i) { c[i] = crow[i - 1]; g[i] = grow[i - 1]; }
+            for (uint64_t s = p.len - 1; s >= 1; --s) {      /* step s-1 -> s */
+                const REAL t_next = (REAL)s * step, t_prev = (REAL)(s - 1) * step;
+                for (uint64_t i = 0; i < k; ++i) z[i] = FN(vpath_at)(&p, s, word[i], t_next) - FN(vpath_at)(&p, s - 1, word[i], t_prev);
+                /* coefficients before the step: multiply by exp(-z) */
+                for (uint64_t i = k; i > 0; --i) {
+                    REAL acc = (i & 1) ? -inv_fact[i] : inv_fact[i];
+                    for (uint64_t j = 0; j + 1 < i; ++j) {
+                        const uint64_t m = i - j - 1;
+                        acc = acc * z[j] + c[j + 1] * ((m & 1) ? -inv_fact[m] : inv_fact[m]);
+                    }
+                    c[i] += acc * z[i - 1];
+                }
+                for (uint64_t i = 0; i < k; ++i) dz[i] = (REAL)0;
+                for (uint64_t i = 1; i <= k; ++i) {
+                    st[0] = inv_fact[i];
+                    for (uint64_t j = 0; j + 1 < i; ++j) st[j + 1] = st[j] * z[j] + c[j + 1] * inv_fact[i - j - 1];
+                    const REAL gi = g[i];
+                    dz[i - 1] += gi * st[i - 1];
+                    REAL sd = gi * z[i - 1];
+                    for (uint64_t j = i - 1; j-- > 0;) {
+                        dz[j] += sd * st[j];
+                        g[j + 1] += sd * inv_fact[i - j - 1];
+                        sd *= z[j];
+                    }
+                }
+                for (uint64_t i = 0; i < k; ++i) {
+                    dx[s * p.d + word[i]] += dz[i];
+                    dx[(s - 1) * p.d + word[i]] -= dz[i];
+                }
+            }
+            word += k; crow += k; grow += k;
+        }
+        /* augmented-path gradient -> raw path gradient (adjoint of the augmentation) */
+        REAL *o = out + b * d_raw * len_raw;
+        for (uint64_t i = 0; i < len_raw; ++i)
+            for (uint64_t j = 0; j < d_raw; ++j) {
+                if (!lead_lag) { o[i * d_raw + j] = p.len ? dx[i * p.d + j] : (REAL)0; continue; }
+                REAL v = dx[(2 * i) * p.d + j] + dx[(2 * i) * p.d + d_raw + j];
+                if (i + 1 < len_raw) v += dx[(2 * i + 1) * p.d + j];
+                if (i >= 1) v += dx[(2 * i - 1) * p.d + d_raw + j];
+                o[i * d_raw + j] = v;
+            }
+    }
+    free(c); free(dx);
+    return 0;
+}
+
 #undef FN
 #undef CAT
 #undef CAT_

@@ -3,10 +3,12 @@
 Drop-in for ``pysiglib.sig`` / ``pysiglib.sig_backprop`` / ``pysiglib.torch_api.sig`` on GPU tensors.
 """
 from . import torch_api
+from .coef import extract_sig_coef, sig_coef, sig_coef_backprop, word_to_idx
 from .ops import (linear_sig, sig_combine, sig_combine_backprop, sig_join, sig_join_backprop, transform_path,
                   transform_path_backprop)
 from .sig import sig, sig_backprop, signature
 from .sig_length import sig_length
 
 __all__ = ["sig", "signature", "sig_backprop", "sig_length", "sig_combine", "sig_combine_backprop", "sig_join",
-           "sig_join_backprop", "linear_sig", "transform_path", "transform_path_backprop", "torch_api"]
+           "sig_join_backprop", "linear_sig", "transform_path", "transform_path_backprop", "sig_coef", "sig_coef_backprop",
+           "extract_sig_coef", "word_to_idx", "torch_api"]

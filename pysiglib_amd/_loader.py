@@ -81,6 +81,14 @@ CUSIG_SIG_JOIN_BACKPROP = _table("sig_join_backprop_cuda", lambda r: (
     POINTER(r), POINTER(r), POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool, c_bool))
 
 
+CUSIG_SIG_COEF = _table("sig_coef_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(c_uint64), c_uint64, POINTER(c_uint64), c_uint64, c_uint64, c_uint64, c_bool))
+
+CUSIG_SIG_COEF_BACKPROP = _table("sig_coef_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), POINTER(r), POINTER(c_uint64), c_uint64, POINTER(c_uint64), c_uint64, c_uint64,
+    c_uint64))
+
+
 def last_error_message():
     msg = CUSIG.cusig_last_error_message()
     return msg.decode("utf-8", errors="replace") if msg else ""

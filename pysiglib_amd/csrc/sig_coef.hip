@@ -1,0 +1,331 @@
+// Coefficients of selected words and their backward pass, behind the reference's entry points
+//   sig_coef_cuda_{f,d}, sig_coef_backprop_cuda_{f,d}   (decl siglib/cusig/cusig.h:450-494; arithmetic of
+//   siglib/cpsig/cp_sig_coef_impl.cpp:35-84,296-305 forward and :360-485 backward).
+// One lane sweeps the path for one (path, word) pair and keeps the word's prefix coefficients in registers: the
+// per-word Horner chain is the prefix chain of the signature sweep without a subtree below it.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <mutex>
+#include <vector>
+
+#include "../../include/cusig_amd.h"
+#include "sig_host.h"
+#include "sig_kernels.h"
+
+namespace sigamd {
+
+constexpr int kCoefMaxDegree = 64;
+// 1/i!, i = 0 .. 64, rounded the way the reference builds its table (each entry the previous one divided by i,
+// siglib/cpsig/cp_sig_coef_impl.cpp:186-191)
+__constant__ double kInvFact[kCoefMaxDegree + 1] = {
+    1.0, 1.0, 0.5, 0.16666666666666666, 0.041666666666666664, 0.008333333333333333, 0.001388888888888889,
+    0.0001984126984126984, 2.48015873015873e-05, 2.7557319223985893e-06, 2.7557319223985894e-07,
+    2.505210838544172e-08, 2.08767569878681e-09, 1.6059043836821616e-10, 1.1470745597729726e-11,
+    7.647163731819817e-13, 4.779477332387386e-14, 2.811457254345521e-15, 1.5619206968586228e-16,
+    8.220635246624331e-18, 4.1103176233121653e-19, 1.9572941063391263e-20, 8.896791392450574e-22,
+    3.868170170630684e-23, 1.6117375710961184e-24, 6.446950284384474e-26, 2.4795962632247976e-27,
+    9.183689863795547e-29, 3.2798892370698385e-30, 1.1309962886447718e-31, 3.769987628815906e-33,
+    1.2161250415535181e-34, 3.800390754854744e-36, 1.151633562077195e-37, 3.387157535521162e-39,
+    9.67759295863189e-41, 2.6882202662866363e-42, 7.265460179153071e-44, 1.911963205040282e-45,
+    4.902469756513544e-47, 1.2256174391283858e-48, 2.9893108271424046e-50, 7.117406731291439e-52,
+    1.6552108677421951e-53, 3.7618428812322616e-55, 8.359650847182803e-57, 1.817315401561479e-58,
+    3.8666285139605935e-60, 8.055476070751236e-62, 1.6439747083165788e-63, 3.2879494166331576e-65,
+    6.446959640457172e-67, 1.2397999308571486e-68, 2.3392451525606576e-70, 4.3319354677049213e-72,
+    7.876246304918039e-74, 1.4064725544496498e-75, 2.467495709560789e-77, 4.2543029475186016e-79,
+    7.210682961895935e-81, 1.2017804936493225e-82, 1.970131956802168e-84, 3.1776321883905935e-86,
+    5.043860616493006e-88, 7.881032213270321e-90};
+
+struct WordList {
+    const uint64_t* letters;     // all words end to end
+    const uint64_t* start;       // first letter of word w
+    const uint64_t* out_start;   // first output column of word w
+    const uint64_t* degree;
+    uint64_t count;
+};
+
+// c_i += z_{i-1} * (((1/i!) z_0 + c_1/(i-1)!) z_1 + ... + c_{i-1}/1!),  i = k .. 1  (descending: every read of a
+// shorter prefix still sees the value from before the step).  SIGN = -1 applies exp(-z) instead of exp(z).
+// UF: unroll factor of every loop over letters (KMAX + 1 = fully unrolled, the arrays live in registers; 1 = rolled
+// loops over arrays in scratch memory, for long words).
+template <typename T, int KMAX, int UF, int SIGN>
+__device__ __forceinline__ void word_step(T (&c)[KMAX + 1], const T (&z)[KMAX], int k)
+{
+#pragma unroll UF
+    for (int i = KMAX; i >= 1; --i) {
+        if (i <= k) {
+            T acc = T((SIGN < 0 && (i & 1)) ? -kInvFact[i] : kInvFact[i]);
+#pragma unroll UF
+            for (int j = 0; j + 1 < i; ++j) {
+                const int m = i - j - 1;
+                acc = fmadd(acc, z[j], c[j + 1] * T((SIGN < 0 && (m & 1)) ? -kInvFact[m] : kInvFact[m]));
+            }
+            c[i] = fmadd(acc, z[i - 1], c[i]);
+        }
+    }
+}
+
+template <typename T, int KMAX, int UF>
+__global__ __launch_bounds__(kBlock) void sig_coef_kernel(
+    const T* __restrict__ path, T* __restrict__ out, WordList words, int64_t batch, int64_t d, int64_t len, int64_t row,
+    int prefixes)
+{
+    const int64_t total = batch * int64_t(words.count);
+    for (int64_t item = int64_t(blockIdx.x) * kBlock + threadIdx.x; item < total; item += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = item / int64_t(words.count), w = item % int64_t(words.count);
+        const int k = int(words.degree[w]);
+        T* o = out + b * row + (prefixes ? int64_t(words.out_start[w]) : w);
+        if (k == 0) { o[0] = T(1); continue; }
+        if (k > KMAX) continue;     // the host picks KMAX >= the largest degree
+        int64_t let[KMAX];
+        T c[KMAX + 1], z[KMAX], prev[KMAX];
+        const T* x = path + b * len * d;
+#pragma unroll UF
+        for (int i = 0; i < KMAX; ++i) {
+            let[i] = i < k ? int64_t(words.letters[words.start[w] + i]) : 0;
+            prev[i] = len > 0 ? x[let[i]] : T(0);
+            c[i + 1] = T(0);
+        }
+        c[0] = T(1);
+        for (int64_t s = 1; s < len; ++s) {
+            const T* xs = x + s * d;
+#pragma unroll UF
+            for (int i = 0; i < KMAX; ++i) {
+                const T cur = xs[let[i]];
+                z[i] = cur - prev[i];
+                prev[i] = cur;
+            }
+            word_step<T, KMAX, UF, 1>(c, z, k);
+        }
+        if (prefixes) {
+#pragma unroll UF
+            for (int i = 1; i <= KMAX; ++i)
+                if (i <= k) o[i - 1] = c[i];
+        } else {
+            T last = c[1];
+#pragma unroll UF
+            for (int i = 2; i <= KMAX; ++i)
+                if (i == k) last = c[i];
+            o[0] = last;
+        }
+    }
+}
+
+// Reverse sweep of one (path, word) pair: coefficients before the step by exp(-z), then the adjoint of the step:
+// with st_j = ((1/i!) z_0 + c_1/(i-1)!) z_1 + ... (the Horner values of prefix length i),
+//   dz_{i-1} += g_i st_{i-1};  walking j = i-2 .. 0 with sd = g_i z_{i-1} z_{i-2} ..:  dz_j += sd st_j,
+//   g_{j+1} += sd / (i-j-1)!.   The increment gradient goes to the two path points of the step with atomics
+// (several words, and several letters of one word, share path entries); `out` is zeroed beforehand.
+template <typename T, int KMAX, int UF>
+__global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
+    const T* __restrict__ path, T* __restrict__ out, const T* __restrict__ coefs, const T* __restrict__ derivs,
+    WordList words, int64_t batch, int64_t d, int64_t len, int64_t row)
+{
+    const int64_t total = batch * int64_t(words.count);
+    for (int64_t item = int64_t(blockIdx.x) * kBlock + threadIdx.x; item < total; item += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = item / int64_t(words.count), w = item % int64_t(words.count);
+        const int k = int(words.degree[w]);
+        if (k == 0 || k > KMAX || len < 2) continue;
+        int64_t let[KMAX];
+        T c[KMAX + 1], g[KMAX + 1], z[KMAX], next[KMAX], st[KMAX], dz[KMAX];
+        const T* x = path + b * len * d;
+        T* gx = out + b * len * d;
+        const T* crow = coefs + b * row + int64_t(words.out_start[w]);
+        const T* grow = derivs + b * row + int64_t(words.out_start[w]);
+        c[0] = T(1);
+        g[0] = T(0);
+#pragma unroll UF
+        for (int i = 0; i < KMAX; ++i) {
+            let[i] = i < k ? int64_t(words.letters[words.start[w] + i]) : 0;
+            next[i] = x[(len - 1) * d + let[i]];
+            c[i + 1] = i < k ? crow[i] : T(0);
+            g[i + 1] = i < k ? grow[i] : T(0);
+        }
+        for (int64_t s = len - 1; s >= 1; --s) {        // step s-1 -> s
+            const T* xp = x + (s - 1) * d;
+#pragma unroll UF
+            for (int i = 0; i < KMAX; ++i) {
+                const T cur = xp[let[i]];
+                z[i] = next[i] - cur;
+                next[i] = cur;
+            }
+            word_step<T, KMAX, UF, -1>(c, z, k);
+#pragma unroll UF
+            for (int i = 0; i < KMAX; ++i) dz[i] = T(0);
+#pragma unroll UF
+            for (int i = 1; i <= KMAX; ++i) {
+                if (i <= k) {
+                    st[0] = T(kInvFact[i]);
+#pragma unroll UF
+                    for (int j = 0; j + 1 < i; ++j) st[j + 1] = fmadd(st[j], z[j], c[j + 1] * T(kInvFact[i - j - 1]));
+                    const T gi = g[i];
+                    dz[i - 1] = fmadd(gi, st[i - 1], dz[i - 1]);
+                    T sd = gi * z[i - 1];
+#pragma unroll UF
+                    for (int j = i - 2; j >= 0; --j) {
+                        dz[j] = fmadd(sd, st[j], dz[j]);
+                        g[j + 1] = fmadd(sd, T(kInvFact[i - j - 1]), g[j + 1]);
+                        sd *= z[j];
+                    }
+                }
+            }
+#pragma unroll UF
+            for (int i = 0; i < KMAX; ++i) {
+                if (i < k) {
+                    dev_add(&gx[s * d + let[i]], dz[i]);
+                    dev_add(&gx[(s - 1) * d + let[i]], -dz[i]);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct HostWords {
+    std::vector<uint64_t> table;     // [start | out_start | degree], count entries each
+    uint64_t count = 0, row = 0, max_degree = 0, letters = 0;
+};
+
+// copies the word list to the host, validates it and lays out the per-word offsets
+static HostWords read_words(const uint64_t* multi_idx, uint64_t num_words, const uint64_t* degrees, uint64_t dimension,
+                            bool prefix_layout, const char* who)
+{
+    HostWords h;
+    h.count = num_words;
+    if (num_words == 0) return h;
+    if (!degrees) throw std::invalid_argument(std::string(who) + ": degrees is null");
+    std::vector<uint64_t> deg(num_words);
+    SIG_HIP(hipMemcpy(deg.data(), degrees, num_words * sizeof(uint64_t), hipMemcpyDeviceToHost));
+    h.table.resize(3 * num_words);
+    for (uint64_t w = 0; w < num_words; ++w) {
+        h.table[w] = h.letters;
+        h.table[num_words + w] = h.row;
+        h.table[2 * num_words + w] = deg[w];
+        h.letters = checked_mul(1, h.letters + deg[w], who);
+        h.row += prefix_layout ? (deg[w] ? deg[w] : 1) : 1;
+        h.max_degree = std::max(h.max_degree, deg[w]);
+    }
+    if (h.letters) {
+        if (!multi_idx) throw std::invalid_argument(std::string(who) + ": multi_idx is null");
+        std::vector<uint64_t> let(h.letters);
+        SIG_HIP(hipMemcpy(let.data(), multi_idx, h.letters * sizeof(uint64_t), hipMemcpyDeviceToHost));
+        for (uint64_t v : let)
+            if (v >= dimension) throw std::invalid_argument(std::string(who) + ": multi_idx element out of range");
+    }
+    if (h.max_degree > uint64_t(kCoefMaxDegree))
+        throw std::runtime_error(std::string(who) + ": words longer than 64 letters are not implemented in this build");
+    return h;
+}
+
+template <typename F>
+static void with_degree_bucket(uint64_t max_degree, F&& f)
+{
+    // (largest word length served, unroll factor)
+    if (max_degree <= 4) f(IntC<4>{}, IntC<5>{});
+    else if (max_degree <= 8) f(IntC<8>{}, IntC<9>{});
+    else if (max_degree <= 16) f(IntC<16>{}, IntC<17>{});
+    else f(IntC<kCoefMaxDegree>{}, IntC<1>{});
+}
+
+static WordList upload_words(const HostWords& h, const uint64_t* multi_idx, hipStream_t stream)
+{
+    uint64_t* dev = static_cast<uint64_t*>(workspace(6, h.table.size() * sizeof(uint64_t)));
+    SIG_HIP(hipMemcpyAsync(dev, h.table.data(), h.table.size() * sizeof(uint64_t), hipMemcpyHostToDevice, stream));
+    SIG_HIP(hipStreamSynchronize(stream));       // the host vector may go away once the caller returns
+    return WordList{multi_idx, dev, dev + h.count, dev + 2 * h.count, h.count};
+}
+
+template <typename T>
+static void sig_coef_impl(const T* path, T* out, const uint64_t* multi_idx, uint64_t num_words, const uint64_t* degrees,
+                          uint64_t batch, uint64_t dimension, uint64_t length, bool prefixes)
+{
+    if (dimension == 0) throw std::invalid_argument("sig_coef received path of dimension 0");
+    if (dimension > 0x3fffffff || length > (uint64_t(1) << 40)) throw std::invalid_argument("sig_coef_cuda: shape out of range");
+    SIG_HIP(hipDeviceSynchronize());
+    const HostWords h = read_words(multi_idx, num_words, degrees, dimension, true, "sig_coef");
+    if (batch == 0 || num_words == 0) return;
+    const uint64_t row = prefixes ? h.row : num_words;
+    checked_mul(checked_mul(batch, row, "coefficients"), sizeof(T), "coefficients");
+    checked_mul(checked_mul(checked_mul(batch, length, "path"), dimension, "path"), sizeof(T), "path");
+    const uint64_t items = checked_mul(batch, num_words, "work items");
+    hipStream_t stream = nullptr;
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    const WordList words = upload_words(h, multi_idx, stream);
+    with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
+        constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;
+        hipLaunchKernelGGL((sig_coef_kernel<T, KMAX, UF>), dim3(grid_for(items)), dim3(kBlock), 0, stream, path, out, words,
+                           int64_t(batch), int64_t(dimension), int64_t(length), int64_t(row), int(prefixes));
+    });
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+template <typename T>
+static void sig_coef_backprop_impl(const T* path, T* out, const T* coefs, const T* derivs, const uint64_t* multi_idx,
+                                   uint64_t num_words, const uint64_t* degrees, uint64_t batch, uint64_t dimension,
+                                   uint64_t length)
+{
+    if (dimension == 0) throw std::invalid_argument("sig_coef_backprop received path of dimension 0");
+    if (dimension > 0x3fffffff || length > (uint64_t(1) << 40)) throw std::invalid_argument("sig_coef_backprop_cuda: shape out of range");
+    SIG_HIP(hipDeviceSynchronize());
+    const HostWords h = read_words(multi_idx, num_words, degrees, dimension, true, "sig_coef_backprop");
+    const uint64_t path_elems = checked_mul(checked_mul(batch, length, "path"), dimension, "path");
+    checked_mul(path_elems, sizeof(T), "path");
+    if (path_elems == 0) return;
+    hipStream_t stream = nullptr;
+    hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(path_elems)), dim3(kBlock), 0, stream, out, int64_t(path_elems));
+    if (num_words > 0 && length >= 2 && h.max_degree > 0) {
+        const uint64_t items = checked_mul(batch, num_words, "work items");
+        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        const WordList words = upload_words(h, multi_idx, stream);
+        with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
+            constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;
+            hipLaunchKernelGGL((sig_coef_bwd_kernel<T, KMAX, UF>), dim3(grid_for(items)), dim3(kBlock), 0, stream, path, out, coefs,
+                               derivs, words, int64_t(batch), int64_t(dimension), int64_t(length), int64_t(h.row));
+        });
+        SIG_HIP(hipGetLastError());
+        SIG_HIP(hipStreamSynchronize(stream));
+        return;
+    }
+    SIG_HIP(hipGetLastError());
+    SIG_HIP(hipStreamSynchronize(stream));
+}
+
+}  // namespace sigamd
+
+using namespace sigamd;
+
+extern "C" {
+
+CUSIG_AMD_API int sig_coef_cuda_f(const float* path, float* out, const uint64_t* multi_idx, uint64_t num_multi_idx,
+                                  const uint64_t* degrees, uint64_t batch_size, uint64_t dimension, uint64_t length,
+                                  bool prefixes) noexcept
+{
+    return guarded([&] { sig_coef_impl<float>(path, out, multi_idx, num_multi_idx, degrees, batch_size, dimension, length, prefixes); });
+}
+CUSIG_AMD_API int sig_coef_cuda_d(const double* path, double* out, const uint64_t* multi_idx, uint64_t num_multi_idx,
+                                  const uint64_t* degrees, uint64_t batch_size, uint64_t dimension, uint64_t length,
+                                  bool prefixes) noexcept
+{
+    return guarded([&] { sig_coef_impl<double>(path, out, multi_idx, num_multi_idx, degrees, batch_size, dimension, length, prefixes); });
+}
+CUSIG_AMD_API int sig_coef_backprop_cuda_f(const float* path, float* out, const float* coefs, const float* derivs,
+                                           const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
+                                           uint64_t batch_size, uint64_t dimension, uint64_t length) noexcept
+{
+    return guarded([&] {
+        sig_coef_backprop_impl<float>(path, out, coefs, derivs, multi_idx, num_multi_idx, degrees, batch_size, dimension, length);
+    });
+}
+CUSIG_AMD_API int sig_coef_backprop_cuda_d(const double* path, double* out, const double* coefs, const double* derivs,
+                                           const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
+                                           uint64_t batch_size, uint64_t dimension, uint64_t length) noexcept
+{
+    return guarded([&] {
+        sig_coef_backprop_impl<double>(path, out, coefs, derivs, multi_idx, num_multi_idx, degrees, batch_size, dimension, length);
+    });
+}
+
+}  // extern "C"

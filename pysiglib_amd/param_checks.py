@@ -62,3 +62,29 @@ def own_contiguous(arr):
             return np.ascontiguousarray(arr.copy())
         return arr
     raise TypeError("expected a numpy.ndarray or torch.Tensor")
+
+
+def check_word(word, max_val, word_name):
+    """A word is a tuple of integer letters in [0, max_val) (pysiglib/param_checks.py:124-133)."""
+    if not isinstance(word, tuple):
+        raise TypeError(word_name + " must be a tuple of integers.")
+    for i in word:
+        if not isinstance(i, int):
+            raise TypeError(word_name + " must be a tuple of integers. Found element of type " + str(type(i)) + " instead.")
+        if not 0 <= i < max_val:
+            raise ValueError(word_name + " must only contain letters in the range [0, " + str(max_val) + ")")
+
+
+def check_word_or_word_list(param, max_val, param_name):
+    """Returns the words as a list (pysiglib/param_checks.py:135-153)."""
+    try:
+        if isinstance(param, tuple):
+            check_word(param, max_val, param_name)
+            return [param]
+        if isinstance(param, list):
+            for word in param:
+                check_word(word, max_val, "Every word in " + param_name)
+            return param
+    except Exception as e:
+        raise type(e)("Error processing words: " + str(e)) from e
+    raise TypeError(param_name + " must be a tuple of integers or a list of tuples of integers.")

@@ -96,3 +96,35 @@ class SigJoin(torch.autograd.Function):
 def sig_join(sig, displacement, dimension, degree, *, prepend=False, n_jobs=1):
     """Differentiable ``sig_join``."""
     return SigJoin.apply(sig, displacement, dimension, degree, bool(prepend))
+
+
+class SigCoef(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, path, words, time_aug, lead_lag, end_time):
+        from .coef import sig_coef as _coef
+        coefs = _coef(path, words, time_aug=time_aug, lead_lag=lead_lag, end_time=end_time, prefixes=True)
+        ctx.save_for_backward(coefs, path)
+        ctx.args = (words, time_aug, lead_lag, end_time)
+        return coefs
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .coef import sig_coef_backprop as _coef_backprop
+        coefs, path = ctx.saved_tensors
+        words, time_aug, lead_lag, end_time = ctx.args
+        grad = _coef_backprop(path, words, coefs, grad_output, time_aug=time_aug, lead_lag=lead_lag, end_time=end_time)
+        return grad, None, None, None, None
+
+
+def sig_coef(path, words, *, time_aug=False, lead_lag=False, end_time=1., prefixes=False, n_jobs=1):
+    """Differentiable ``sig_coef``: computes the prefixes layout and, without ``prefixes``, keeps each word's last
+    entry (pysiglib/torch_api/torch_api.py:156-202)."""
+    coefs = SigCoef.apply(path, words, time_aug, lead_lag, end_time)
+    if prefixes:
+        return coefs
+    word_list = [words] if isinstance(words, tuple) else words
+    ends, pos = [], 0
+    for w in word_list:
+        pos += max(len(w), 1)
+        ends.append(pos - 1)
+    return coefs[..., ends].contiguous()

@@ -389,3 +389,120 @@ def test_wide_index_arithmetic(P, oracle):
     finally:
         L.CUSIG.cusig_amd_force_segments(0)
         L.CUSIG.cusig_amd_force_wide_index(0)
+
+
+# ---------------------------------------------------------------------------
+# sig_coef / sig_coef_backprop
+# ---------------------------------------------------------------------------
+def _all_words(d, degree):
+    import itertools
+    return [w for k in range(1, degree + 1) for w in itertools.product(range(d), repeat=k)]
+
+
+def test_sig_coef_trivial_cases(P):
+    x = torch.tensor([[0., 0.], [1., 1.]], device=DEV)
+    np.testing.assert_array_equal(P.sig_coef(x, [(0,), (1,)]).cpu().numpy(), [1., 1.])
+    np.testing.assert_array_equal(P.sig_coef(x[None], [(0,), (1,)]).cpu().numpy(), [[1., 1.]])
+    np.testing.assert_array_equal(P.sig_coef(x[:1], [(0,), (1,)]).cpu().numpy(), [0., 0.])
+    np.testing.assert_array_equal(P.sig_coef(x, [(), (0, 1)], prefixes=True).cpu().numpy(), [1., 1., 0.5])
+    np.testing.assert_array_equal(P.sig_coef(x, (1, 0)).cpu().numpy(), [0.5])
+
+
+@pytest.mark.parametrize("aug", [{}, dict(time_aug=True, end_time=1.5), dict(lead_lag=True), dict(time_aug=True, lead_lag=True)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("shape", [(3, 15, 2), (70, 40, 3), (1, 2, 5)])
+def test_sig_coef_vs_oracle(P, oracle, aug, dtype, shape):
+    rng = np.random.default_rng(shape[0] + shape[1])
+    x = rng.uniform(size=shape).astype(dtype)
+    d = shape[2]
+    da = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    words = [(da - 1,), (0, da - 1), (1, 0, 1, da - 1), (), (da - 1, da - 1, 0), (0, 0), (0, 1, 0, 1, 0, 1, 1),
+             tuple(i % da for i in range(12)), tuple((3 * i + 1) % da for i in range(20))]
+    for prefixes in (False, True):
+        want = oracle.sig_coef(x, words, prefixes=prefixes, **aug)
+        got = P.sig_coef(dev(x), words, prefixes=prefixes, **aug).cpu().numpy()
+        assert got.shape == want.shape and got.dtype == dtype
+        if dtype == np.float64:
+            np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-13)
+        else:       # tiny high-degree coefficients cancel in float32: measured against the largest entry of the row
+            assert bwd_err(got, want) < TOL[dtype]
+    cp = oracle.sig_coef(x, words, prefixes=True, **aug)
+    g = rng.standard_normal(cp.shape).astype(dtype)
+    want = oracle.sig_coef_backprop(x, words, cp, g, **aug)
+    got = P.sig_coef_backprop(dev(x), words, dev(cp), dev(g), **aug).cpu().numpy()
+    assert got.shape == x.shape
+    assert bwd_err(got, want) < TOL[dtype]
+
+
+def bwd_err(got, ref):
+    got = got.reshape(ref.shape[0], -1).astype(np.float64)
+    ref = ref.reshape(ref.shape[0], -1).astype(np.float64)
+    den = np.maximum(np.abs(ref).max(axis=1), np.finfo(np.float64).tiny)
+    return float((np.abs(got - ref).max(axis=1) / den).max())
+
+
+@pytest.mark.parametrize("kw", [{}, dict(time_aug=True), dict(lead_lag=True), dict(time_aug=True, lead_lag=True)])
+def test_sig_coef_full_word_set_is_the_signature(P, kw):
+    # the reference's own test of sig_coef (tests/test_sig_coef.py:114-163)
+    rng = np.random.default_rng(3)
+    x = dev(rng.uniform(size=(10, 100, 2)))
+    da = (4 if kw.get("lead_lag") else 2) + (1 if kw.get("time_aug") else 0)
+    deg = 4
+    words = _all_words(da, deg)
+    sig = P.sig(x, deg, **kw)
+    np.testing.assert_allclose(P.sig_coef(x, words, **kw).cpu().numpy(), sig.cpu().numpy(), rtol=1e-10, atol=1e-13)
+    np.testing.assert_array_equal(P.extract_sig_coef(sig, words, 2, **kw).cpu().numpy(), sig.cpu().numpy())
+    one = P.extract_sig_coef(P.sig(x, deg, scalar_term=True, **kw), [(da - 1, 0)], 2, scalar_term=True, **kw)
+    np.testing.assert_array_equal(one.cpu().numpy()[:, 0], sig.cpu().numpy()[:, P.word_to_idx((da - 1, 0), da, deg)])
+
+
+def test_sig_coef_autograd_and_batch_shapes(P, oracle):
+    rng = np.random.default_rng(12)
+    words = [(2, 0, 1), (1, 1), (), (0,)]
+    x = dev(rng.uniform(size=(2, 3, 9, 3)))
+    xr = x.clone().requires_grad_(True)
+    out = P.torch_api.sig_coef(xr, words, time_aug=True, end_time=0.5)
+    assert out.shape == (2, 3, 4)
+    w = torch.rand_like(out)
+    (out * w).sum().backward()
+    # gradient of the selected coefficients == backprop with the weight on each word's last prefix
+    cp = P.sig_coef(x, words, prefixes=True, time_aug=True, end_time=0.5)
+    assert cp.shape == (2, 3, 7)
+    g = torch.zeros_like(cp)
+    g[..., [2, 4, 5, 6]] = w
+    want = oracle.sig_coef_backprop(x.cpu().numpy().reshape(6, 9, 3), words, cp.cpu().numpy().reshape(6, 7),
+                                    g.cpu().numpy().reshape(6, 7), time_aug=True, end_time=0.5)
+    np.testing.assert_allclose(xr.grad.cpu().numpy().reshape(6, 9, 3), want, rtol=1e-11, atol=1e-12)
+    pre = P.torch_api.sig_coef(x, words, prefixes=True, time_aug=True, end_time=0.5)
+    np.testing.assert_array_equal(pre.cpu().numpy(), cp.cpu().numpy())
+    assert P.sig_coef(x[0, 0], (0, 1)).shape == (1,)
+    empty = torch.empty((0, 9, 3), dtype=torch.float64, device=DEV)
+    assert P.sig_coef(empty, words).shape == (0, 4)
+    assert P.sig_coef_backprop(empty, words, torch.empty((0, 7), dtype=torch.float64, device=DEV),
+                               torch.empty((0, 7), dtype=torch.float64, device=DEV)).shape == (0, 9, 3)
+    with pytest.raises(ValueError):
+        P.sig_coef(x, [(3,)])
+    with pytest.raises(ValueError):
+        P.sig_coef(x, [])
+    with pytest.raises(TypeError):
+        P.sig_coef(x, [[0, 1]])
+    with pytest.raises(ValueError):
+        P.sig_coef_backprop(x, words, cp[..., :-1], g[..., :-1])
+    with pytest.raises(RuntimeError):
+        P.sig_coef(x.cpu(), words)
+    with pytest.raises(Exception, match="not implemented"):
+        P.sig_coef(x, [(0,) * 65])
+
+
+def test_sig_coef_abi_rejects_bad_letters(P):
+    import ctypes
+    from pysiglib_amd import _loader as L
+    x = torch.rand((2, 5, 3), dtype=torch.float64, device=DEV)
+    out = torch.empty((2, 1), dtype=torch.float64, device=DEV)
+    letters = torch.tensor([0, 3], dtype=torch.int64, device=DEV)       # 3 is out of range for 3 channels
+    degrees = torch.tensor([2], dtype=torch.int64, device=DEV)
+    pd = lambda t: ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_double))
+    pu = lambda t: ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_uint64))
+    assert L.CUSIG_SIG_COEF["float64"](pd(x), pd(out), pu(letters), 1, pu(degrees), 2, 3, 5, False) == 2
+    assert "out of range" in L.last_error_message()
+    assert L.CUSIG_SIG_COEF["float64"](pd(x), pd(out), pu(letters), 1, pu(degrees), 2, 0, 5, False) == 2

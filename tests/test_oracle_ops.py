@@ -245,3 +245,110 @@ def test_sig_join_backprop_finite_differences():
         zm[:, j] -= h
         num = ((sigref.sig_join(s, zp, d, deg) - sigref.sig_join(s, zm, d, deg)) * g).sum(axis=1) / (2 * h)
         np.testing.assert_allclose(dz[:, j], num, rtol=1e-6, atol=1e-7)
+
+
+# ---------------------------------------------------------------------------
+# sig_coef / sig_coef_backprop: pinned by the (already pinned) signature and its backward pass, which is also how the
+# reference tests them (tests/test_sig_coef.py:46-55, tests/test_sig_coef_backprop.py), by the reference's trivial
+# cases (tests/test_sig_coef.py:58-80) and by autograd through the independent Chen product.
+# ---------------------------------------------------------------------------
+def _widx(word, d):
+    idx = 0
+    for letter in word:
+        idx = idx * d + letter + 1
+    return idx - 1
+
+
+def _all_words(d, degree):
+    import itertools
+    return [w for k in range(1, degree + 1) for w in itertools.product(range(d), repeat=k)]
+
+
+COEF_AUGS = [{}, dict(time_aug=True, end_time=1.5), dict(lead_lag=True), dict(time_aug=True, lead_lag=True)]
+
+
+def test_sig_coef_trivial_cases():
+    x = np.array([[0., 0.], [1., 1.]])
+    np.testing.assert_array_equal(sigref.sig_coef(x, [(0,), (1,)]), [1., 1.])
+    np.testing.assert_array_equal(sigref.sig_coef(x[None], [(0,), (1,)]), [[1., 1.]])
+    np.testing.assert_array_equal(sigref.sig_coef(x[:1], [(0,), (1,)]), [0., 0.])
+    np.testing.assert_array_equal(sigref.sig_coef(x, [(), (0, 1)]), [1., 0.5])
+    np.testing.assert_array_equal(sigref.sig_coef(x, [(), (0, 1)], prefixes=True), [1., 1., 0.5])
+
+
+@pytest.mark.parametrize("aug", COEF_AUGS)
+@pytest.mark.parametrize("dtype,tol", [(np.float64, 1e-12), (np.float32, 1e-4)])
+def test_sig_coef_equals_signature_entries(aug, dtype, tol):
+    rng = np.random.default_rng(21)
+    d, deg = 2, 4
+    x = rng.uniform(size=(3, 15, d)).astype(dtype)
+    da = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    s = sigref.signature(x, deg, **aug)
+    every = _all_words(da, 3)
+    got = sigref.sig_coef(x, every, **aug)
+    assert got.dtype == dtype
+    np.testing.assert_allclose(got, s[:, :len(every)], rtol=tol, atol=tol)
+    words = [(da - 1,), (0, da - 1), (1, 0, 1, da - 1), (da - 1, da - 1, 0), ()]
+    got = sigref.sig_coef(x, words, **aug)
+    want = np.stack([s[:, _widx(w, da)] if w else np.ones(3) for w in words], axis=1)
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
+    pre = [w[:i] for w in words for i in range(1, len(w) + 1)] 
+    gotp = sigref.sig_coef(x, words, prefixes=True, **aug)
+    wantp = np.concatenate([np.stack([s[:, _widx(w[:i], da)] for i in range(1, len(w) + 1)], axis=1) if w else np.ones((3, 1))
+                            for w in words], axis=1)
+    assert gotp.shape == (3, len(pre) + 1)
+    np.testing.assert_allclose(gotp, wantp, rtol=tol, atol=tol)
+
+
+def test_sig_coef_long_word_closed_form():
+    # one channel: the coefficient of the word (0,)*k is (x_end - x_0)^k / k!
+    rng = np.random.default_rng(2)
+    x = np.cumsum(rng.uniform(0.1, 0.3, size=(2, 9, 1)), axis=1)
+    k = 24
+    got = sigref.sig_coef(x, [(0,) * k], prefixes=True)
+    inc = x[:, -1, 0] - x[:, 0, 0]
+    fact = np.cumprod(np.arange(1, k + 1, dtype=np.float64))
+    np.testing.assert_allclose(got, inc[:, None] ** np.arange(1, k + 1) / fact, rtol=1e-12, atol=0)
+
+
+@pytest.mark.parametrize("aug", COEF_AUGS)
+def test_sig_coef_backprop_equals_signature_backprop(aug):
+    rng = np.random.default_rng(33)
+    d, deg = 2, 4
+    x = rng.uniform(size=(3, 8, d))
+    da = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    words = [(da - 1,), (0, da - 1), (1, 0, 1, da - 1), (), (da - 1, da - 1, 0), (0, 0)]
+    cp = sigref.sig_coef(x, words, prefixes=True, **aug)
+    g = rng.standard_normal(cp.shape)
+    s = sigref.signature(x, deg, **aug)
+    G = np.zeros_like(s)
+    col = 0
+    for w in words:
+        if not w:
+            col += 1
+            continue
+        for i in range(1, len(w) + 1):
+            G[:, _widx(w[:i], da)] += g[:, col]
+            col += 1
+    want = sigref.sig_backprop(x, s, G, deg, **aug)
+    got = sigref.sig_coef_backprop(x, words, cp, g, **aug)
+    np.testing.assert_allclose(got, want, rtol=1e-11, atol=1e-12)
+    gotf = sigref.sig_coef_backprop(x.astype(np.float32), words, cp.astype(np.float32), g.astype(np.float32), **aug)
+    assert gotf.dtype == np.float32
+    np.testing.assert_allclose(gotf, want, rtol=2e-4, atol=2e-4)
+
+
+def test_sig_coef_backprop_vs_autograd():
+    rng = np.random.default_rng(34)
+    d, deg = 3, 3
+    words = [(2, 0, 1), (1, 1), (0,)]
+    x = torch.tensor(rng.uniform(size=(2, 6, d)), requires_grad=True)
+    s = M.signature(M.augment(x, time_aug=True, end_time=0.7), deg)
+    cols = [_widx(w[:i], d + 1) for w in words for i in range(1, len(w) + 1)]
+    g = rng.standard_normal((2, len(cols)))
+    (s[:, cols] * torch.tensor(g)).sum().backward()
+    xn = x.detach().numpy()
+    cp = sigref.sig_coef(xn, words, prefixes=True, time_aug=True, end_time=0.7)
+    np.testing.assert_allclose(cp, s[:, cols].detach().numpy(), rtol=1e-12, atol=1e-13)
+    got = sigref.sig_coef_backprop(xn, words, cp, g, time_aug=True, end_time=0.7)
+    np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-11, atol=1e-12)
