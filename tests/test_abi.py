@@ -52,7 +52,7 @@ def test_reference_loader_symbols_exported(lib):
 
 def test_out_of_scope_symbols_report_not_implemented(lib):
     lib.cusig_last_error_message.restype = ctypes.c_char_p
-    assert lib.sig_coef_cuda_d(None, None, None, 0, 0, 0) == 10
+    assert lib.sig_kernel_cuda_d(None, None, None, 0, 0, 0) == 10
     assert b"not implemented" in lib.cusig_last_error_message()
     assert lib.prepare_log_sig_cuda(2, 2, 0, False) == 10
 
