@@ -156,6 +156,26 @@ CUSIG_AMD_API int sig_coef_backprop_cuda_d(const double* path, double* out, cons
                                            const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
                                            uint64_t batch_size, uint64_t dimension, uint64_t length) CUSIG_AMD_NOEXCEPT;
 
+/* Expanded (tensor) logarithm of each signature; same row layout in and out, scalar slot of the result 0.
+ * method 0 only: methods 1 and 2 (Lyndon coordinates) return status 10.
+ * Replaces: sig_to_log_sig_cuda_{f,d} (decl siglib/cusig/cusig.h:407-409; arithmetic siglib/cpsig/cp_tensor_log.h:40-125),
+ * bound by pysiglib/load_siglib.py (CUSIG_SIG_TO_LOG_SIG), called from pysiglib/log_sig.py:223-311. */
+CUSIG_AMD_API int sig_to_log_sig_cuda_f(const float* sig, float* out, uint64_t batch_size, uint64_t dimension, uint64_t degree,
+                                        int method, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_to_log_sig_cuda_d(const double* sig, double* out, uint64_t batch_size, uint64_t dimension,
+                                        uint64_t degree, int method, bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
+/* Gradient w.r.t. the signature given dF/d(log signature) (method 0 layout); scalar slot of the result 0.
+ * Replaces: sig_to_log_sig_backprop_cuda_{f,d} (decl siglib/cusig/cusig.h:429-431; arithmetic
+ * siglib/cpsig/cp_tensor_log.h:164-221), bound by pysiglib/load_siglib.py (CUSIG_SIG_TO_LOG_SIG_BACKPROP), called from
+ * pysiglib/log_sig_backprop.py:30-137. */
+CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_f(const float* sig, float* out, const float* log_sig_derivs, uint64_t batch_size,
+                                                 uint64_t dimension, uint64_t degree, int method,
+                                                 bool scalar_term) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_d(const double* sig, double* out, const double* log_sig_derivs,
+                                                 uint64_t batch_size, uint64_t dimension, uint64_t degree, int method,
+                                                 bool scalar_term) CUSIG_AMD_NOEXCEPT;
+
 /* Message of the last failing call made by the calling thread ("" if none).
  * Replaces: cusig_last_error_message, probed by pysiglib/load_siglib.py:108-110
  * and read by pysiglib/error_codes.py:28-42. */

@@ -83,6 +83,15 @@ int sigref_sig_coef_d(const double *path, double *out, const uint64_t *multi_idx
 int sigref_sig_coef_backprop_d(const double *path, double *out, const double *coefs, const double *derivs,
                                const uint64_t *multi_idx, uint64_t num_multi_idx, const uint64_t *degrees, uint64_t batch,
                                uint64_t dimension, uint64_t length, int time_aug, int lead_lag, double end_time);
+/* sig_to_log_sig_{f,d} and its backprop with method 0 (expanded tensor logarithm), dimension already augmented. */
+int sigref_sig_to_log_sig_f(const float *sig, float *out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                            int scalar_term);
+int sigref_sig_to_log_sig_backprop_f(const float *sig, float *out, const float *log_sig_derivs, uint64_t batch,
+                                     uint64_t dimension, uint64_t degree, int scalar_term);
+int sigref_sig_to_log_sig_d(const double *sig, double *out, uint64_t batch, uint64_t dimension, uint64_t degree,
+                            int scalar_term);
+int sigref_sig_to_log_sig_backprop_d(const double *sig, double *out, const double *log_sig_derivs, uint64_t batch,
+                                     uint64_t dimension, uint64_t degree, int scalar_term);
 #ifdef __cplusplus
 }
 #endif

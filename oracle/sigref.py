@@ -55,6 +55,12 @@ def _load():
         f = getattr(lib, "sigref_sig_coef_backprop_" + suf)
         f.restype = i32
         f.argtypes = (ptr, ptr, ptr, ptr, pu, u64, pu, u64, u64, u64, i32, i32, real)
+        f = getattr(lib, "sigref_sig_to_log_sig_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, u64, u64, u64, i32)
+        f = getattr(lib, "sigref_sig_to_log_sig_backprop_" + suf)
+        f.restype = i32
+        f.argtypes = (ptr, ptr, ptr, u64, u64, u64, i32)
         f = getattr(lib, "sigref_linear_sig_" + suf)
         f.restype = i32
         f.argtypes = (ptr, ptr, u64, u64, u64, i32)
@@ -300,3 +306,33 @@ def sig_coef_backprop(path, words, coefs, derivs, time_aug=False, lead_lag=False
     if rc:
         raise RuntimeError("sigref_sig_coef_backprop returned %d" % rc)
     return out[0] if single else out
+
+
+def sig_to_log_sig(sig, dimension, degree):
+    """Oracle expanded (method 0) log signature; ``dimension`` is the augmented dimension."""
+    sig = np.asarray(sig)
+    suf, real = _suffix(sig.dtype)
+    a = _rows(sig, sig.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    out = np.empty_like(a)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_to_log_sig_" + suf)(a.ctypes.data_as(ptr), out.ctypes.data_as(ptr), a.shape[0], dimension,
+                                                      degree, int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_to_log_sig returned %d" % rc)
+    return out.reshape(sig.shape)
+
+
+def sig_to_log_sig_backprop(sig, derivs, dimension, degree):
+    sig = np.asarray(sig)
+    suf, real = _suffix(sig.dtype)
+    a, g = _rows(sig, sig.dtype), _rows(derivs, sig.dtype)
+    scalar_term = a.shape[1] == sig_length(dimension, degree)
+    out = np.empty_like(a)
+    ptr = ctypes.POINTER(real)
+    rc = getattr(LIB, "sigref_sig_to_log_sig_backprop_" + suf)(a.ctypes.data_as(ptr), out.ctypes.data_as(ptr),
+                                                               g.ctypes.data_as(ptr), a.shape[0], dimension, degree,
+                                                               int(scalar_term))
+    if rc:
+        raise RuntimeError("sigref_sig_to_log_sig_backprop returned %d" % rc)
+    return out.reshape(sig.shape)

@@ -773,6 +773,121 @@ int FN(sigref_sig_coef_backprop)(const REAL *path, REAL *out, const REAL *coefs,
     return 0;
 }
 
+/* Product without the identity terms: c_t = sum_{l=1..t-1} a_l (x) b_{t-l} for 2 <= t <= maxlevel (full layout). */
+static void FN(tail_product)(const REAL *a, const REAL *b, REAL *c, uint64_t maxlevel, const uint64_t *lvl)
+{
+    for (uint64_t t = 2; t <= maxlevel; ++t) {
+        REAL *res = c + lvl[t];
+        for (uint64_t i = 0; i < lvl[t + 1] - lvl[t]; ++i) res[i] = (REAL)0;
+        for (uint64_t left = 1; left < t; ++left) {
+            const uint64_t right = t - left, nl = lvl[left + 1] - lvl[left], nr = lvl[right + 1] - lvl[right];
+            for (uint64_t i = 0; i < nl; ++i)
+                for (uint64_t j = 0; j < nr; ++j) res[i * nr + j] += a[lvl[left] + i] * b[lvl[right] + j];
+        }
+    }
+}
+
+/* siglib/cpsig/cp_tensor_log.h:40-113 tensor_log_: with x = sig - 1,
+ *   log(1 + x) = P_1,  P_k = x / k - x (x) P_{k+1},  P_{N+1} = 0   (P_k needs levels <= N - k + 1).
+ * `P` (optional) receives P_2 .. P_N, each in full layout, zero above its top level. */
+static int FN(tensor_log)(const REAL *x /* full layout, x[0] ignored */, REAL *out, REAL *P, uint64_t d, uint64_t degree,
+                          const uint64_t *lvl)
+{
+    const uint64_t full = lvl[degree + 1];
+    REAL *cur = (REAL *)calloc(2 * full, sizeof(REAL));
+    if (!cur) return 1;
+    REAL *prod = cur + full;
+    (void)d;
+    for (uint64_t k = degree; k >= 1; --k) {
+        const uint64_t top = degree - k + 1;
+        FN(tail_product)(x, cur, prod, top, lvl);       /* x (x) P_{k+1}; empty for k = N */
+        const REAL inv = (REAL)1 / (REAL)k;
+        for (uint64_t i = 0; i < full; ++i) cur[i] = (REAL)0;
+        for (uint64_t t = 1; t <= top; ++t)
+            for (uint64_t i = lvl[t]; i < lvl[t + 1]; ++i) cur[i] = inv * x[i] - (t >= 2 ? prod[i] : (REAL)0);
+        if (P && k >= 2) memcpy(P + (k - 2) * full, cur, full * sizeof(REAL));
+    }
+    memcpy(out, cur, full * sizeof(REAL));
+    out[0] = (REAL)0;
+    free(cur);
+    return 0;
+}
+
+/* siglib/cpsig/cp_tensor_log.h:115-125 log_sig_expanded / sig_to_log_sig with method 0 */
+int FN(sigref_sig_to_log_sig)(const REAL *sig, REAL *out, uint64_t batch, uint64_t d, uint64_t degree, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1, off = scalar_term ? 0 : 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *x = (REAL *)malloc(2 * full * sizeof(REAL));
+    if (!lvl || !x) { free(lvl); free(x); return 1; }
+    REAL *o = x + full;
+    sigref_level_index(lvl, d, degree + 2);
+    int rc = 0;
+    for (uint64_t i = 0; i < batch && !rc; ++i) {
+        x[0] = (REAL)1;
+        memcpy(x + off, sig + i * stride, stride * sizeof(REAL));
+        rc = FN(tensor_log)(x, o, NULL, d, degree, lvl);
+        memcpy(out + i * stride, o + off, stride * sizeof(REAL));
+    }
+    free(lvl); free(x);
+    return rc;
+}
+
+/* siglib/cpsig/cp_tensor_log.h:164-221 tensor_log_backprop_: the adjoint of the recursion above, walked from P_1
+ * (where the upstream gradient enters) to P_N:  dx += g_k / k - [adjoint of x (x) P_{k+1} w.r.t. x],
+ * g_{k+1} = -[adjoint w.r.t. P_{k+1}]. */
+int FN(sigref_sig_to_log_sig_backprop)(const REAL *sig, REAL *out, const REAL *derivs, uint64_t batch, uint64_t d,
+                                       uint64_t degree, int scalar_term)
+{
+    if (d == 0) return 2;
+    const uint64_t full = sigref_sig_length(d, degree);
+    if (full == 0) return 10;
+    const uint64_t stride = scalar_term ? full : full - 1, off = scalar_term ? 0 : 1;
+    uint64_t *lvl = (uint64_t *)malloc((degree + 2) * sizeof(uint64_t));
+    REAL *x = (REAL *)malloc((5 + (degree > 1 ? degree - 1 : 1)) * full * sizeof(REAL));
+    if (!lvl || !x) { free(lvl); free(x); return 1; }
+    REAL *o = x + full, *g = o + full, *gn = g + full, *dx = gn + full, *P = dx + full;
+    sigref_level_index(lvl, d, degree + 2);
+    int rc = 0;
+    for (uint64_t b = 0; b < batch && !rc; ++b) {
+        x[0] = (REAL)1;
+        memcpy(x + off, sig + b * stride, stride * sizeof(REAL));
+        g[0] = (REAL)0;
+        memcpy(g + off, derivs + b * stride, stride * sizeof(REAL));
+        g[0] = (REAL)0;
+        for (uint64_t i = 0; i < full; ++i) dx[i] = (REAL)0;
+        if (degree >= 1) {
+            rc = FN(tensor_log)(x, o, P, d, degree, lvl);
+            for (uint64_t k = 1; k <= degree && !rc; ++k) {
+                const uint64_t top = degree - k + 1;
+                const REAL inv = (REAL)1 / (REAL)k;
+                for (uint64_t i = lvl[1]; i < lvl[top + 1]; ++i) dx[i] += inv * g[i];
+                if (k == degree) break;
+                const REAL *Pn = P + (k - 1) * full;        /* P_{k+1} */
+                for (uint64_t i = 0; i < full; ++i) gn[i] = (REAL)0;
+                for (uint64_t t = 2; t <= top; ++t)
+                    for (uint64_t left = 1; left < t; ++left) {
+                        const uint64_t right = t - left, nl = lvl[left + 1] - lvl[left], nr = lvl[right + 1] - lvl[right];
+                        const REAL *gt = g + lvl[t];
+                        for (uint64_t i = 0; i < nl; ++i)
+                            for (uint64_t j = 0; j < nr; ++j) {
+                                dx[lvl[left] + i] -= gt[i * nr + j] * Pn[lvl[right] + j];
+                                gn[lvl[right] + j] -= gt[i * nr + j] * x[lvl[left] + i];
+                            }
+                    }
+                memcpy(g, gn, full * sizeof(REAL));
+            }
+        }
+        dx[0] = (REAL)0;
+        memcpy(out + b * stride, dx + off, stride * sizeof(REAL));
+    }
+    free(lvl); free(x);
+    return rc;
+}
+
 #undef FN
 #undef CAT
 #undef CAT_

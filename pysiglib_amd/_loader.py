@@ -89,6 +89,13 @@ CUSIG_SIG_COEF_BACKPROP = _table("sig_coef_backprop_cuda", lambda r: (
     c_uint64))
 
 
+CUSIG_SIG_TO_LOG_SIG = _table("sig_to_log_sig_cuda", lambda r: (
+    POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_int, c_bool))
+
+CUSIG_SIG_TO_LOG_SIG_BACKPROP = _table("sig_to_log_sig_backprop_cuda", lambda r: (
+    POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_int, c_bool))
+
+
 def last_error_message():
     msg = CUSIG.cusig_last_error_message()
     return msg.decode("utf-8", errors="replace") if msg else ""

@@ -14,7 +14,7 @@ namespace sigamd {
 extern thread_local char g_last_error[4096];
 
 // Grow-only device buffers, one per (current device, slot), released by cusig_shutdown(); hold g_ws_mutex while a
-// buffer is in use (defined in sig_api.hip).  Slots 0-3: signature sweeps; 4-5: sig_join_backprop; 6: word tables of sig_coef.
+// buffer is in use (defined in sig_api.hip).  Slots 0-3: signature sweeps; 4-5: sig_join_backprop; 6: word tables of sig_coef; 7: tensor logarithm.
 extern std::mutex g_ws_mutex;
 void* workspace(int slot, size_t bytes);
 

@@ -28,8 +28,6 @@ STUB_PAIR(log_sig_combine_cuda)
 STUB_PAIR(log_sig_from_path_cuda)
 STUB_PAIR(log_sig_from_path_backprop_cuda)
 STUB_PAIR(log_sig_combine_backprop_cuda)
-STUB_PAIR(sig_to_log_sig_cuda)
-STUB_PAIR(sig_to_log_sig_backprop_cuda)
 STUB_PAIR(sig_kernel_cuda)
 STUB_PAIR(sig_kernel_poly_cuda)
 STUB_PAIR(sig_kernel_poly_backprop_cuda)

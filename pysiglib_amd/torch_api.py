@@ -128,3 +128,31 @@ def sig_coef(path, words, *, time_aug=False, lead_lag=False, end_time=1., prefix
         pos += max(len(w), 1)
         ends.append(pos - 1)
     return coefs[..., ends].contiguous()
+
+
+class SigToLogSig(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, sig_, dimension, degree, time_aug, lead_lag, method):
+        from .log_sig import sig_to_log_sig as _to_log
+        ctx.save_for_backward(sig_)
+        ctx.args = (dimension, degree, time_aug, lead_lag, method)
+        return _to_log(sig_, dimension, degree, time_aug=time_aug, lead_lag=lead_lag, method=method)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .log_sig import sig_to_log_sig_backprop as _to_log_backprop
+        (sig_,) = ctx.saved_tensors
+        dimension, degree, time_aug, lead_lag, method = ctx.args
+        grad = _to_log_backprop(sig_, grad_output, dimension, degree, time_aug=time_aug, lead_lag=lead_lag, method=method)
+        return grad, None, None, None, None, None
+
+
+def sig_to_log_sig(sig_, dimension, degree, *, time_aug=False, lead_lag=False, method=1, n_jobs=1):
+    """Differentiable ``sig_to_log_sig``."""
+    return SigToLogSig.apply(sig_, dimension, degree, time_aug, lead_lag, method)
+
+
+def log_sig(path, degree, *, time_aug=False, lead_lag=False, end_time=1., method=1, scalar_term=False, n_jobs=1):
+    """Differentiable ``log_sig``: the differentiable signature followed by the differentiable ``sig_to_log_sig``."""
+    sig_ = sig(path, degree, time_aug=time_aug, lead_lag=lead_lag, end_time=end_time, scalar_term=scalar_term)
+    return sig_to_log_sig(sig_, path.shape[-1], degree, time_aug=time_aug, lead_lag=lead_lag, method=method)

@@ -506,3 +506,103 @@ def test_sig_coef_abi_rejects_bad_letters(P):
     assert L.CUSIG_SIG_COEF["float64"](pd(x), pd(out), pu(letters), 1, pu(degrees), 2, 3, 5, False) == 2
     assert "out of range" in L.last_error_message()
     assert L.CUSIG_SIG_COEF["float64"](pd(x), pd(out), pu(letters), 1, pu(degrees), 2, 0, 5, False) == 2
+
+
+# ---------------------------------------------------------------------------
+# sig_to_log_sig / log_sig (method 0)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_log_sig_golden(P, fixtures, deg, dtype):
+    # the reference's own tests of the expanded log signature (tests/test_log_sig.py:101-144)
+    x = dev(fixtures["path"].astype(dtype))
+    tol = TOL[dtype]
+    np.testing.assert_allclose(P.log_sig(x, deg, method=0).cpu().numpy(), fixtures["logsig_exp__d%d" % deg], rtol=0, atol=tol)
+    np.testing.assert_allclose(P.log_sig(x[0], deg, method=0).cpu().numpy(), fixtures["logsig_exp__d%d" % deg][0], rtol=0, atol=tol)
+    np.testing.assert_allclose(P.log_sig(x, deg, time_aug=True, method=0).cpu().numpy(), fixtures["logsig_exp_ta__d%d" % deg],
+                               rtol=0, atol=tol)
+    if deg <= 4:
+        np.testing.assert_allclose(P.log_sig(x[:2], deg, lead_lag=True, method=0).cpu().numpy(),
+                                   fixtures["logsig_exp_ll__d%d" % deg], rtol=0, atol=tol)
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_log_sig_backprop_golden(P, fixtures, deg, dtype):
+    # tests/test_log_sig_backprop.py:49-100 of the reference: path gradient through log_sig(method=0)
+    for key, kw in (("logsig_bp_exp", {}), ("logsig_bp_exp_ta", dict(time_aug=True))):
+        x = torch.tensor(fixtures["path"], dtype=dtype, device=DEV, requires_grad=True)
+        ls = P.torch_api.log_sig(x, deg, method=0, **kw)
+        ls.backward(torch.tensor(fixtures["%s_derivs__d%d" % (key, deg)], dtype=dtype, device=DEV))
+        np.testing.assert_allclose(x.grad.cpu().numpy(), fixtures["%s_expected__d%d" % (key, deg)], rtol=0,
+                                   atol=1e-5 if dtype == torch.float64 else 1e-4)
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 6, 5), (3, 4, 70), (5, 3, 4), (1, 5, 3), (4, 1, 2), (3, 0, 3), (10, 5, 32),
+                                         (40, 2, 3), (2, 12, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_sig_to_log_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+    rng = np.random.default_rng(3 * d + deg)
+    n = oracle.sig_length(d, deg) - 1
+    scale = np.concatenate([np.full(d ** k, 0.5 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)]) if deg else np.zeros(0)
+    a = (rng.standard_normal((batch, n)) * scale).astype(dtype)
+    g = rng.standard_normal((batch, n)).astype(dtype)
+    if scalar_term:
+        a = np.hstack([np.ones((batch, 1), dtype=dtype), a])
+        g = np.hstack([np.full((batch, 1), 3.0, dtype=dtype), g])
+    elif deg == 0:
+        pytest.skip("empty rows")
+    off = 1 if scalar_term else 0
+    want = oracle.sig_to_log_sig(a, d, deg)
+    got = P.sig_to_log_sig(dev(a), d, deg, method=0).cpu().numpy()
+    assert got.shape == want.shape and got.dtype == dtype
+    if scalar_term:
+        assert np.all(got[:, 0] == 0)
+    if deg:
+        assert np.max(level_rel_err(got[:, off:], want[:, off:], d, deg)) < TOL[dtype]
+    wantb = oracle.sig_to_log_sig_backprop(a, g, d, deg)
+    gotb = P.sig_to_log_sig_backprop(dev(a), dev(g), d, deg, method=0).cpu().numpy()
+    assert gotb.shape == wantb.shape
+    if scalar_term:
+        assert np.all(gotb[:, 0] == 0)
+    if deg:
+        assert row_rel_err(gotb[:, off:], wantb[:, off:]) < TOL[dtype] * (1 if dtype == np.float64 else 10)
+
+
+def test_log_sig_identities_shapes_and_errors(P):
+    rng = np.random.default_rng(6)
+    d, deg = 3, 5
+    z = dev(rng.standard_normal((2, 4, d)))
+    lg = P.sig_to_log_sig(P.linear_sig(z, d, deg), d, deg, method=0)        # log(exp(z)) = z
+    assert lg.shape == (2, 4, P.sig_length(d, deg))
+    np.testing.assert_allclose(lg[..., :d].cpu().numpy(), z.cpu().numpy(), rtol=0, atol=1e-14)
+    np.testing.assert_allclose(lg[..., d:].cpu().numpy(), 0, rtol=0, atol=1e-13)
+    x = dev(rng.uniform(size=(3, 20, d)))
+    s = P.sig(x, deg, scalar_term=True)
+    np.testing.assert_array_equal(P.sig_to_log_sig(s, d, deg, method=0)[:, 1:].cpu().numpy(),
+                                  P.log_sig(x, deg, method=0).cpu().numpy())
+    sr = s.clone().requires_grad_(True)
+    out = P.torch_api.sig_to_log_sig(sr, d, deg, method=0)
+    w = torch.rand_like(out)
+    (out * w).sum().backward()
+    np.testing.assert_allclose(sr.grad.cpu().numpy(), P.sig_to_log_sig_backprop(s, w, d, deg, method=0).cpu().numpy(),
+                               rtol=1e-14, atol=1e-14)
+    empty = torch.empty((0, P.sig_length(d, deg)), dtype=torch.float64, device=DEV)
+    assert P.sig_to_log_sig(empty, d, deg, method=0).shape == empty.shape
+    with pytest.raises(NotImplementedError):
+        P.sig_to_log_sig(s, d, deg)                     # the reference's default, method=1, needs Lyndon tables
+    with pytest.raises(NotImplementedError):
+        P.log_sig(x, deg, method=3)
+    with pytest.raises(ValueError):
+        P.sig_to_log_sig(s, d, deg, method=7)
+    with pytest.raises(ValueError):
+        P.sig_to_log_sig(s[:, :-2], d, deg, method=0)
+    # the C ABI itself reports the unsupported methods with status 10
+    import ctypes
+    from pysiglib_amd import _loader as L
+    pd = lambda t: ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_double))
+    o = torch.empty_like(s)
+    assert L.CUSIG_SIG_TO_LOG_SIG["float64"](pd(s), pd(o), 3, d, deg, 1, True) == 10
+    assert "not implemented" in L.last_error_message()
+    assert L.CUSIG_SIG_TO_LOG_SIG["float64"](pd(s), pd(o), 3, d, deg, 5, True) == 2

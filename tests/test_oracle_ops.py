@@ -352,3 +352,87 @@ def test_sig_coef_backprop_vs_autograd():
     np.testing.assert_allclose(cp, s[:, cols].detach().numpy(), rtol=1e-12, atol=1e-13)
     got = sigref.sig_coef_backprop(xn, words, cp, g, time_aug=True, end_time=0.7)
     np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-11, atol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# sig_to_log_sig (method 0) and its backward pass: the reference's golden vectors for the expanded log signature
+# (tests/test_log_sig.py:101-144, tests/test_log_sig_backprop.py:49-100), the power series of log(1 + x) written with
+# the independent Chen product, autograd through it, and log(exp(z)) = z.
+# ---------------------------------------------------------------------------
+def _log_series(levels, degree):
+    """log(1 + x) = sum_n (-1)^(n+1) x^n / n with x given as level tensors (scalar part 0)."""
+    B = levels[0].shape[0]
+
+    def mul(a, b):      # product of two elements with zero scalar part
+        out = []
+        for t in range(1, degree + 1):
+            acc = torch.zeros_like(levels[t - 1])
+            for k in range(1, t):
+                acc = acc + (a[k - 1].unsqueeze(2) * b[t - k - 1].unsqueeze(1)).reshape(B, -1)
+            out.append(acc)
+        return out
+
+    power, total = levels, [l.clone() for l in levels]
+    for n in range(2, degree + 1):
+        power = mul(power, levels)
+        total = [t + ((-1) ** (n + 1)) * p / n for t, p in zip(total, power)]
+    return total
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+def test_log_sig_golden(fixtures, deg):
+    x = fixtures["path"]
+    for key, kw, d in (("logsig_exp", {}, 3), ("logsig_exp_ta", dict(time_aug=True), 4)):
+        s = sigref.signature(x, deg, **kw)
+        np.testing.assert_allclose(sigref.sig_to_log_sig(s, d, deg), fixtures["%s__d%d" % (key, deg)], rtol=0, atol=1e-10)
+        one = np.hstack([np.ones((len(s), 1)), s])
+        got1 = sigref.sig_to_log_sig(one, d, deg)
+        assert np.all(got1[:, 0] == 0)
+        np.testing.assert_array_equal(got1[:, 1:], sigref.sig_to_log_sig(s, d, deg))
+    if deg <= 4:
+        s = sigref.signature(x[:2], deg, lead_lag=True)
+        np.testing.assert_allclose(sigref.sig_to_log_sig(s, 6, deg), fixtures["logsig_exp_ll__d%d" % deg], rtol=0, atol=1e-10)
+    sf = sigref.signature(x.astype(np.float32), deg)
+    gotf = sigref.sig_to_log_sig(sf, 3, deg)
+    assert gotf.dtype == np.float32
+    np.testing.assert_allclose(gotf, fixtures["logsig_exp__d%d" % deg], rtol=0, atol=1e-4)
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+def test_log_sig_backprop_golden(fixtures, deg):
+    # the reference checks the path gradient through log_sig(method=0): tensor-log adjoint, then the pinned sig_backprop
+    x = fixtures["path"]
+    for key, kw, d in (("logsig_bp_exp", {}, 3), ("logsig_bp_exp_ta", dict(time_aug=True), 4)):
+        s = sigref.signature(x, deg, **kw)
+        ds = sigref.sig_to_log_sig_backprop(s, fixtures["%s_derivs__d%d" % (key, deg)], d, deg)
+        got = sigref.sig_backprop(x, s, ds, deg, **kw)
+        np.testing.assert_allclose(got, fixtures["%s_expected__d%d" % (key, deg)], rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("d,deg", [(2, 6), (3, 4), (5, 3), (1, 5), (4, 1), (3, 2)])
+def test_log_sig_vs_power_series_and_autograd(d, deg):
+    rng = np.random.default_rng(d * 7 + deg)
+    n = sigref.sig_length(d, deg) - 1
+    a = rng.standard_normal((3, n)) * 0.5           # arbitrary tensors, not group-like
+    g = rng.standard_normal((3, n))
+    ta = torch.tensor(a, requires_grad=True)
+    want = torch.cat(_log_series(_levels(ta, d, deg), deg), dim=1)
+    np.testing.assert_allclose(sigref.sig_to_log_sig(a, d, deg), want.detach().numpy(), rtol=1e-12, atol=1e-12)
+    want.backward(torch.tensor(g))
+    got = sigref.sig_to_log_sig_backprop(a, g, d, deg)
+    np.testing.assert_allclose(got, ta.grad.numpy(), rtol=1e-11, atol=1e-11)
+    one, zero = np.ones((3, 1)), np.zeros((3, 1))
+    got1 = sigref.sig_to_log_sig_backprop(np.hstack([one, a]), np.hstack([zero + 5.0, g]), d, deg)
+    assert np.all(got1[:, 0] == 0)
+    np.testing.assert_allclose(got1[:, 1:], got, rtol=1e-13, atol=1e-13)
+    gotf = sigref.sig_to_log_sig_backprop(a.astype(np.float32), g.astype(np.float32), d, deg)
+    np.testing.assert_allclose(gotf, got, rtol=1e-3, atol=1e-3)
+
+
+def test_log_of_segment_exponential_is_the_increment():
+    rng = np.random.default_rng(4)
+    d, deg = 3, 5
+    z = rng.standard_normal((4, d))
+    lg = sigref.sig_to_log_sig(sigref.linear_sig(z, d, deg), d, deg)
+    np.testing.assert_allclose(lg[:, :d], z, rtol=0, atol=1e-14)
+    np.testing.assert_allclose(lg[:, d:], 0, rtol=0, atol=1e-13)
