@@ -153,6 +153,20 @@ def bench_ops(args, torch, loader):
     def p(t):
         return ctypes.cast(t.data_ptr(), ctypes.POINTER(real))
 
+    def pu(t):
+        return ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_uint64))
+
+    # sig_coef: every word of 3 letters over 10 channels (1000 words, prefixes layout), 256 paths of 1000 points
+    import itertools
+    words = list(itertools.product(range(d), repeat=3))
+    n_words, cb, clen = len(words), 256, 1000
+    letters = torch.tensor([i for w in words for i in w], dtype=torch.int64, device="cuda:0")
+    degrees = torch.full((n_words,), 3, dtype=torch.int64, device="cuda:0")
+    cpath = torch.rand((cb, clen, d), **f64)
+    cout = torch.empty((cb, 3 * n_words), **f64)
+    cg = torch.rand((cb, 3 * n_words), **f64)
+    cgrad = torch.empty_like(cpath)
+
     sig_bytes = batch * n * 8
     cases = [
         ("sig_combine", lambda: loader.CUSIG_SIG_COMBINE["float64"](p(a), p(b), p(o1), batch, d, deg, False), 3 * sig_bytes),
@@ -160,6 +174,10 @@ def bench_ops(args, torch, loader):
         ("linear_sig", lambda: loader.CUSIG_LINEAR_SIG["float64"](p(z), p(o1), batch, d, deg, False), sig_bytes),
         ("sig_join", lambda: loader.CUSIG_SIG_JOIN["float64"](p(a), p(z), p(o1), batch, d, deg, False, False), 2 * sig_bytes),
         ("sig_join_backprop", lambda: loader.CUSIG_SIG_JOIN_BACKPROP["float64"](p(g), p(o1), p(oz), p(a), p(z), batch, d, deg, False, False), 3 * sig_bytes),
+        ("sig_to_log_sig", lambda: loader.CUSIG_SIG_TO_LOG_SIG["float64"](p(a), p(o1), batch, d, deg, 0, False), 2 * sig_bytes),
+        ("sig_to_log_sig_backprop", lambda: loader.CUSIG_SIG_TO_LOG_SIG_BACKPROP["float64"](p(a), p(o1), p(g), batch, d, deg, 0, False), 3 * sig_bytes),
+        ("sig_coef", lambda: loader.CUSIG_SIG_COEF["float64"](p(cpath), p(cout), pu(letters), n_words, pu(degrees), cb, d, clen, True), (cpath.numel() + cout.numel()) * 8),
+        ("sig_coef_backprop", lambda: loader.CUSIG_SIG_COEF_BACKPROP["float64"](p(cpath), p(cgrad), p(cout), p(cg), pu(letters), n_words, pu(degrees), cb, d, clen), (2 * cpath.numel() + 2 * cout.numel()) * 8),
         ("transform_path", lambda: loader.CUSIG_TRANSFORM_PATH["float64"](p(path), p(tpath), pb, pdim, plen, True, True, 1.0), (path.numel() + tpath.numel()) * 8),
         ("transform_path_backprop", lambda: loader.CUSIG_TRANSFORM_PATH_BACKPROP["float64"](p(tpath), p(gpath), pb, pdim, plen, True, True, 1.0), (path.numel() + tpath.numel()) * 8),
     ]
@@ -181,7 +199,9 @@ def bench_ops(args, torch, loader):
                       "unit": "GB/s", "peak": 8000.0, "dtype": "f64", "data": "synthetic", "steps": args.steps,
                       "warmup": args.warmup,
                       "config": {"workload": "signatures: batch %d, dim %d, degree %d (%d coefficients); paths: (%d, %d, %d) "
-                                             "with lead-lag + time" % (batch, d, deg, n, pb, plen, pdim)},
+                                             "with lead-lag + time; sig_coef: %d words of 3 letters, paths (%d, %d, %d) "
+                                             "(a sweep: compute-bound, its GB/s is not a bandwidth figure)"
+                                             % (batch, d, deg, n, pb, plen, pdim, n_words, cb, clen, d)},
                       "ops": out}))
 
 

@@ -114,69 +114,111 @@ __global__ __launch_bounds__(kBlock) void sig_coef_kernel(
 // Reverse sweep of one (path, word) pair: coefficients before the step by exp(-z), then the adjoint of the step:
 // with st_j = ((1/i!) z_0 + c_1/(i-1)!) z_1 + ... (the Horner values of prefix length i),
 //   dz_{i-1} += g_i st_{i-1};  walking j = i-2 .. 0 with sd = g_i z_{i-1} z_{i-2} ..:  dz_j += sd st_j,
-//   g_{j+1} += sd / (i-j-1)!.   The increment gradient goes to the two path points of the step with atomics
-// (several words, and several letters of one word, share path entries); `out` is zeroed beforehand.
+//   g_{j+1} += sd / (i-j-1)!.
+// A block serves the words blockIdx.x * blockDim.x .. of ONE path and walks the steps in lockstep: all its lanes
+// add their increment gradients of a step into per-channel LDS sums (`copies` private sets, chosen by lane, because
+// few channels mean many lanes per word of LDS), and lane j then owns channel j: path point s-1 receives
+// -dz(step s) + dz(step s-1), so the lane carries the first term over to the next step and issues ONE atomic per
+// (block, point, channel).  use_lds = 0 (very wide paths): every lane adds straight to HBM.  `out` is zeroed beforehand.
 template <typename T, int KMAX, int UF>
-__global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
+__global__ void sig_coef_bwd_kernel(
     const T* __restrict__ path, T* __restrict__ out, const T* __restrict__ coefs, const T* __restrict__ derivs,
-    WordList words, int64_t batch, int64_t d, int64_t len, int64_t row)
+    WordList words, int64_t batch, int64_t d, int64_t len, int64_t row, int use_lds, int copies)
 {
-    const int64_t total = batch * int64_t(words.count);
-    for (int64_t item = int64_t(blockIdx.x) * kBlock + threadIdx.x; item < total; item += int64_t(gridDim.x) * kBlock) {
-        const int64_t b = item / int64_t(words.count), w = item % int64_t(words.count);
-        const int k = int(words.degree[w]);
-        if (k == 0 || k > KMAX || len < 2) continue;
+    extern __shared__ double coef_lds_raw[];
+    T* acc = reinterpret_cast<T*>(coef_lds_raw);
+    const int64_t w = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const bool live = w < int64_t(words.count);
+    const int k = live ? int(words.degree[w]) : 0;
+    const bool active = k > 0 && k <= KMAX;
+    T* mine = acc + int64_t(threadIdx.x % copies) * d;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         int64_t let[KMAX];
         T c[KMAX + 1], g[KMAX + 1], z[KMAX], next[KMAX], st[KMAX], dz[KMAX];
         const T* x = path + b * len * d;
         T* gx = out + b * len * d;
-        const T* crow = coefs + b * row + int64_t(words.out_start[w]);
-        const T* grow = derivs + b * row + int64_t(words.out_start[w]);
         c[0] = T(1);
         g[0] = T(0);
-#pragma unroll UF
-        for (int i = 0; i < KMAX; ++i) {
-            let[i] = i < k ? int64_t(words.letters[words.start[w] + i]) : 0;
-            next[i] = x[(len - 1) * d + let[i]];
-            c[i + 1] = i < k ? crow[i] : T(0);
-            g[i + 1] = i < k ? grow[i] : T(0);
-        }
-        for (int64_t s = len - 1; s >= 1; --s) {        // step s-1 -> s
-            const T* xp = x + (s - 1) * d;
+        if (active) {
+            const T* crow = coefs + b * row + int64_t(words.out_start[w]);
+            const T* grow = derivs + b * row + int64_t(words.out_start[w]);
 #pragma unroll UF
             for (int i = 0; i < KMAX; ++i) {
-                const T cur = xp[let[i]];
-                z[i] = next[i] - cur;
-                next[i] = cur;
+                let[i] = i < k ? int64_t(words.letters[words.start[w] + i]) : 0;
+                next[i] = x[(len - 1) * d + let[i]];
+                c[i + 1] = i < k ? crow[i] : T(0);
+                g[i + 1] = i < k ? grow[i] : T(0);
             }
-            word_step<T, KMAX, UF, -1>(c, z, k);
+        }
+        if (use_lds) {
+            __syncthreads();        // the previous path's sums have been consumed
+            for (int64_t j = threadIdx.x; j < int64_t(copies) * d; j += blockDim.x) acc[j] = T(0);
+            __syncthreads();
+        }
+        T carry = T(0);             // lane j: -dz(step s)[j], still to be added to point s-1
+        for (int64_t s = len - 1; s >= 1; --s) {        // step s-1 -> s
+            if (active) {
+                const T* xp = x + (s - 1) * d;
 #pragma unroll UF
-            for (int i = 0; i < KMAX; ++i) dz[i] = T(0);
+                for (int i = 0; i < KMAX; ++i) {
+                    const T cur = xp[let[i]];
+                    z[i] = next[i] - cur;
+                    next[i] = cur;
+                }
+                word_step<T, KMAX, UF, -1>(c, z, k);
 #pragma unroll UF
-            for (int i = 1; i <= KMAX; ++i) {
-                if (i <= k) {
-                    st[0] = T(kInvFact[i]);
+                for (int i = 0; i < KMAX; ++i) dz[i] = T(0);
 #pragma unroll UF
-                    for (int j = 0; j + 1 < i; ++j) st[j + 1] = fmadd(st[j], z[j], c[j + 1] * T(kInvFact[i - j - 1]));
-                    const T gi = g[i];
-                    dz[i - 1] = fmadd(gi, st[i - 1], dz[i - 1]);
-                    T sd = gi * z[i - 1];
+                for (int i = 1; i <= KMAX; ++i) {
+                    if (i <= k) {
+                        st[0] = T(kInvFact[i]);
 #pragma unroll UF
-                    for (int j = i - 2; j >= 0; --j) {
-                        dz[j] = fmadd(sd, st[j], dz[j]);
-                        g[j + 1] = fmadd(sd, T(kInvFact[i - j - 1]), g[j + 1]);
-                        sd *= z[j];
+                        for (int j = 0; j + 1 < i; ++j) st[j + 1] = fmadd(st[j], z[j], c[j + 1] * T(kInvFact[i - j - 1]));
+                        const T gi = g[i];
+                        dz[i - 1] = fmadd(gi, st[i - 1], dz[i - 1]);
+                        T sd = gi * z[i - 1];
+#pragma unroll UF
+                        for (int j = i - 2; j >= 0; --j) {
+                            dz[j] = fmadd(sd, st[j], dz[j]);
+                            g[j + 1] = fmadd(sd, T(kInvFact[i - j - 1]), g[j + 1]);
+                            sd *= z[j];
+                        }
+                    }
+                }
+#pragma unroll UF
+                for (int i = 0; i < KMAX; ++i) {
+                    if (i < k) {
+                        if (use_lds) {
+                            lds_add_shared(&mine[let[i]], dz[i]);
+                        } else {
+                            dev_add(&gx[s * d + let[i]], dz[i]);
+                            dev_add(&gx[(s - 1) * d + let[i]], -dz[i]);
+                        }
                     }
                 }
             }
-#pragma unroll UF
-            for (int i = 0; i < KMAX; ++i) {
-                if (i < k) {
-                    dev_add(&gx[s * d + let[i]], dz[i]);
-                    dev_add(&gx[(s - 1) * d + let[i]], -dz[i]);
+            if (use_lds) {
+                __syncthreads();
+                for (int64_t j = threadIdx.x; j < d; j += blockDim.x) {
+                    T sum = T(0);
+                    for (int q = 0; q < copies; ++q) {
+                        sum += acc[int64_t(q) * d + j];
+                        acc[int64_t(q) * d + j] = T(0);
+                    }
+                    // d <= blockDim.x is not required: a lane's `carry` belongs to channel j only when it owns one
+                    // channel, so wider paths add both terms directly
+                    if (d <= int64_t(blockDim.x)) {
+                        dev_add(&gx[s * d + j], sum + carry);
+                        carry = -sum;
+                    } else {
+                        dev_add(&gx[s * d + j], sum);
+                        dev_add(&gx[(s - 1) * d + j], -sum);
+                    }
                 }
+                __syncthreads();
             }
         }
+        if (use_lds && d <= int64_t(blockDim.x) && int64_t(threadIdx.x) < d && len >= 2) dev_add(&gx[threadIdx.x], carry);
     }
 }
 
@@ -280,10 +322,19 @@ static void sig_coef_backprop_impl(const T* path, T* out, const T* coefs, const 
         const uint64_t items = checked_mul(batch, num_words, "work items");
         std::lock_guard<std::mutex> lk(g_ws_mutex);
         const WordList words = upload_words(h, multi_idx, stream);
+        (void)items;
+        // one block = up to 256 words of one path; per-channel sums in LDS unless the path is too wide for it
+        const unsigned threads = num_words <= 64 ? 64u : unsigned(kBlock);
+        const uint64_t gx = (num_words + threads - 1) / threads;
+        if (gx > 0x7fffffffull) throw std::runtime_error("sig_coef_backprop_cuda: too many words");
+        const int use_lds = dimension <= 4096;
+        const int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(32, 4096 / dimension))) : 1;
+        const size_t lds = use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0;
+        const dim3 grid{unsigned(gx), unsigned(std::min<uint64_t>(batch, 65535)), 1};
         with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
             constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;
-            hipLaunchKernelGGL((sig_coef_bwd_kernel<T, KMAX, UF>), dim3(grid_for(items)), dim3(kBlock), 0, stream, path, out, coefs,
-                               derivs, words, int64_t(batch), int64_t(dimension), int64_t(length), int64_t(h.row));
+            hipLaunchKernelGGL((sig_coef_bwd_kernel<T, KMAX, UF>), grid, dim3(threads), lds, stream, path, out, coefs, derivs,
+                               words, int64_t(batch), int64_t(dimension), int64_t(length), int64_t(h.row), use_lds, copies);
         });
         SIG_HIP(hipGetLastError());
         SIG_HIP(hipStreamSynchronize(stream));
