@@ -306,12 +306,13 @@ static Shape make_shape(uint64_t dimension, uint64_t length, uint64_t degree, bo
 
 template <typename T>
 static void compute_increments(const T* path, T* inc, uint64_t batch, uint64_t dimension, uint64_t length,
-                               bool time_aug, bool lead_lag, T end_time, const Shape& s, hipStream_t stream)
+                               bool time_aug, bool lead_lag, T end_time, const Shape& s, hipStream_t stream,
+                               T* zero_out = nullptr, uint64_t zero_count = 0)
 {
     const T time_step = s.len_aug > 1 ? end_time / T(s.len_aug - 1) : T(0);
     hipLaunchKernelGGL((increments_kernel<T>), dim3(grid_for(batch * (s.L + 2) * s.d_aug)), dim3(kBlock), 0, stream,
                        path, inc, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
-                       int(lead_lag), time_step);
+                       int(lead_lag), time_step, zero_out, int64_t(zero_count));
     SIG_HIP(hipGetLastError());
 }
 
@@ -457,10 +458,8 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;
         T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
         T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
-        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
-        hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(dz_elems)), dim3(kBlock), 0, stream, dzinc,
-                           int64_t(dz_elems));
-        SIG_HIP(hipGetLastError());
+        // one launch writes the increments and clears the increment-gradient accumulator (dz_elems <= increment elements)
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
         BwdParams p;
         p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
         p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;

@@ -27,8 +27,10 @@ __device__ __forceinline__ void static_for(F&& f)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void increments_kernel(
     const T* __restrict__ path, T* __restrict__ inc, int64_t batch, int64_t len_raw, int d_raw,
-    int time_aug, int lead_lag, T time_step)
+    int time_aug, int lead_lag, T time_step, T* __restrict__ zero_out, int64_t zero_count)
 {
+    // zero_out (optional, zero_count <= number of increment elements): cleared in the same launch; the backward
+    // accumulates its increment gradient there with atomics.
     // Layout [batch][L + 2][d]: row t + 1 holds the increment of step t; rows 0 and L + 1 are zero so
     // that the sweeps may prefetch one row past either end of a path without a bounds test.
     const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
@@ -57,6 +59,7 @@ __global__ __launch_bounds__(kBlock) void increments_kernel(
             }
         }
         inc[e] = v;
+        if (e < zero_count) zero_out[e] = T(0);
     }
 }
 
