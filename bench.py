@@ -255,6 +255,23 @@ def main():
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     value = r1.c["batch"] / (ms_per_step * 1e-3)
 
+    # the same steps with the library in stream-ordered mode: calls only enqueue, the host syncs once at the end
+    loader.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
+    loader.CUSIG.cusig_amd_set_stream_ordered.restype = None
+    loader.CUSIG.cusig_amd_set_stream_ordered(1)
+    try:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ordered_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    finally:
+        loader.CUSIG.cusig_amd_set_stream_ordered(0)
+        torch.cuda.synchronize()
+
     # per-kernel figures (HIP events inside the library, on the launch stream)
     wall_f, kms_f, name_f = time_calls(r1.forward, torch, loader, 1, max(5, args.steps))
     wall_b, kms_b, name_b = time_calls(r5.backward, torch, loader, 1, max(5, args.steps))
@@ -303,6 +320,10 @@ def main():
             "fwd_bwd_combined_frac": (r1.flops_fwd + r5.flops_bwd) / ((kms_f + kms_b) * 1e-3) / 1e12 / peak,
         },
         "configs": configs,
+        "stream_ordered": {"value": r1.c["batch"] / (ordered_ms * 1e-3), "ms_per_step": ordered_ms,
+                           "note": "same steps with cusig_amd_set_stream_ordered(1): calls enqueue on the null stream, "
+                                   "one host synchronisation after the last step; `value` above is the reference's "
+                                   "synchronous contract"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(np, cfgmod)

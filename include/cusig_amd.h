@@ -204,6 +204,12 @@ CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only
  * taken for rows of 2^31 coefficients or more) whatever the size. */
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
+/* Stream-ordered mode (no counterpart in the reference, off by default).  When enabled, signature_cuda_{f,d} and
+ * sig_backprop_cuda_{f,d} enqueue their kernels on the null stream and return without waiting, and do not wait for
+ * other streams on entry: inputs must be ordered before, and consumers after, the null stream (true for PyTorch's
+ * default stream and for blocking streams).  Kernel faults then surface at the caller's next synchronisation.
+ * Process-wide. */
+CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: prefer the compiled lane partition (tail, k) where a shape has several; tail = 0 restores
  * the defaults.  Not thread-safe; meant for offline sweeps. */
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) CUSIG_AMD_NOEXCEPT;

@@ -216,6 +216,20 @@ struct MainKernelTimer {
     }
 };
 
+// Stream-ordered mode (off by default): signature_cuda / sig_backprop_cuda only enqueue their kernels on the null
+// stream and return; neither the device-wide wait on entry nor the wait for completion is made.  Correct for callers
+// whose producers and consumers are ordered with the null stream (PyTorch's default stream is the null stream, and
+// blocking streams synchronise with it implicitly); it removes the host round trip between consecutive calls.
+static int g_stream_ordered = 0;
+static void entry_sync()
+{
+    if (!g_stream_ordered) SIG_HIP(hipDeviceSynchronize());
+}
+static void exit_sync(hipStream_t stream)
+{
+    if (!g_stream_ordered) SIG_HIP(hipStreamSynchronize(stream));
+}
+
 // ---------------------------------------------------------------------------
 // time segmentation of the forward sweep
 // ---------------------------------------------------------------------------
@@ -333,7 +347,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
     const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
     checked_mul(checked_mul(batch, s.stride, "signature output"), sizeof(T), "signature output");
     hipStream_t stream = nullptr;
-    SIG_HIP(hipDeviceSynchronize());   // inputs may have been produced on any stream
+    entry_sync();   // inputs may have been produced on any stream
 
     const int sc = scalar_term ? 1 : 0;
     if (s.len_aug <= 1) {
@@ -412,11 +426,11 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                 acc_stride = int64_t(n_coef);
             }
         }
-        SIG_HIP(hipStreamSynchronize(stream));
+        exit_sync(stream);
         return;
     }
     SIG_HIP(hipGetLastError());
-    SIG_HIP(hipStreamSynchronize(stream));
+    exit_sync(stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -436,7 +450,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
     const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
     const uint64_t out_elems = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
     hipStream_t stream = nullptr;
-    SIG_HIP(hipDeviceSynchronize());
+    entry_sync();
     const int sc = scalar_term ? 1 : 0;
 
     if (s.len_aug <= 1 || degree == 0) {
@@ -470,11 +484,11 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         hipLaunchKernelGGL((path_grad_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, dzinc, out,
                            int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
         SIG_HIP(hipGetLastError());
-        SIG_HIP(hipStreamSynchronize(stream));
+        exit_sync(stream);
         return;
     }
     SIG_HIP(hipGetLastError());
-    SIG_HIP(hipStreamSynchronize(stream));
+    exit_sync(stream);
 }
 
 }  // namespace sigamd
@@ -549,6 +563,8 @@ CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_seg
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
 
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
+
+CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {

@@ -378,3 +378,34 @@ def test_config5_backward_full_size(P, oracle):
     sig_gpu = P.sig(dev(x), 5)
     got3 = P.sig_backprop(dev(x), sig_gpu, dev(g), 5).cpu().numpy()
     assert bwd_rel_err(got3, ref) <= 1e-10
+
+
+def test_stream_ordered_mode(P, oracle):
+    """Calls that only enqueue on the null stream: results after one synchronisation equal the synchronous ones,
+    also when consecutive calls reuse the library's workspaces with different shapes."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_stream_ordered.restype = None
+    rng = np.random.default_rng(99)
+    cases = [((6, 50, 4), 4), ((3, 120, 10), 5), ((9, 20, 3), 6), ((2, 300, 2), 3)]
+    xs = [dev(rng.standard_normal(shape) * 0.3) for shape, _ in cases]
+    want = []
+    for x, (_, deg) in zip(xs, cases):
+        s = P.sig(x, deg)
+        g = torch.ones_like(s)
+        want.append((s.cpu().numpy(), P.sig_backprop(x, s, g, deg).cpu().numpy()))
+    L.CUSIG.cusig_amd_set_stream_ordered(1)
+    try:
+        got = []
+        for _ in range(3):
+            got = []
+            for x, (_, deg) in zip(xs, cases):
+                s = P.sig(x, deg)
+                got.append((s, P.sig_backprop(x, s, torch.ones_like(s), deg)))
+        torch.cuda.synchronize()
+    finally:
+        L.CUSIG.cusig_amd_set_stream_ordered(0)
+    for (s, gr), (ws, wg) in zip(got, want):
+        np.testing.assert_allclose(s.cpu().numpy(), ws, rtol=0, atol=0)
+        np.testing.assert_allclose(gr.cpu().numpy(), wg, rtol=1e-12, atol=1e-13)
