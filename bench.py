@@ -25,7 +25,6 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 TRAFFIC_BYTES = {
     "fwd_f64_d10_n5_t2_k5_lds": 53.0e6,
     "bwd_f64_d10_n5_t2_k5_lds": 152.0e6,
-    "fwd_f32_d5_n7_t2_k5_lds": 71.4e6,
     "fwd_f64_d3_n12_t4_k3": 462.6e6,
     "fwd_f32_d17_n4_t1_k17": 323.0e6,
 }
