@@ -5,7 +5,7 @@ from ctypes import POINTER, c_uint64, cast
 import torch
 
 from ._loader import CUSIG_SIG_COEF, CUSIG_SIG_COEF_BACKPROP
-from .data_handlers import PathInput, SigInput, empty_like_input
+from .data_handlers import PathInput, SigInput, empty_like_input, on_device
 from .error_codes import err_msg
 from .ops import _same, transform_path, transform_path_backprop
 from .param_checks import check_n_jobs, check_non_neg, check_type, check_word, check_word_or_word_list
@@ -72,7 +72,7 @@ def sig_coef(path, words, *, time_aug=False, lead_lag=False, end_time=1., prefix
         return out
     check_n_jobs(n_jobs)
     letters, degrees = _device_words(words, data.device)
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_SIG_COEF[data.dtype](data.data_ptr, out_ptr, _u64(letters), len(words), _u64(degrees), data.batch_size,
                                           data.data_dimension, data.data_length, prefixes)
     if code:
@@ -104,7 +104,7 @@ def sig_coef_backprop(path, words, coefs, derivs, *, time_aug=False, lead_lag=Fa
         return out
     check_n_jobs(n_jobs)
     letters, degrees = _device_words(words, data.device)
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_SIG_COEF_BACKPROP[data.dtype](data.data_ptr, out_ptr, c.data_ptr, g.data_ptr, _u64(letters), len(words),
                                                    _u64(degrees), data.batch_size, data.data_dimension, data.data_length)
     if code:

@@ -71,3 +71,23 @@ def empty_like_input(data, shape):
     dtype = torch.float32 if data.dtype == "float32" else torch.float64
     out = torch.empty((*data.batch_shape, *shape), dtype=dtype, device=data.device)
     return out, cast(out.data_ptr(), POINTER(DTYPES[data.dtype]))
+
+
+class on_device:
+    """``with on_device(dev):`` makes ``dev`` the current device for the C call; free when it already is."""
+
+    def __init__(self, device):
+        self.idx = device.index if device.index is not None else torch.cuda.current_device()
+        self.prev = None
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False

@@ -4,7 +4,7 @@ reference's signatures (pysiglib/log_sig.py:223-470, pysiglib/log_sig_backprop.p
 import torch
 
 from ._loader import CUSIG_SIG_TO_LOG_SIG, CUSIG_SIG_TO_LOG_SIG_BACKPROP
-from .data_handlers import SigInput, empty_like_input
+from .data_handlers import SigInput, empty_like_input, on_device
 from .error_codes import err_msg
 from .ops import _same
 from .param_checks import check_n_jobs, check_non_neg, check_type
@@ -42,7 +42,7 @@ def sig_to_log_sig(sig_, dimension, degree, *, time_aug=False, lead_lag=False, m
     if data.batch_size == 0:
         return out
     check_n_jobs(n_jobs)
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_SIG_TO_LOG_SIG[data.dtype](data.data_ptr, out_ptr, data.batch_size, d, degree, method, scalar_term)
     if code:
         raise Exception("Error in pysiglib.sig_to_log_sig: " + err_msg(code))
@@ -64,7 +64,7 @@ def sig_to_log_sig_backprop(sig_, log_sig_derivs, dimension, degree, *, time_aug
     if data.batch_size == 0:
         return out
     check_n_jobs(n_jobs)
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_SIG_TO_LOG_SIG_BACKPROP[data.dtype](data.data_ptr, out_ptr, derivs.data_ptr, data.batch_size, d, degree,
                                                          method, scalar_term)
     if code:

@@ -6,7 +6,7 @@ import torch
 
 from ._loader import (CUSIG_LINEAR_SIG, CUSIG_SIG_COMBINE, CUSIG_SIG_COMBINE_BACKPROP, CUSIG_SIG_JOIN,
                       CUSIG_SIG_JOIN_BACKPROP, CUSIG_TRANSFORM_PATH, CUSIG_TRANSFORM_PATH_BACKPROP)
-from .data_handlers import PathInput, SigInput, empty_like_input
+from .data_handlers import PathInput, SigInput, empty_like_input, on_device
 from .error_codes import err_msg
 from .param_checks import check_n_jobs, check_non_neg, check_type
 from .sig_length import aug_dim, infer_scalar_term, sig_length
@@ -40,7 +40,7 @@ def sig_combine(sig1, sig2, dimension, degree, *, time_aug=False, lead_lag=False
     out, out_ptr = empty_like_input(a, (n,))
     if a.batch_size == 0:
         return out
-    with torch.cuda.device(a.device):
+    with on_device(a.device):
         code = CUSIG_SIG_COMBINE[a.dtype](a.data_ptr, b.data_ptr, out_ptr, a.batch_size, d, degree, scalar_term)
     if code:
         raise Exception("Error in pysiglib.sig_combine: " + err_msg(code))
@@ -63,7 +63,7 @@ def sig_combine_backprop(derivs, sig1, sig2, dimension, degree, *, time_aug=Fals
     d2, d2_ptr = empty_like_input(a, (n,))
     if a.batch_size == 0:
         return d1, d2
-    with torch.cuda.device(a.device):
+    with on_device(a.device):
         code = CUSIG_SIG_COMBINE_BACKPROP[a.dtype](g.data_ptr, d1_ptr, d2_ptr, a.data_ptr, b.data_ptr, a.batch_size, d,
                                                    degree, scalar_term)
     if code:
@@ -85,7 +85,7 @@ def transform_path(path, *, time_aug=False, lead_lag=False, end_time=1., n_jobs=
     out, out_ptr = empty_like_input(data, (data.length, data.dimension))
     if data.batch_size == 0:
         return out
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_TRANSFORM_PATH[data.dtype](data.data_ptr, out_ptr, data.batch_size, data.data_dimension,
                                                 data.data_length, time_aug, lead_lag, end_time)
     if code:
@@ -116,7 +116,7 @@ def transform_path_backprop(derivs, *, time_aug=False, lead_lag=False, end_time=
     out, out_ptr = empty_like_input(data, (length, dim))
     if data.batch_size == 0:
         return out
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_TRANSFORM_PATH_BACKPROP[data.dtype](data.data_ptr, out_ptr, data.batch_size, dim, length, time_aug,
                                                          lead_lag, end_time)
     if code:
@@ -137,7 +137,7 @@ def linear_sig(displacement, dimension, degree, *, scalar_term=False, n_jobs=1):
     out, out_ptr = empty_like_input(z, (n,))
     if z.batch_size == 0:
         return out
-    with torch.cuda.device(z.device):
+    with on_device(z.device):
         code = CUSIG_LINEAR_SIG[z.dtype](z.data_ptr, out_ptr, z.batch_size, dimension, degree, scalar_term)
     if code:
         raise Exception("Error in pysiglib.linear_sig: " + err_msg(code))
@@ -158,7 +158,7 @@ def sig_join(sig, displacement, dimension, degree, *, prepend=False, n_jobs=1):
     out, out_ptr = empty_like_input(a, (n,))
     if a.batch_size == 0:
         return out
-    with torch.cuda.device(a.device):
+    with on_device(a.device):
         code = CUSIG_SIG_JOIN[a.dtype](a.data_ptr, z.data_ptr, out_ptr, a.batch_size, dimension, degree, bool(prepend),
                                        scalar_term)
     if code:
@@ -181,7 +181,7 @@ def sig_join_backprop(d_out, sig, displacement, dimension, degree, *, prepend=Fa
     d_disp, d_disp_ptr = empty_like_input(g, (dimension,))
     if g.batch_size == 0:
         return d_sig, d_disp
-    with torch.cuda.device(g.device):
+    with on_device(g.device):
         code = CUSIG_SIG_JOIN_BACKPROP[g.dtype](g.data_ptr, d_sig_ptr, d_disp_ptr, a.data_ptr, z.data_ptr, g.batch_size,
                                                 dimension, degree, bool(prepend), scalar_term)
     if code:

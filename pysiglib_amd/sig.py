@@ -5,7 +5,7 @@ import warnings
 import torch
 
 from ._loader import CUSIG_SIG_BACKPROP, CUSIG_SIGNATURE
-from .data_handlers import PathInput, SigInput, empty_like_input
+from .data_handlers import PathInput, SigInput, empty_like_input, on_device
 from .error_codes import err_msg
 from .param_checks import check_n_jobs, check_non_neg, check_type
 from .sig_length import infer_scalar_term, sig_length
@@ -39,13 +39,13 @@ def sig(path, degree, *, time_aug=False, lead_lag=False, end_time=1., horner=Tru
     out, out_ptr = empty_like_input(data, (n,))
     if data.batch_size == 0:
         return out
-    with torch.cuda.device(data.device):
+    with on_device(data.device):
         code = CUSIG_SIGNATURE[data.dtype](
             data.data_ptr, out_ptr, data.batch_size, data.data_dimension, data.data_length, degree,
             time_aug, lead_lag, end_time, horner, scalar_term, None, 0, 0, 0)
     if code:
         raise Exception("Error in pysiglib.sig: " + err_msg(code))
-    if torch.isnan(out).any().item() or torch.isinf(out).any().item():
+    if not torch.isfinite(out).all().item():
         warnings.warn(
             "sig produced NaN or Inf values. This is typically caused by paths with large increments, "
             "leading to numerical overflow. Consider normalizing your paths.", RuntimeWarning, stacklevel=2)
@@ -86,7 +86,7 @@ def sig_backprop(path, sig, sig_derivs, degree, *, time_aug=False, lead_lag=Fals
     if pdata.device != sdata.device:
         raise ValueError("path, sig and sig_derivs must be on the same device")
     check_n_jobs(n_jobs)
-    with torch.cuda.device(pdata.device):
+    with on_device(pdata.device):
         code = CUSIG_SIG_BACKPROP[pdata.dtype](
             pdata.data_ptr, out_ptr, gdata.data_ptr, sdata.data_ptr, pdata.batch_size, pdata.data_dimension,
             pdata.data_length, degree, time_aug, lead_lag, end_time, scalar_term, None, 0, 0, 0)
