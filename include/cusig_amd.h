@@ -199,6 +199,8 @@ CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
+/* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */
+CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: how increments reach the waves: -1 automatic, 0 scalar loads, 1 LDS-staged where compiled. */
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only

@@ -154,7 +154,7 @@ def main():
                              "int64_t, int, int64_t, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T))
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
-                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int);" % (T, D, N, tail, K, zs, T, T, T, T))
+                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))
         lines.append("")
         lines.append("#if !defined(__HIP_DEVICE_COMPILE__)   // the launcher table is host data")
         lines.append("static const KernelEntry kEntries_%02d[] = {" % fi)

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "../../include/cusig_amd.h"
+#include "sig_chen_adjoint.h"
 #include "sig_host.h"
 #include "sig_kernels.h"
 #include "sig_registry.h"
@@ -255,9 +256,27 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
     const int64_t simds = simd_count();
     if (waves <= 0 || waves * 2 > simds) return 1;
     int64_t g = int64_t(std::min(waves_per_simd, 2)) * simds / waves;
-    g = std::min<int64_t>(g, 8);
+    g = std::min<int64_t>(g, 32);
     g = std::min<int64_t>(g, L / 48);
     if (sig_bytes_all_paths > 0) g = std::min<int64_t>(g, int64_t((uint64_t(256) << 20) / sig_bytes_all_paths));
+    return int(std::max<int64_t>(g, 1));
+}
+
+// The backward sweep can be cut in time as well: the state at the end of segment g is the Chen product of the
+// segment signatures up to g, and the adjoint of that state is the upstream gradient pulled back through the product
+// with the remaining segments.  That costs a segmented forward sweep, two chains of Chen products and one product
+// adjoint, all over (path, segment) rows, so it is only taken when whole-path sweeps leave at least half of the
+// SIMDs idle and the paths are long; the aim is two waves per SIMD.
+static int g_force_bwd_segments = 0;   // tuning hook (0 = automatic)
+
+static int choose_bwd_segments(int64_t waves, int64_t L, uint64_t sig_bytes_all_paths)
+{
+    const int64_t simds = simd_count();
+    if (waves <= 0 || waves * 2 > simds) return 1;
+    int64_t g = 2 * simds / waves;
+    g = std::min<int64_t>(g, 64);
+    g = std::min<int64_t>(g, L / 32);
+    if (sig_bytes_all_paths > 0) g = std::min<int64_t>(g, int64_t((uint64_t(64) << 20) / sig_bytes_all_paths));
     return int(std::max<int64_t>(g, 1));
 }
 
@@ -391,16 +410,17 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         p.nseg = nseg;
         p.batch = int64_t(batch) * nseg;
         T* segs = nullptr;
-        T* tmp[2] = {nullptr, nullptr};
+        T* folds = nullptr;
         if (nseg == 1) {
             p.out = out; p.out_stride = int64_t(s.stride); p.scalar = sc;
         } else {
             const uint64_t row_elems = checked_mul(batch, n_coef, "segment signatures");
-            segs = static_cast<T*>(workspace(2, checked_mul(checked_mul(row_elems, uint64_t(nseg), "segment signatures"), sizeof(T), "segment signatures")));
-            if (nseg > 2) {
-                T* t2 = static_cast<T*>(workspace(3, checked_mul(checked_mul(row_elems, 2, "segment signatures"), sizeof(T), "segment signatures")));
-                tmp[0] = t2; tmp[1] = t2 + row_elems;
-            }
+            const uint64_t bytes = checked_mul(checked_mul(row_elems, uint64_t(nseg), "segment signatures"), sizeof(T), "segment signatures");
+            segs = static_cast<T*>(workspace(2, bytes));
+            // every halving step's rows, one step after the other: at most nseg + log2(nseg) rows per path
+            if (nseg > 2)
+                folds = static_cast<T*>(workspace(3, checked_mul(checked_mul(row_elems, uint64_t(nseg) + 32, "segment signatures"),
+                                                                 sizeof(T), "segment signatures")));
             p.out = segs; p.out_stride = int64_t(n_coef); p.scalar = 0;
         }
         e = pick_variant(false, e, total_waves(geom, p.batch));
@@ -408,22 +428,22 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         SIG_HIP(e->fwd(p));
         timer.stop();
         if (nseg > 1) {
-            const T* acc = segs;
-            int64_t acc_stride = int64_t(n_coef) * nseg;
-            for (int g = 1; g < nseg; ++g) {
-                const bool last = g == nseg - 1;
-                T* dst = last ? out : tmp[(g - 1) & 1];
-                const int64_t b_stride = int64_t(n_coef) * nseg, c_stride = last ? int64_t(s.stride) : int64_t(n_coef);
-                const T* rhs = segs + uint64_t(g) * n_coef;
-                launch_indexed(n_coef, n_coef, batch, [&](auto ix, dim3 grid) {
+            // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches
+            const T* src = segs;
+            T* next = folds;
+            for (int m = nseg; m > 1; m = (m + 1) / 2) {
+                const bool last = m == 2;
+                const int half = (m + 1) / 2;
+                T* dst = last ? out : next;
+                launch_indexed(n_coef, n_coef, batch * uint64_t(half), [&](auto ix, dim3 grid) {
                     using I = decltype(ix);
-                    hipLaunchKernelGGL((sig_combine_kernel<T, I>), grid, dim3(kBlock), 0, stream, acc, rhs, dst,
-                                       int64_t(batch), DivBy<I>(s.d_aug), I(n_coef), acc_stride, b_stride, c_stride, 0, 0,
-                                       last ? sc : 0);
+                    hipLaunchKernelGGL((chen_fold_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, src, dst, int64_t(batch), m,
+                                       last ? int64_t(s.stride) : int64_t(n_coef) * half, last ? sc : 0, DivBy<I>(s.d_aug),
+                                       I(n_coef));
                 });
                 SIG_HIP(hipGetLastError());
-                acc = dst;
-                acc_stride = int64_t(n_coef);
+                src = dst;
+                next += batch * n_coef * uint64_t(half);
             }
         }
         exit_sync(stream);
@@ -477,7 +497,65 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         BwdParams p;
         p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
         p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
-        e = pick_variant(true, e, total_waves(make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0), int64_t(batch)));
+        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0);
+        const uint64_t n_coef = s.full_len - 1;
+        const KernelEntry* ef = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch);
+        int nseg = (!ef || degree > uint64_t(kCombMaxLevels)) ? 1
+                   : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
+                                              : choose_bwd_segments(total_waves(geom, int64_t(batch)), int64_t(s.L),
+                                                                    batch * n_coef * sizeof(T));
+        if (nseg > 1) {
+            const int64_t lseg = (int64_t(s.L) + nseg - 1) / nseg;
+            nseg = int((int64_t(s.L) + lseg - 1) / lseg);
+        }
+        if (nseg > 1) {
+            // (path, segment) rows, scalar-free: segment signatures, their running products from the left (the state
+            // at each segment's end), from the right (what follows each segment), and the adjoints of the states
+            const int64_t lseg = (int64_t(s.L) + nseg - 1) / nseg;
+            const uint64_t rows = checked_mul(batch, uint64_t(nseg), "segment signatures");
+            const uint64_t bytes = checked_mul(checked_mul(rows, n_coef, "segment signatures"), sizeof(T), "segment signatures");
+            T* segs = static_cast<T*>(workspace(2, bytes));
+            T* left = static_cast<T*>(workspace(8, bytes));
+            T* right = static_cast<T*>(workspace(9, bytes));
+            T* adj = static_cast<T*>(workspace(10, bytes));
+            const int64_t n = int64_t(n_coef);
+            FwdParams f;
+            f.inc = inc; f.batch = int64_t(rows); f.L = int64_t(s.L); f.d = int(s.d_aug); f.stream = stream;
+            f.lseg = lseg; f.nseg = nseg; f.out = segs; f.out_stride = n; f.scalar = 0;
+            const TreeGeom fgeom = make_geom(int(s.d_aug), ef->N - ef->tail, ef->k, ef->D > 0);
+            ef = pick_variant(false, ef, total_waves(fgeom, f.batch));
+            SIG_HIP(ef->fwd(f));
+            // both scans by doubling: ceil(log2(nseg)) launches, ping-ponging between two scratch copies
+            int steps = 0;
+            while ((1 << steps) < nseg) ++steps;
+            T* scratch = steps > 1 ? static_cast<T*>(workspace(11, checked_mul(bytes, steps > 2 ? 4 : 2, "segment signatures")))
+                                   : nullptr;
+            const uint64_t buf = rows * n_coef;
+            const T* xsrc = segs;
+            const T* zsrc = segs;
+            for (int k = 0; k < steps; ++k) {
+                const bool last = k == steps - 1;
+                T* xdst = last ? left : scratch + uint64_t(k & 1) * 2 * buf;
+                T* zdst = last ? right : scratch + (uint64_t(k & 1) * 2 + 1) * buf;
+                launch_indexed(n_coef, n_coef, 2 * rows, [&](auto ix, dim3 grid) {
+                    using I = decltype(ix);
+                    hipLaunchKernelGGL((chen_scan_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, xsrc, zsrc, xdst, zdst,
+                                       int64_t(batch), nseg, 1 << k, k == 0 ? 1 : 0, DivBy<I>(s.d_aug), I(n_coef));
+                });
+                xsrc = xdst;
+                zsrc = zdst;
+            }
+            SIG_HIP(hipGetLastError());
+            SigShape rs;
+            rs.n_coef = n_coef; rs.stride = n_coef; rs.off = 0;
+            SharedRows up;
+            up.share = nseg; up.stride = int64_t(s.stride); up.off = sc;
+            launch_combine_bwd<T>(sig_derivs, adj, nullptr, nullptr, right, rows, s.d_aug, degree, rs, stream, 1, up, 1);
+            SIG_HIP(hipGetLastError());
+            p.sig = left; p.gsig = adj; p.sig_stride = n; p.scalar = 0;
+            p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
+        }
+        e = pick_variant(true, e, total_waves(geom, p.batch));
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->bwd(p));
         timer.stop();
@@ -559,6 +637,8 @@ CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
 
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
+
+CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force_bwd_segments = segments; }
 
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
 

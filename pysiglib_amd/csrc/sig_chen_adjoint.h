@@ -20,6 +20,8 @@ namespace sigamd {
 // are set to dC by sig_combine_bwd_init_kernel first and receive their parts through atomics.
 // identity = 0 drops the dC_t[w] terms: the adjoint of the product without its "+ A + B" part, sum_l A_l (x) B_{t-l},
 // which is what the tensor logarithm is built from.
+// The rows of dC may be laid out differently from the others (stride dc_stride, dc_off leading slots) and shared:
+// item b reads row b / dc_share.  families = 1 computes dA only (dB and A are not touched).
 constexpr int kCombChunk = 256;
 constexpr int kCombMaxLevels = 64;
 template <typename I>
@@ -61,13 +63,13 @@ static CombBwdPlan<I> make_comb_plan(uint64_t d, uint64_t degree)
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_bwd_init_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, int64_t batch, I init_len, int64_t stride, int off,
-    int identity)
+    int identity, int64_t dc_share, int64_t dc_stride, int dc_off, int families)
 {
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < init_len; r += I(gridDim.x) * kBlock) {
-            const T v = identity ? dC[b * stride + off + r] : T(0);
+            const T v = identity ? dC[(b / dc_share) * dc_stride + dc_off + r] : T(0);
             dA[b * stride + off + r] = v;
-            dB[b * stride + off + r] = v;
+            if (families > 1) dB[b * stride + off + r] = v;
         }
     }
 }
@@ -75,12 +77,13 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_init_kernel(
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, const T* __restrict__ A,
-    const T* __restrict__ B, int64_t batch, CombBwdPlan<I> plan, int64_t stride, int off, int identity)
+    const T* __restrict__ B, int64_t batch, CombBwdPlan<I> plan, int64_t stride, int off, int identity,
+    int64_t dc_share, int64_t dc_stride, int dc_off, int families)
 {
     const int N = plan.degree;
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
-        const T* g = dC + b * stride + off;
-        for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < 2 * plan.items; it += I(gridDim.x) * kBlock) {
+        const T* g = dC + (b / dc_share) * dc_stride + dc_off;
+        for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < I(families) * plan.items; it += I(gridDim.x) * kBlock) {
             const bool fam_b = it >= plan.items;
             const I i2 = fam_b ? it - plan.items : it;
             int t = 1;
@@ -121,7 +124,10 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
             T* dst = (fam_b ? dB : dA) + b * stride + off + r;
             if (plan.parts[t] == 1) *dst = (identity ? g[r] : T(0)) + (s0 + s1);
             else dev_add(dst, s0 + s1);
-            if (off && it == 0) { dA[b * stride] = T(0); dB[b * stride] = T(0); }
+            if (off && it == 0) {
+                dA[b * stride] = T(0);
+                if (families > 1) dB[b * stride] = T(0);
+            }
         }
     }
 }
@@ -144,11 +150,20 @@ static SigShape sig_shape(uint64_t dimension, uint64_t degree, bool scalar_term,
     return s;
 }
 
+// how the rows of dC are found when they differ from the other operands' layout
+struct SharedRows {
+    int64_t share = 1;      // consecutive items reading one row
+    int64_t stride = -1;    // < 0: same stride and offset as the other operands
+    int off = 0;
+};
+
 // launches the adjoint of the Chen product (both kernels) on `stream`
 template <typename T>
 static void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint64_t batch, uint64_t dimension,
-                               uint64_t degree, const SigShape& s, hipStream_t stream, int identity = 1)
+                               uint64_t degree, const SigShape& s, hipStream_t stream, int identity = 1,
+                               SharedRows dc = SharedRows(), int families = 2)
 {
+    if (dc.stride < 0) { dc.stride = int64_t(s.stride); dc.off = s.off; }
     if (degree > uint64_t(kCombMaxLevels)) throw std::runtime_error("sig_combine_backprop_cuda: degree too high");
     launch_indexed(3 * s.n_coef + 1024, 1, batch, [&](auto ix, dim3) {      // 2 * items <= 2 n (1 + degree / kCombChunk)
         using I = decltype(ix);
@@ -156,11 +171,12 @@ static void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B
         if (plan.init_len > 0)
             launch_indexed(0, uint64_t(plan.init_len), batch, [&](auto, dim3 grid) {
                 hipLaunchKernelGGL((sig_combine_bwd_init_kernel<T, I>), grid, dim3(kBlock), 0, stream, dC, dA, dB,
-                                   int64_t(batch), plan.init_len, int64_t(s.stride), s.off, identity);
+                                   int64_t(batch), plan.init_len, int64_t(s.stride), s.off, identity, dc.share, dc.stride,
+                                   dc.off, families);
             });
-        launch_indexed(0, 2 * uint64_t(plan.items), batch, [&](auto, dim3 grid) {
+        launch_indexed(0, uint64_t(families) * uint64_t(plan.items), batch, [&](auto, dim3 grid) {
             hipLaunchKernelGGL((sig_combine_bwd_kernel<T, I>), grid, dim3(kBlock), 0, stream, dC, dA, dB, A, B, int64_t(batch),
-                               plan, int64_t(s.stride), s.off, identity);
+                               plan, int64_t(s.stride), s.off, identity, dc.share, dc.stride, dc.off, families);
         });
     });
 }

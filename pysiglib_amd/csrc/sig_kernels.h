@@ -450,8 +450,14 @@ template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
     T* __restrict__ dzinc, int64_t batch, int64_t L, int d_rt, int64_t sig_stride, int scalar,
-    int use_lds)
+    int use_lds, int nseg, int64_t lseg)
 {
+    // `batch` counts (path, time segment) items: item vb = path * nseg + segment walks the increments of steps
+    // [segment * lseg, min(L, (segment + 1) * lseg)) backwards, starting from the state `sig[vb]` (signature of the
+    // path up to the segment's end) and the adjoint `gsig[vb]` (gradient w.r.t. that state).  nseg == 1 is the
+    // plain whole-path sweep.  Steps are counted locally (count - 1 .. 0) so that every wave-level decision stays
+    // uniform; when several items share a wave all of them run lseg steps and the surplus steps of a shorter
+    // (last) segment, which walk into the previous segment, are dead: their gradient is not emitted.
     using Tr = Tree<T, D, N, TAIL, K>;
     using Ad = TreeAdj<T, D, N, TAIL, K>;
     using Cx = LaneCtx<T, D, N, TAIL, K>;
@@ -529,8 +535,22 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + wave_in_block;
         b_first = (slots > 1) ? wave * slots : (wave / cx.G.wpp);
     }
-    int cs = 0;                 // steps already written into the current chunk
-    int64_t t_chunk = L - 1;    // step held by chunk slot 0
+    // this lane's item
+    const int64_t it_path = cx.id.b / nseg;
+    const int64_t it_t0 = (cx.id.b % nseg) * lseg;
+    const int64_t it_ns = (L - it_t0 < lseg) ? L - it_t0 : lseg;
+    const int64_t count = slots > 1 ? lseg : it_ns;       // steps this wave runs (wave-uniform)
+    // element index of dz[path][step of local index 0][0] of an item, and its number of live steps
+    auto item_base = [&](int64_t vb, int64_t& live) -> int64_t {
+        const int64_t pth = vb / nseg, s0 = (vb % nseg) * lseg;
+        live = (L - s0 < lseg) ? L - s0 : lseg;
+        return (pth * L + s0 + live - count) * d;
+    };
+    [[maybe_unused]] int64_t wave_live;
+    const int64_t wave_base = item_base(b_first < batch ? b_first : batch - 1, wave_live);   // used when the wave serves one item
+    const int64_t lane_base = (it_path * L + it_t0 + it_ns - count) * d;
+    int cs = 0;                     // steps already written into the current chunk
+    int64_t t_chunk = count - 1;    // local step held by chunk slot 0
 
     auto reduce_chunk = [&](int n_slots) {
         wave_lds_sync();
@@ -559,15 +579,20 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
             }
             T sum = (s0 + s1) + (s2 + s3);
             const int slot = r / RS, j = r % RS;
+            const int64_t tl = t_chunk - slot;      // local step of this row
             if constexpr (PAIR) {
                 const int letter = j + RS * sg;      // the two halves of a row belong to different letters
-                if (letter < d && b_first < batch) dev_add(&dzinc[(b_first * L + (t_chunk - slot)) * d + letter], sum);
+                if (letter < d && b_first < batch) dev_add(&dzinc[wave_base + tl * d + letter], sum);
             } else if (slots > 1) {
                 const int64_t bb = b_first + sg;
-                if (bb < batch) dev_add(&dzinc[(bb * L + (t_chunk - slot)) * d + j], sum);
+                if (bb < batch) {
+                    int64_t live;
+                    const int64_t base = item_base(bb, live);
+                    if (tl >= count - live) dev_add(&dzinc[base + tl * d + j], sum);
+                }
             } else {
                 sum += __shfl_xor(sum, 1);      // the two halves of a row sit in neighbouring lanes
-                if (sg == 0 && b_first < batch) dev_add(&dzinc[(b_first * L + (t_chunk - slot)) * d + j], sum);
+                if (sg == 0 && b_first < batch) dev_add(&dzinc[wave_base + tl * d + j], sum);
             }
         }
         wave_lds_sync();
@@ -625,7 +650,8 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 t_chunk = t - 1;
             }
         } else {
-            T* grow_t = dzinc + (cx.id.b * L + t) * d;
+            T* grow_t = dzinc + lane_base + t * d;
+            const bool live_step = t >= count - it_ns;
             if (use_lds) {
                 if (active) {
 #pragma unroll
@@ -643,10 +669,14 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                     const T v = wbuf[e];
                     wbuf[e] = T(0);
                     const int64_t bb = b_first + e / d;
-                    if (bb < batch) dev_add(&dzinc[(bb * L + t) * d + e % d], v);
+                    if (bb < batch) {
+                        int64_t live;
+                        const int64_t base = item_base(bb, live);
+                        if (t >= count - live) dev_add(&dzinc[base + t * d + e % d], v);
+                    }
                 }
                 wave_lds_sync();
-            } else if (active) {
+            } else if (active && live_step) {
                 if constexpr (TAIL >= 2) {
 #pragma unroll
                     for (int j = 0; j < Tr::DD; ++j) dev_add(&grow_t[j], dz.dj[j]);
@@ -660,7 +690,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         }
     };
 
-    const T* row = inc + (cx.id.b * (L + 2) + L) * d;      // row of the last step
+    const T* row = inc + (it_path * (L + 2) + it_t0 + it_ns) * d;      // row of the item's last step
     if constexpr (ZL) {
         static_assert(WIDE, "staged increments need the wide layout");
         T* lds_wave = lds + kWavesPerBlock * Plan::tile_elems(Tr::DD) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
@@ -668,13 +698,13 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         if constexpr (NG <= 3) {
             static_for<0, NG - 1>([&](auto gc) {
                 if (cx.id.g == decltype(gc)::value)
-                    sweep_staged<-1, decltype(gc)::value * K, Tr>(cx, row, L - 1, L, lds_wave, do_step);
+                    sweep_staged<-1, decltype(gc)::value * K, Tr>(cx, row, count - 1, count, lds_wave, do_step);
             });
         } else {
-            sweep_staged<-1, -1, Tr>(cx, row, L - 1, L, lds_wave, do_step);
+            sweep_staged<-1, -1, Tr>(cx, row, count - 1, count, lds_wave, do_step);
         }
     } else {
-        sweep_direct<-1, false, Cx, typename Tr::Inc>(cx, row, L - 1, L, do_step);
+        sweep_direct<-1, false, Cx, typename Tr::Inc>(cx, row, count - 1, count, do_step);
     }
 }
 
@@ -864,37 +894,104 @@ __device__ __forceinline__ WordPos<I> word_pos(I r, I d)
 // (siglib/cpsig/cp_sig_combine.h:35-66).  One thread per output coefficient; rows
 // of A, B, C may have different strides and C may carry a leading scalar slot.
 // ---------------------------------------------------------------------------
+// coefficient r of A (x) B for scalar-free rows a, b
+template <typename T, typename I>
+__device__ __forceinline__ T chen_coefficient(const T* __restrict__ a, const T* __restrict__ bb, I r, const DivBy<I>& dv)
+{
+    const I d = I(dv.d);
+    const WordPos<I> p = word_pos<I>(r, d);
+    T acc = a[p.lo + p.w] + bb[p.lo + p.w];
+    // split after k letters, k = t-1 .. 1: the prefix loses its last letter, which becomes the
+    // leading letter of the suffix
+    I pre = p.w, suf = 0, pw = 1;       // pw = d^(t-k-1)
+    I a_lo = p.lo, a_sz = p.size;       // level k+1 of A
+    I b_lo = 0;                         // start of level t-k of B
+    for (int k = p.t - 1; k >= 1; --k) {
+        const I q = dv.quot(pre);
+        suf += (pre - q * d) * pw;
+        pw *= d;
+        pre = q;
+        a_sz = dv.quot(a_sz);
+        a_lo -= a_sz;
+        acc = fmadd(a[a_lo + pre], bb[b_lo + suf], acc);
+        b_lo += pw;
+    }
+    return acc;
+}
+
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void sig_combine_kernel(
     const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int64_t batch, DivBy<I> dv,
     I sig_len /* sum_{k=1..degree} d^k */, int64_t a_stride, int64_t b_stride, int64_t c_stride,
     int a_off, int b_off, int c_off)
 {
-    const I d = I(dv.d);
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * a_stride + a_off;
         const T* bb = B + b * b_stride + b_off;
         T* c = C + b * c_stride;
         for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T acc = a[p.lo + p.w] + bb[p.lo + p.w];
-            // split after k letters, k = t-1 .. 1: the prefix loses its last letter, which becomes the
-            // leading letter of the suffix
-            I pre = p.w, suf = 0, pw = 1;       // pw = d^(t-k-1)
-            I a_lo = p.lo, a_sz = p.size;       // level k+1 of A
-            I b_lo = 0;                         // start of level t-k of B
-            for (int k = p.t - 1; k >= 1; --k) {
-                const I q = dv.quot(pre);
-                suf += (pre - q * d) * pw;
-                pw *= d;
-                pre = q;
-                a_sz = dv.quot(a_sz);
-                a_lo -= a_sz;
-                acc = fmadd(a[a_lo + pre], bb[b_lo + suf], acc);
-                b_lo += pw;
-            }
-            c[c_off + r] = acc;
+            c[c_off + r] = chen_coefficient<T, I>(a, bb, r, dv);
             if (c_off && r == 0) c[0] = T(1);
+        }
+    }
+}
+
+// One doubling step of two scans over the segment signatures seg[path][g] (rows of sig_len coefficients, nseg per
+// path): the running products from the left, X[g] = seg[0] (x) .. (x) seg[g], and the products of everything to the
+// right, Z[g] = seg[g+1] (x) .. (x) seg[nseg-1] (the unit for the last segment; a unit is a zero row).  A step with
+// shift s maps X[g] <- X[g-s] (x) X[g] and Z[g] <- Z[g] (x) Z[g+s], rows beyond either end being units; after the
+// steps s = 1, 2, 4, .. < nseg both scans are complete.  In the first step (z_first) the rows of Z are read from the
+// segment signatures one row further right.  Work item: (scan, path, g) on blockIdx.y, coefficients on blockIdx.x.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void chen_scan_step_kernel(
+    const T* __restrict__ xsrc, const T* __restrict__ zsrc, T* __restrict__ xdst, T* __restrict__ zdst, int64_t paths,
+    int nseg, int shift, int z_first, DivBy<I> dv, I sig_len)
+{
+    const int64_t rows = paths * nseg;
+    for (int64_t y = blockIdx.y; y < 2 * rows; y += gridDim.y) {
+        const bool right = y >= rows;
+        const int64_t row = right ? y - rows : y;
+        const int g = int(row % nseg);
+        const T* a = nullptr;
+        const T* bb = nullptr;
+        T* c = (right ? zdst : xdst) + row * int64_t(sig_len);
+        if (!right) {
+            if (g - shift >= 0) a = xsrc + (row - shift) * int64_t(sig_len);
+            bb = xsrc + row * int64_t(sig_len);
+        } else {
+            const int g0 = g + z_first;      // row holding Z[g]
+            if (g0 < nseg) a = zsrc + (row + z_first) * int64_t(sig_len);
+            if (g0 + shift < nseg) bb = zsrc + (row + z_first + shift) * int64_t(sig_len);
+        }
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            T v;
+            if (a && bb) v = chen_coefficient<T, I>(a, bb, r, dv);
+            else if (a) v = a[r];
+            else if (bb) v = bb[r];
+            else v = T(0);
+            c[r] = v;
+        }
+    }
+}
+
+// One halving step of the ordered product of m rows per path: dst[path][j] = src[path][2j] (x) src[path][2j+1]
+// (a copy when the right neighbour does not exist).  dst rows have their own stride between paths and may carry a
+// leading scalar slot, so the last step (m = 2) can write the caller's signature directly.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void chen_fold_step_kernel(
+    const T* __restrict__ src, T* __restrict__ dst, int64_t paths, int m, int64_t dst_path_stride, int dst_off,
+    DivBy<I> dv, I sig_len)
+{
+    const int half = (m + 1) / 2;
+    for (int64_t y = blockIdx.y; y < paths * half; y += gridDim.y) {
+        const int64_t path = y / half;
+        const int j = int(y % half);
+        const T* a = src + (path * m + 2 * j) * int64_t(sig_len);
+        const T* bb = 2 * j + 1 < m ? a + int64_t(sig_len) : nullptr;
+        T* c = dst + path * dst_path_stride + int64_t(j) * int64_t(sig_len);
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+            c[dst_off + r] = bb ? chen_coefficient<T, I>(a, bb, r, dv) : a[r];
+            if (dst_off && r == 0) c[0] = T(1);
         }
     }
 }

@@ -77,7 +77,7 @@ hipError_t launch_tree_bwd(const BwdParams& p)
     hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
                        static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,
-                       p.sig_stride, p.scalar, use_lds);
+                       p.sig_stride, p.scalar, use_lds, p.nseg, p.lseg > 0 ? p.lseg : p.L);
     return hipGetLastError();
 }
 

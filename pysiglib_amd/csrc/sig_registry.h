@@ -27,6 +27,8 @@ struct BwdParams {
     int64_t sig_stride;
     int scalar;
     hipStream_t stream;
+    int nseg = 1;           // time segments per path; batch counts (path, segment) items
+    int64_t lseg = 0;       // steps per segment (0: L)
 };
 
 typedef hipError_t (*FwdFn)(const FwdParams&);

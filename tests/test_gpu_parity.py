@@ -273,7 +273,7 @@ def test_reused_buffers_and_repeatability(P, oracle):
                            oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)) <= 1e-10
 
 
-@pytest.mark.parametrize("segments", [1, 2, 3, 5, 8])
+@pytest.mark.parametrize("segments", [1, 2, 3, 5, 8, 13, 32])
 def test_time_segmented_forward(P, oracle, segments):
     """The forward sweep may split paths into time segments folded with Chen's identity; every split must agree."""
     import ctypes
@@ -297,6 +297,40 @@ def test_time_segmented_forward(P, oracle, segments):
                 assert level_rel_err(got[:, off:], ref[:, off:], d_aug, deg) <= TOL[dtype], (shape, aug, dtype)
     finally:
         L.CUSIG.cusig_amd_force_segments(0)
+
+
+@pytest.mark.parametrize("segments", [2, 3, 7, 16])
+def test_time_segmented_backward(P, oracle, segments):
+    """The backward sweep may be cut in time too (states from running Chen products of the segment signatures,
+    adjoints from the product's pullback); every split must give the whole-path gradient."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_bwd_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_bwd_segments.restype = None
+    rng = np.random.default_rng(140 + segments)
+    cases = [((3, 41, 3, 4), {}, False),                                  # a few paths per wave
+             ((2, 64, 10, 5), {}, True),                                  # wide layout, paired reduction in f64
+             ((2, 33, 2, 6), dict(time_aug=True, lead_lag=True), False),
+             ((5, 18, 6, 3), {}, True),
+             ((1, 100, 5, 7), {}, False),
+             ((70, 23, 2, 3), dict(lead_lag=True), True),                 # many paths per wave, ragged last segment
+             ((9, 50, 2, 2), {}, False),
+             ((2, 40, 20, 3), {}, False),                                 # run-time-dimension kernel
+             ((2, 37, 40, 2), {}, True),                                  # too wide for the reduction tile
+             ((3, 130, 6, 4), dict(time_aug=True), False)]
+    try:
+        L.CUSIG.cusig_amd_force_bwd_segments(segments)
+        for (shape, aug, scalar_term) in cases:
+            b, length, d, deg = shape
+            for dtype in (np.float64, np.float32):
+                x = (np.cumsum(rng.standard_normal(shape[:3]), axis=1) * (0.8 / np.sqrt(length))).astype(dtype)
+                ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+                g = rng.standard_normal(ref.shape).astype(dtype)
+                want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+                got = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+                assert bwd_rel_err(got, want) <= TOL[dtype], (shape, aug, dtype, bwd_rel_err(got, want))
+    finally:
+        L.CUSIG.cusig_amd_force_bwd_segments(0)
 
 
 @pytest.mark.parametrize("shape,dtype", [
