@@ -33,8 +33,9 @@ TRAFFIC_BYTES = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # a step is about 1 ms: the defaults run long enough for the GPU clocks to settle under load
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-configs", action="store_true", help="also time configs 2-4 (reported under 'configs')")
     ap.add_argument("--ops", action="store_true",
@@ -288,7 +289,7 @@ def main():
     if args.all_configs:
         for k in (2, 3, 4):
             r = Runner(k, torch, np, loader, cfgmod)
-            n = 3 if k == 3 else max(5, args.steps)
+            n = 3 if k == 3 else max(5, min(args.steps, 50))
             wall, kms, name = time_calls(r.forward, torch, loader, 1, n)
             tf = r.flops_fwd / (kms * 1e-3) / 1e12
             configs["C%d" % k] = {"signatures_per_s": r.c["batch"] / wall, "call_ms": wall * 1e3, "kernel": name,

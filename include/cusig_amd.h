@@ -197,6 +197,11 @@ CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree)
 CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
+/* Whether the last signature_cuda_* call on this thread stored a NaN or an infinity: 1 yes, 0 no, -1 not
+ * reported (the call failed, or ran in stream-ordered mode, where the answer is not known at return).  The
+ * kernels that store the result set the flag, so a caller who must warn about overflow (pysiglib/sig.py:299-311
+ * scans the result for NaN and Inf) needs no pass of its own over the output.  No counterpart in the reference. */
+CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */

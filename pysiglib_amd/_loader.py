@@ -27,6 +27,8 @@ CUSIG.cusig_shutdown.argtypes = ()
 CUSIG.cusig_shutdown.restype = None
 CUSIG.cusig_amd_sig_length.argtypes = (c_uint64, c_uint64)
 CUSIG.cusig_amd_sig_length.restype = c_uint64
+CUSIG.cusig_amd_last_sig_nonfinite.argtypes = ()
+CUSIG.cusig_amd_last_sig_nonfinite.restype = c_int
 CUSIG.cusig_amd_set_profiling.argtypes = (c_int,)
 CUSIG.cusig_amd_set_profiling.restype = None
 CUSIG.cusig_amd_last_kernel_ms.argtypes = ()

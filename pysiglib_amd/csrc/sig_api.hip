@@ -171,6 +171,8 @@ void* workspace(int slot, size_t bytes)
     return w.ptr;
 }
 
+static int* g_flag_host = nullptr;     // pinned word the forward kernels report NaN / infinity through
+
 static void release_workspaces() noexcept
 {
     std::lock_guard<std::mutex> lk(g_ws_mutex);
@@ -184,6 +186,10 @@ static void release_workspaces() noexcept
         }
     }
     g_ws.clear();
+    if (g_flag_host) {
+        (void)hipHostFree(g_flag_host);
+        g_flag_host = nullptr;
+    }
     (void)hipGetLastError();
 }
 
@@ -229,6 +235,23 @@ static void entry_sync()
 static void exit_sync(hipStream_t stream)
 {
     if (!g_stream_ordered) SIG_HIP(hipStreamSynchronize(stream));
+}
+
+// ---------------------------------------------------------------------------
+// NaN / infinity report of the forward pass
+// ---------------------------------------------------------------------------
+// The kernels that store a signature set a flag when a stored value is not finite, so that callers who must warn
+// about overflow (pysiglib/sig.py:299-311 scans the result for NaN and Inf) need no pass of their own over the
+// output.  The flag is one word of pinned host memory mapped into the device: it costs nothing to read after the
+// call's final synchronisation.  Calls are serialised by the workspace mutex; each thread keeps its own last answer.
+static thread_local int tl_sig_nonfinite = -1;     // -1: the last forward call on this thread did not report
+
+static int* nonfinite_flag()
+{
+    if (!g_flag_host) SIG_HIP(hipHostMalloc(reinterpret_cast<void**>(&g_flag_host), 64, hipHostMallocMapped | hipHostMallocPortable));
+    int* dev = nullptr;
+    SIG_HIP(hipHostGetDevicePointer(reinterpret_cast<void**>(&dev), g_flag_host, 0));
+    return dev;
 }
 
 // ---------------------------------------------------------------------------
@@ -368,6 +391,15 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
     hipStream_t stream = nullptr;
     entry_sync();   // inputs may have been produced on any stream
 
+    // everything below runs under the workspace mutex: one flag serves all callers
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    tl_sig_nonfinite = -1;
+    int* flag = nullptr;
+    if (!g_stream_ordered) {
+        flag = nonfinite_flag();
+        *g_flag_host = 0;
+    }
+
     const int sc = scalar_term ? 1 : 0;
     if (s.len_aug <= 1) {
         if (s.stride)
@@ -379,18 +411,17 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                                int64_t(batch), int64_t(1), 1);
     } else if (s.d_aug == 1) {
         hipLaunchKernelGGL((dim_one_fwd_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, path, out,
-                           int64_t(batch), int64_t(length), int(degree), sc);
+                           int64_t(batch), int64_t(length), int(degree), sc, flag);
     } else if (degree == 1) {
         const T time_step = end_time / T(s.len_aug - 1);
         hipLaunchKernelGGL((degree_one_fwd_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
                            path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
-                           int(lead_lag), time_step, sc);
+                           int(lead_lag), time_step, sc, flag);
     } else {
         const KernelEntry* e = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch);
         if (!e)
             throw std::runtime_error("signature_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
-        std::lock_guard<std::mutex> lk(g_ws_mutex);
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;    // staged sweeps read whole chunks past either end
         T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
@@ -412,7 +443,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         T* segs = nullptr;
         T* folds = nullptr;
         if (nseg == 1) {
-            p.out = out; p.out_stride = int64_t(s.stride); p.scalar = sc;
+            p.out = out; p.out_stride = int64_t(s.stride); p.scalar = sc; p.nonfinite = flag;
         } else {
             const uint64_t row_elems = checked_mul(batch, n_coef, "segment signatures");
             const uint64_t bytes = checked_mul(checked_mul(row_elems, uint64_t(nseg), "segment signatures"), sizeof(T), "segment signatures");
@@ -439,7 +470,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                     using I = decltype(ix);
                     hipLaunchKernelGGL((chen_fold_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, src, dst, int64_t(batch), m,
                                        last ? int64_t(s.stride) : int64_t(n_coef) * half, last ? sc : 0, DivBy<I>(s.d_aug),
-                                       I(n_coef));
+                                       I(n_coef), last ? flag : nullptr);
                 });
                 SIG_HIP(hipGetLastError());
                 src = dst;
@@ -447,10 +478,12 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             }
         }
         exit_sync(stream);
+        if (flag) tl_sig_nonfinite = *g_flag_host;
         return;
     }
     SIG_HIP(hipGetLastError());
     exit_sync(stream);
+    if (flag) tl_sig_nonfinite = *g_flag_host;
 }
 
 // ---------------------------------------------------------------------------
@@ -645,6 +678,8 @@ CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = 
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
 
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
+
+CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {

@@ -1,6 +1,8 @@
 // Kernels of the signature hot path: increment pre-pass, tree forward sweep,
 // tree reverse sweep, increment-gradient fold-back and the closed-form cases.
 #pragma once
+#include <limits>
+
 #include "sig_tree.h"
 
 namespace sigamd {
@@ -121,6 +123,10 @@ struct LaneCtx {
         return o;
     }
 };
+
+// NaN or infinity
+__device__ __forceinline__ bool not_finite(double v) { return !(__builtin_fabs(v) <= std::numeric_limits<double>::max()); }
+__device__ __forceinline__ bool not_finite(float v) { return !(__builtin_fabsf(v) <= std::numeric_limits<float>::max()); }
 
 // Nothing may be scheduled across this point: the loads above it are issued
 // before any of the arithmetic below it.
@@ -313,8 +319,9 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d_rt,
-    int64_t out_stride, int scalar, int nseg, int64_t lseg)
+    int64_t out_stride, int scalar, int nseg, int64_t lseg, int* __restrict__ nonfinite)
 {
+    // `nonfinite` (may be null): set to 1 when any stored value is NaN or infinite.
     // `batch` counts (path, time segment) pairs: item vb = path * nseg + segment sweeps the
     // increments [segment * lseg, min(L, (segment + 1) * lseg)) and stores the signature of
     // that piece in row vb of `out`.  nseg == 1 is the plain whole-path sweep.
@@ -358,12 +365,15 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     if (!cx.id.active) return;
     T* o = out + cx.id.b * out_stride;
     if (scalar && cx.id.q == 0 && cx.id.g == 0) o[0] = T(1);
+    // chk stays 0 while every value is finite: x * 0 is NaN for x = NaN or +-Inf
+    T chk = T(0);
     // chain nodes are stored by the lane whose remaining prefix letters are 0
     {
         int64_t rest = 1;   // d^(M-l)
 #pragma unroll
         for (int l = M; l >= 1; --l) {
             if (cx.id.g == 0 && cx.id.q % rest == 0) o[cx.level_off(l, scalar) + cx.id.q / rest] = S.c[l - 1];
+            chk = fmadd(S.c[l - 1], T(0), chk);
             rest *= d;
         }
     }
@@ -380,6 +390,9 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
             }
         }
     });
+#pragma unroll
+    for (int i = 0; i < Tr::SUB; ++i) chk = fmadd(S.s[i], T(0), chk);      // unused slots hold 0
+    if (nonfinite && !(chk == T(0))) *nonfinite = 1;
 }
 
 // ---------------------------------------------------------------------------
@@ -535,20 +548,31 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + wave_in_block;
         b_first = (slots > 1) ? wave * slots : (wave / cx.G.wpp);
     }
+    // path and first step of an item (whole paths skip the divisions)
+    auto split_item = [&](int64_t vb, int64_t& pth, int64_t& s0) {
+        if (nseg == 1) {
+            pth = vb;
+            s0 = 0;
+        } else {
+            pth = vb / nseg;
+            s0 = (vb - pth * nseg) * lseg;
+        }
+    };
     // this lane's item
-    const int64_t it_path = cx.id.b / nseg;
-    const int64_t it_t0 = (cx.id.b % nseg) * lseg;
-    const int64_t it_ns = (L - it_t0 < lseg) ? L - it_t0 : lseg;
-    const int64_t count = slots > 1 ? lseg : it_ns;       // steps this wave runs (wave-uniform)
+    int64_t it_path, it_t0;
+    split_item(cx.id.b, it_path, it_t0);
+    const int64_t it_ns = nseg == 1 ? L : (L - it_t0 < lseg) ? L - it_t0 : lseg;
+    const int64_t count = nseg == 1 ? L : slots > 1 ? lseg : it_ns;       // steps this wave runs (wave-uniform)
     // element index of dz[path][step of local index 0][0] of an item, and its number of live steps
     auto item_base = [&](int64_t vb, int64_t& live) -> int64_t {
-        const int64_t pth = vb / nseg, s0 = (vb % nseg) * lseg;
+        int64_t pth, s0;
+        split_item(vb, pth, s0);
         live = (L - s0 < lseg) ? L - s0 : lseg;
         return (pth * L + s0 + live - count) * d;
     };
-    [[maybe_unused]] int64_t wave_live;
-    const int64_t wave_base = item_base(b_first < batch ? b_first : batch - 1, wave_live);   // used when the wave serves one item
     const int64_t lane_base = (it_path * L + it_t0 + it_ns - count) * d;
+    // when the wave serves one item every lane holds that item, so its base is the lane's
+    const int64_t wave_base = lane_base;
     int cs = 0;                     // steps already written into the current chunk
     int64_t t_chunk = count - 1;    // local step held by chunk slot 0
 
@@ -762,7 +786,7 @@ __global__ __launch_bounds__(kBlock) void zero_kernel(T* __restrict__ out, int64
 template <typename T>
 __global__ __launch_bounds__(kBlock) void degree_one_fwd_kernel(
     const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int d_raw,
-    int time_aug, int lead_lag, T time_step, int scalar)
+    int time_aug, int lead_lag, T time_step, int scalar, int* __restrict__ nonfinite)
 {
     const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
     const int64_t len = lead_lag ? 2 * len_raw - 1 : len_raw;
@@ -783,13 +807,15 @@ __global__ __launch_bounds__(kBlock) void degree_one_fwd_kernel(
             v = x[(len_raw - 1) * d_raw + cr] - x[cr];
         }
         out[e] = v;
+        if (nonfinite && not_finite(v)) *nonfinite = 1;
     }
 }
 
 // effective dimension 1: level k = Delta^k / k!
 template <typename T>
 __global__ __launch_bounds__(kBlock) void dim_one_fwd_kernel(
-    const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int degree, int scalar)
+    const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int degree, int scalar,
+    int* __restrict__ nonfinite)
 {
     for (int64_t b = int64_t(blockIdx.x) * kBlock + threadIdx.x; b < batch; b += int64_t(gridDim.x) * kBlock) {
         const T inc = path[b * len_raw + len_raw - 1] - path[b * len_raw];
@@ -800,6 +826,7 @@ __global__ __launch_bounds__(kBlock) void dim_one_fwd_kernel(
             v *= inc / T(k);
             *o++ = v;
         }
+        if (nonfinite && not_finite(v)) *nonfinite = 1;      // once a level is not finite, so is the last
     }
 }
 
@@ -980,7 +1007,7 @@ __global__ __launch_bounds__(kBlock) void chen_scan_step_kernel(
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void chen_fold_step_kernel(
     const T* __restrict__ src, T* __restrict__ dst, int64_t paths, int m, int64_t dst_path_stride, int dst_off,
-    DivBy<I> dv, I sig_len)
+    DivBy<I> dv, I sig_len, int* __restrict__ nonfinite)
 {
     const int half = (m + 1) / 2;
     for (int64_t y = blockIdx.y; y < paths * half; y += gridDim.y) {
@@ -990,7 +1017,9 @@ __global__ __launch_bounds__(kBlock) void chen_fold_step_kernel(
         const T* bb = 2 * j + 1 < m ? a + int64_t(sig_len) : nullptr;
         T* c = dst + path * dst_path_stride + int64_t(j) * int64_t(sig_len);
         for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            c[dst_off + r] = bb ? chen_coefficient<T, I>(a, bb, r, dv) : a[r];
+            const T v = bb ? chen_coefficient<T, I>(a, bb, r, dv) : a[r];
+            c[dst_off + r] = v;
+            if (nonfinite && not_finite(v)) *nonfinite = 1;
             if (dst_off && r == 0) c[0] = T(1);
         }
     }

@@ -34,7 +34,7 @@ hipError_t launch_tree_fwd(const FwdParams& p)
     }
     hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
-                       p.out_stride, p.scalar, p.nseg, p.lseg);
+                       p.out_stride, p.scalar, p.nseg, p.lseg, p.nonfinite);
     return hipGetLastError();
 }
 

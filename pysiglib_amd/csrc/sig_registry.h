@@ -15,6 +15,7 @@ struct FwdParams {
     hipStream_t stream;
     int nseg;        // time segments per path; batch counts (path, segment) items
     int64_t lseg;    // increments per segment
+    int* nonfinite = nullptr;   // device-visible flag set when a stored value is NaN or infinite (may be null)
 };
 
 struct BwdParams {

@@ -4,7 +4,7 @@ import warnings
 
 import torch
 
-from ._loader import CUSIG_SIG_BACKPROP, CUSIG_SIGNATURE
+from ._loader import CUSIG, CUSIG_SIG_BACKPROP, CUSIG_SIGNATURE
 from .data_handlers import PathInput, SigInput, empty_like_input, on_device
 from .error_codes import err_msg
 from .param_checks import check_n_jobs, check_non_neg, check_type
@@ -45,7 +45,9 @@ def sig(path, degree, *, time_aug=False, lead_lag=False, end_time=1., horner=Tru
             time_aug, lead_lag, end_time, horner, scalar_term, None, 0, 0, 0)
     if code:
         raise Exception("Error in pysiglib.sig: " + err_msg(code))
-    if not torch.isfinite(out).all().item():
+    # the kernels that store the signature report NaN / Inf themselves; scan only when they could not
+    reported = CUSIG.cusig_amd_last_sig_nonfinite()
+    if reported == 1 or (reported < 0 and not torch.isfinite(out).all().item()):
         warnings.warn(
             "sig produced NaN or Inf values. This is typically caused by paths with large increments, "
             "leading to numerical overflow. Consider normalizing your paths.", RuntimeWarning, stacklevel=2)

@@ -209,6 +209,47 @@ def test_batch_dims_views_and_warnings(P, oracle):
         P.sig(torch.full((1, 3, 2), 1e200, dtype=torch.float64, device=DEV).cumsum(1), 3)
 
 
+def test_overflow_report(P):
+    """The kernels that store the signature flag NaN / Inf themselves (the reference scans the result,
+    pysiglib/sig.py:299-310): the report must agree with a scan on every forward route."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_stream_ordered.restype = None
+    rng = np.random.default_rng(77)
+    shapes = [(3, 20, 3, 4), (2, 40, 10, 5), (70, 9, 2, 3), (2, 12, 20, 3), (2, 12, 40, 2),     # packed, wide, many per wave, generic
+              (4, 9, 1, 5), (4, 9, 6, 1), (3, 1, 4, 3)]                                       # dimension one, degree one, single point
+    for segments in (0, 3):
+        try:
+            L.CUSIG.cusig_amd_force_segments(segments)
+            for shape in shapes:
+                for dtype in (torch.float64, torch.float32):
+                    big = 1e200 if dtype == torch.float64 else 1e30
+                    for kind in ("finite", "overflow", "nan"):
+                        x = torch.as_tensor(rng.standard_normal(shape[:3]), dtype=dtype, device=DEV)
+                        if kind == "overflow":
+                            x[shape[0] - 1] *= big        # only the last path
+                        elif kind == "nan":
+                            x[0, shape[1] // 2, 0] = float("nan")
+                        with warnings.catch_warnings(record=True) as caught:
+                            warnings.simplefilter("always")
+                            out = P.sig(x, shape[3], scalar_term=bool(shape[0] % 2))
+                        warned = any(issubclass(w.category, RuntimeWarning) for w in caught)
+                        assert L.CUSIG.cusig_amd_last_sig_nonfinite() in (0, 1)
+                        assert warned == (not bool(torch.isfinite(out).all())), (shape, dtype, kind, segments)
+        finally:
+            L.CUSIG.cusig_amd_force_segments(0)
+    # stream-ordered calls cannot know at return: no report, the wrapper scans
+    try:
+        L.CUSIG.cusig_amd_set_stream_ordered(1)
+        with pytest.warns(RuntimeWarning):
+            P.sig(torch.full((1, 3, 2), 1e200, dtype=torch.float64, device=DEV).cumsum(1), 3)
+        assert L.CUSIG.cusig_amd_last_sig_nonfinite() == -1
+    finally:
+        L.CUSIG.cusig_amd_set_stream_ordered(0)
+
+
 def test_error_codes_through_the_abi(P):
     import ctypes
     from pysiglib_amd import _loader as L
