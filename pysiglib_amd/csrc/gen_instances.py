@@ -18,6 +18,12 @@ import os
 
 MAX_GENERIC_N = 16
 GENERIC_K = 4
+# Paths of many channels (beyond the specialised dimensions) at low degree: run-time-dimension kernels with more
+# letters per lane, (D, K) per direction; D = -1 is the wide layout.  Measured on MI355X for d = 18 .. 100:
+# forward: wide K 8 is fastest wherever it applies except for d close to 32, where packed K 32 wastes no lane;
+# backward: packed K 16.
+MANY_CHANNELS_MAX_N = 5
+MANY_CHANNELS = {"fwd": ((0, 32), (-1, 8)), "bwd": ((0, 16),)}
 
 # value budgets (signature values held per lane); backward holds state + adjoint
 BUDGET = {("f64", "fwd"): 100, ("f64", "bwd"): 60, ("f32", "fwd"): 170, ("f32", "bwd"): 100}
@@ -125,6 +131,9 @@ def main():
         for N in range(2, MAX_GENERIC_N + 1):
             for direction in ("fwd", "bwd"):
                 insts.append((T, 0, N, 1, GENERIC_K, direction, 1, 0))
+                if N <= MANY_CHANNELS_MAX_N:
+                    for (dd, kk) in MANY_CHANNELS[direction]:
+                        insts.append((T, dd, N, 1, kk, direction, 0, 0))
 
     # balance files by a rough compile-cost estimate
     def weight(i):
@@ -162,7 +171,8 @@ def main():
             is64 = 1 if T == "double" else 0
             zs = "true" if zl else "false"
             pol = STAGE_POLICY.get(("f64" if is64 else "f32", D, N, direction), 0)
-            name = "%s_%s_d%d_n%d_t%d_k%d%s" % (direction, "f64" if is64 else "f32", D, N, tail, K, "_lds" if zl else "")
+            name = "%s_%s_d%s_n%d_t%d_k%d%s" % (direction, "f64" if is64 else "f32", "0w" if D < 0 else str(D), N, tail, K,
+                                                "_lds" if zl else "")
             if direction == "fwd":
                 lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))

@@ -53,6 +53,7 @@ struct Table {
 
 // tuning hook: when set (tail > 0), prefer the compiled partition with this (tail, k)
 static int g_force_tail = 0, g_force_k = 0;
+static int g_force_run_time_wide = 0;   // with a forced partition: take the run-time-dimension kernel in the wide layout
 
 static const Table& table()
 {
@@ -78,16 +79,46 @@ static const KernelEntry* choose_entry(bool backward, bool f64, uint64_t d, uint
     return sweep_estimate(gen, int(d), int64_t(batch)) < 0.7 * sweep_estimate(spec, int(d), int64_t(batch)) ? gen : spec;
 }
 
+// Shapes without a specialised instance run a run-time-dimension kernel.  Its default carries few depth-1 letters
+// per lane, which suits small dimensions and high degrees.  Paths of many channels at low degree have variants
+// with more letters per lane (the chain work of a lane is shared by more top-level updates) and, for the forward
+// sweep, a wide-layout variant (one letter group of one path per wave, the group's increments arriving through
+// scalar loads) for paths with at least 48 word prefixes.  Which is fastest was measured for d = 18 .. 100:
+// forward: the wide variant, except near d = 32 where the packed 32-letter variant wastes no lane; backward: the
+// packed 16-letter variant.
+static const KernelEntry* pick_run_time_entry(bool backward, bool f64, int d, int degree)
+{
+    const auto& m = backward ? table().bwd : table().fwd;
+    auto packed = m.find(std::make_tuple(int(f64), 0, degree));
+    if (packed == m.end() || packed->second.empty()) return nullptr;
+    const KernelEntry* best = packed->second.front();
+    if (d < 12) return best;
+    for (const KernelEntry* e : packed->second)
+        if (e->k > best->k && !e->staged) best = e;       // the many-letter variant, if this degree has one
+    if (backward || (d >= 28 && d <= 32)) return best;
+    auto wide = m.find(std::make_tuple(int(f64), -1, degree));
+    if (wide != m.end() && !wide->second.empty() && ipow64(d, degree - 1) >= 48) best = wide->second.front();
+    return best;
+}
+
 static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64_t degree)
 {
     const auto& m = backward ? table().bwd : table().fwd;
     if (d <= 0x7fffffff && degree <= 0x7fffffff) {
         auto it = m.find(std::make_tuple(int(f64), int(d), int(degree)));
-        if (it == m.end()) it = m.find(std::make_tuple(int(f64), 0, int(degree)));
+        const bool run_time = it == m.end();
+        if (run_time) it = m.find(std::make_tuple(int(f64), 0, int(degree)));
         if (it != m.end() && !it->second.empty()) {
-            if (g_force_tail > 0)
-                for (const KernelEntry* e : it->second)
+            if (g_force_tail > 0) {
+                auto from = it;
+                if (run_time && g_force_run_time_wide && ipow64(int64_t(d), int(degree) - 1) >= 48) {
+                    auto w = m.find(std::make_tuple(int(f64), -1, int(degree)));
+                    if (w != m.end()) from = w;
+                }
+                for (const KernelEntry* e : from->second)
                     if (e->tail == g_force_tail && e->k == g_force_k && !e->staged) return e;
+            }
+            if (run_time) return pick_run_time_entry(backward, f64, int(d), int(degree));
             return it->second.front();
         }
     }
@@ -119,7 +150,7 @@ static double lane_step_cost(int d, int n, int tail, int k)
 // lone wave) and the chip-wide issue time of all waves' steps.  Returns a relative figure.
 static double sweep_estimate(const KernelEntry* e, int d, int64_t batch)
 {
-    const TreeGeom g = make_geom(d, e->N - e->tail, e->k, e->D > 0);
+    const TreeGeom g = make_geom(d, e->N - e->tail, e->k, e->D != 0);
     const double rounds = double(total_waves(g, batch)) / double(simd_count());
     const double per_step = lane_step_cost(d, e->N, e->tail, e->k) * (e->D > 0 ? 1.0 : 1.15);
     return per_step * std::max(1.0, rounds * 0.8);
@@ -428,7 +459,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
         // Few paths cannot fill the chip with whole-path sweeps: split every path into time segments,
         // sweep all (path, segment) pairs concurrently and fold the pieces with Chen's identity.
-        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0);
+        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
         int nseg = g_force_segments > 0
                              ? int(std::min<uint64_t>(uint64_t(g_force_segments), s.L))
                              : choose_segments(total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
@@ -530,7 +561,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         BwdParams p;
         p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
         p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
-        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D > 0);
+        const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
         const uint64_t n_coef = s.full_len - 1;
         const KernelEntry* ef = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch);
         int nseg = (!ef || degree > uint64_t(kCombMaxLevels)) ? 1
@@ -555,7 +586,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             FwdParams f;
             f.inc = inc; f.batch = int64_t(rows); f.L = int64_t(s.L); f.d = int(s.d_aug); f.stream = stream;
             f.lseg = lseg; f.nseg = nseg; f.out = segs; f.out_stride = n; f.scalar = 0;
-            const TreeGeom fgeom = make_geom(int(s.d_aug), ef->N - ef->tail, ef->k, ef->D > 0);
+            const TreeGeom fgeom = make_geom(int(s.d_aug), ef->N - ef->tail, ef->k, ef->D != 0);
             ef = pick_variant(false, ef, total_waves(fgeom, f.batch));
             SIG_HIP(ef->fwd(f));
             // both scans by doubling: ceil(log2(nseg)) launches, ping-ponging between two scratch copies
@@ -681,6 +712,8 @@ CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream
 
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
 
+CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { g_force_run_time_wide = enabled; }
+
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {
     g_force_tail = tail;
@@ -694,7 +727,7 @@ CUSIG_AMD_API int cusig_amd_kernel_choice(int backward, int is_f64, uint64_t dim
     if (!e) return 0;
     if (tail) *tail = e->tail;
     if (k) *k = e->k;
-    if (specialised) *specialised = e->D != 0;
+    if (specialised) *specialised = e->D > 0;
     return 1;
 }
 

@@ -72,7 +72,7 @@ template <typename T, int D, int N, int TAIL, int K>
 struct LaneCtx {
     using Tr = Tree<T, D, N, TAIL, K>;
     static constexpr int M = Tr::M;
-    static constexpr bool WIDE = D > 0 && ipow64(D > 0 ? D : 1, M) >= 48;
+    static constexpr bool WIDE = D > 0 ? ipow64(D > 0 ? D : 1, M) >= 48 : D < 0;
     int d;
     TreeGeom G;
     LaneId id;
@@ -82,7 +82,7 @@ struct LaneCtx {
     __device__ __forceinline__ void init(int d_rt, int64_t batch)
     {
         d = D > 0 ? D : d_rt;
-        G = make_geom(d, M, K, D > 0);
+        G = make_geom(d, M, K, D != 0);
         id = lane_id<WIDE>(G, batch);
         // idle lanes shadow a valid lane so that every load stays in bounds;
         // they never store and never contribute

@@ -21,7 +21,8 @@ hipError_t allow_lds(Kern kern, size_t bytes)
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 hipError_t launch_tree_fwd(const FwdParams& p)
 {
-    const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
+    const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);
+    if (D < 0 && !g.wide) return hipErrorInvalidConfiguration;     // the kernel was compiled for the wide layout
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
@@ -53,7 +54,8 @@ int fwd_waves_per_simd()
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
-    const TreeGeom g = make_geom(p.d, N - TAIL, K, D > 0);
+    const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);
+    if (D < 0 && !g.wide) return hipErrorInvalidConfiguration;     // the kernel was compiled for the wide layout
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;

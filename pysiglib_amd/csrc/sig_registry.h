@@ -35,7 +35,7 @@ struct BwdParams {
 typedef hipError_t (*FwdFn)(const FwdParams&);
 typedef hipError_t (*BwdFn)(const BwdParams&);
 
-// D == 0: run-time dimension.  Exactly one of fwd / bwd is set.
+// D == 0: run-time dimension, packed layout; D == -1: run-time dimension, wide layout.  Exactly one of fwd / bwd is set.
 struct KernelEntry {
     int is_f64, D, N, tail, k;
     int staged;      // 1: increments staged through LDS into VGPRs (wide layout, low occupancy)

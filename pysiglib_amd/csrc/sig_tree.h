@@ -14,7 +14,9 @@
 // (siglib/cpsig/cp_signature.h:464-499 forward, :1137-1187 backward) regrouped
 // per word; see the comments on fwd_step / pullback below.
 //
-// D > 0: compile-time path dimension.  D == 0: run-time dimension (TAIL must be 1).
+// D > 0: compile-time path dimension.  D == 0: run-time dimension (TAIL must be 1), lanes of several groups and
+// paths packed into waves.  D == -1: run-time dimension in the wide layout (every wave serves one letter group of
+// one path; needs d^M >= 48, which the host checks before it picks such a kernel).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

@@ -396,6 +396,43 @@ def test_extreme_shapes(P, oracle, shape, dtype):
     assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("shape", [
+    (3, 9, 13, 4), (2, 12, 20, 3), (5, 7, 30, 2), (2, 6, 32, 3), (3, 8, 50, 2), (4, 9, 40, 2), (2, 5, 18, 5), (2, 6, 100, 2),
+    (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_many_channel_shapes(P, oracle, shape, dtype):
+    """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
+    letter counts per lane and two lane layouts: every one of them against the oracle, forward and backward,
+    whole paths and time-split sweeps."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_bwd_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_bwd_segments.restype = None
+    b, length, d, deg = shape
+    rng = np.random.default_rng(b * 1000 + d * 10 + deg)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * 0.3).astype(dtype)
+    ref = oracle.signature(x, deg, n_jobs=-1)
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
+    try:
+        for segments in (0, 2):
+            L.CUSIG.cusig_amd_force_segments(segments)
+            L.CUSIG.cusig_amd_force_bwd_segments(segments)
+            got = P.sig(dev(x), deg).cpu().numpy()
+            assert level_rel_err(got, ref, d, deg) <= TOL[dtype], (shape, segments)
+            got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+            assert bwd_rel_err(got_b, want) <= TOL[dtype], (shape, segments)
+    finally:
+        L.CUSIG.cusig_amd_force_segments(0)
+        L.CUSIG.cusig_amd_force_bwd_segments(0)
+    xa = x[:, :, : min(d, 23)]
+    aug = dict(time_aug=True, lead_lag=(d <= 25))
+    refa = oracle.signature(xa, min(deg, 3), n_jobs=-1, **aug)
+    da = (2 * xa.shape[2] if aug["lead_lag"] else xa.shape[2]) + 1
+    assert level_rel_err(P.sig(dev(xa), min(deg, 3), **aug).cpu().numpy(), refa, da, min(deg, 3)) <= TOL[dtype]
+
+
 def test_wide_degree_one(P):
     x = torch.randn(3, 2, 200000, dtype=torch.float32, device=DEV)
     torch.testing.assert_close(P.sig(x, 1), x[:, 1] - x[:, 0])
