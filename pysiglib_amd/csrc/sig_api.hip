@@ -22,6 +22,7 @@
 
 #include "../../include/cusig_amd.h"
 #include "sig_chen_adjoint.h"
+#include "sig_degree2.h"
 #include "sig_host.h"
 #include "sig_kernels.h"
 #include "sig_registry.h"
@@ -350,6 +351,20 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
 }
 
 // ---------------------------------------------------------------------------
+// degree 2 in closed form (matrix cores): taken for paths of many channels, where no specialised sweep exists
+// ---------------------------------------------------------------------------
+static int g_force_degree2 = -1;    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
+
+// Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
+// forward from about 12 channels on and for small dimensions whenever the sweeps cannot fill the chip.
+static bool use_degree2(bool backward, uint64_t d_aug, uint64_t degree, uint64_t batch)
+{
+    if (degree != 2 || d_aug < 2 || d_aug > 0x7fff) return false;
+    if (g_force_degree2 >= 0) return g_force_degree2 != 0;
+    return backward || d_aug >= 12 || batch * 8 <= uint64_t(simd_count());
+}
+
+// ---------------------------------------------------------------------------
 // shared argument handling
 // ---------------------------------------------------------------------------
 static void validate_correction(const void* correction, uint64_t correction_len, uint64_t dimension,
@@ -448,6 +463,33 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         hipLaunchKernelGGL((degree_one_fwd_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
                            path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), time_step, sc, flag);
+    } else if (use_degree2(false, s.d_aug, degree, batch)) {
+        const int d = int(s.d_aug);
+        const int tiles = (d + 15) / 16, col_groups = (tiles + kDeg2Cols - 1) / kDeg2Cols;
+        const int64_t waves = int64_t(batch) * tiles * col_groups;
+        // A wave walks its time range four steps per iteration, each iteration waiting for its loads: long ranges are
+        // cut into slices that add into the output with atomics (d^2 atomics per slice against slice_len * d^2
+        // products).  Few paths: enough slices for two waves per SIMD; otherwise slices of 256 steps.
+        int64_t slices = waves * 2 <= simd_count() ? std::min<int64_t>(2 * simd_count() / waves, int64_t(s.L) / 64)
+                                                   : int64_t(s.L) / 256;
+        slices = std::max<int64_t>(slices, 1);
+        const int64_t slice_len = ((int64_t(s.L) + slices - 1) / slices + 3) / 4 * 4;
+        slices = (int64_t(s.L) + slice_len - 1) / slice_len;
+        if (slices > 1)
+            hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
+                               int64_t(batch * s.stride));
+        const int64_t total = waves * slices;
+        const int64_t blocks = (total + kWavesPerBlock - 1) / kWavesPerBlock;
+        if (blocks > 2147483647LL) throw std::runtime_error("signature_cuda: launch too large");
+        const T time_step = end_time / T(s.len_aug - 1);
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_fwd_f64" : "degree2_fwd_f32");
+        hipLaunchKernelGGL((degree2_fwd_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), 0, stream, path, out, int64_t(batch),
+                           int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, tiles,
+                           col_groups, int(slices), slice_len, slices > 1 ? nullptr : flag);
+        timer.stop();
+        if (slices > 1 && flag)
+            hipLaunchKernelGGL((finite_rows_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
+                               int64_t(batch * s.stride), flag);
     } else {
         const KernelEntry* e = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch);
         if (!e)
@@ -545,6 +587,31 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         hipLaunchKernelGGL((degree_one_bwd_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream,
                            sig_derivs, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), sc);
+    } else if (use_degree2(true, s.d_aug, degree, batch)) {
+        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        const int d = int(s.d_aug);
+        const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
+        T* h = static_cast<T*>(workspace(12, checked_mul(checked_mul(batch, s.d_aug, "increments"), sizeof(T), "increments")));
+        const T time_step = end_time / T(s.len_aug - 1);
+        hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug)), dim3(kBlock), 0, stream, path, sig_derivs, h,
+                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
+                           int64_t(s.stride), sc);
+        const int tiles = (d + 15) / 16, col_groups = (tiles + kDeg2Cols - 1) / kDeg2Cols;
+        const int64_t time_tiles = (int64_t(s.L) + 15) / 16;
+        const int64_t total = int64_t(batch) * time_tiles * col_groups;
+        const int64_t blocks = (total + kWavesPerBlock - 1) / kWavesPerBlock;
+        if (blocks > 2147483647LL) throw std::runtime_error("sig_backprop_cuda: launch too large");
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_bwd_f64" : "degree2_bwd_f32");
+        hipLaunchKernelGGL((degree2_bwd_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), 0, stream, path, sig_derivs, h, dzinc,
+                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
+                           int64_t(s.stride), sc, time_tiles, col_groups);
+        timer.stop();
+        hipLaunchKernelGGL((path_grad_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, dzinc, out,
+                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+        SIG_HIP(hipGetLastError());
+        exit_sync(stream);      // the workspaces stay locked until the kernels are done
+        return;
     } else {
         const KernelEntry* e = choose_entry(true, sizeof(T) == 8, s.d_aug, degree, batch);
         if (!e)
@@ -711,6 +778,8 @@ CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wi
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
 
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
+
+CUSIG_AMD_API void cusig_amd_force_degree2(int mode) noexcept { g_force_degree2 = mode; }
 
 CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { g_force_run_time_wide = enabled; }
 

@@ -1,0 +1,243 @@
+// Degree 2 in closed form, on the matrix cores.
+//
+// With X_t the (augmented) path, z_t = X_{t+1} - X_t its increments and L their number, the Horner recursion of
+// siglib/cpsig/cp_signature.h:464-499 unrolls at degree 2 to
+//     S1 = X_L - X_0,      S2[a][b] = sum_t U_t[a] * z_t[b],      U_t = (X_t + X_{t+1}) / 2 - X_0,
+// i.e. S2 = U^T Z: one (d x L) by (L x d) product per path, with no dependence between time steps.  Its pullback
+// (the level-2 part of siglib/cpsig/cp_signature.h:1137-1187 summed over the sweep) is
+//     dz_t = h + U_t (G2 - G2^T),      h = G1 + G2 S1,
+// an (L x d) by (d x d) product with the antisymmetric part of the level-2 gradient.  Both run as MFMA 16x16x4 tiles
+// (f32 and f64), operands built on the fly from the raw path: nothing is staged in HBM, lead-lag and time
+// augmentation are evaluated per element.  Used for paths of many channels, where the sweep kernels' per-step work
+// per lane is too small to run well.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "sig_kernels.h"
+
+namespace sigamd {
+
+// point t, channel c of the augmented path (siglib/cpsig/cp_path.h:46-62,262-279): lead-lag doubles the channels
+// (first half lags: it moves on odd steps; second half leads: it moves on even steps), time is the last channel
+template <typename T>
+__device__ __forceinline__ T aug_point(const T* __restrict__ x, int64_t t, int c, int d_raw, int time_aug, int lead_lag,
+                                       int d, T time_step)
+{
+    if (time_aug && c == d - 1) return T(t) * time_step;
+    if (!lead_lag) return x[t * d_raw + c];
+    return c < d_raw ? x[(t >> 1) * d_raw + c] : x[((t + 1) >> 1) * d_raw + (c - d_raw)];
+}
+
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<float> {
+    typedef float Acc __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ int row(int lk, int r) { return 4 * lk + r; }
+};
+template <>
+struct Mfma16<double> {
+    typedef double Acc __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ Acc mma(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ int row(int lk, int r) { return 4 * r + lk; }
+};
+
+// Tile conventions of the 16x16x4 instructions (checked on the device): lane l supplies A[i = l % 16][k = l / 16] and
+// B[k = l / 16][j = l % 16] and receives, in component r of the accumulator, C[i][j = l % 16] with
+// i = 4 * (l / 16) + r for f32 and i = 4 * r + l / 16 for f64 (Mfma16::row).
+constexpr int kDeg2Cols = 4;     // 16-wide column tiles per wave
+constexpr int kDeg2Unroll = 1;   // groups of 4 steps whose loads are in flight together (forward)
+
+// Forward.  One wave per (path, time slice, 16-row tile a, group of kDeg2Cols column tiles b); slices of a path add
+// into the output with atomics (the output is cleared first when there are several).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_fwd_kernel(
+    const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int d_raw, int time_aug, int lead_lag,
+    T time_step, int64_t out_stride, int scalar, int tiles, int col_groups, int slices, int64_t slice_len,
+    int* __restrict__ nonfinite)
+{
+    using M = Mfma16<T>;
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t per_path = int64_t(tiles) * col_groups * slices;
+    const int64_t b = wave / per_path;
+    if (b >= batch) return;
+    int64_t w = wave - b * per_path;
+    const int slice = int(w % slices);
+    w /= slices;
+    const int cg = int(w % col_groups);
+    const int ta = int(w / col_groups);
+    const T* x = path + b * len_raw * d_raw;
+    T* o = out + b * out_stride + scalar;
+
+    const int li = lane & 15, lk = lane >> 4;
+    const int a = ta * 16 + li;                      // row channel this lane feeds
+    const bool a_ok = a < d;
+    const T x0a = a_ok ? aug_point(x, 0, a, d_raw, time_aug, lead_lag, d, time_step) : T(0);
+    typename M::Acc acc[kDeg2Cols];
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) acc[j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+
+    const int nb = tiles - cg * kDeg2Cols < kDeg2Cols ? tiles - cg * kDeg2Cols : kDeg2Cols;     // column tiles in use
+    const int64_t t_begin = int64_t(slice) * slice_len;
+    const int64_t t_end = t_begin + slice_len < L ? t_begin + slice_len : L;
+    // kDeg2Unroll groups of 4 steps per iteration: all their loads are issued before the first product
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += 4 * kDeg2Unroll) {
+        T ua[kDeg2Unroll], zb[kDeg2Unroll][kDeg2Cols];
+#pragma unroll
+        for (int u = 0; u < kDeg2Unroll; ++u) {
+            const int64_t t = t0 + 4 * u + lk;
+            const bool t_ok = t < t_end;
+            ua[u] = T(0);
+            if (t_ok && a_ok) {
+                const T p0 = aug_point(x, t, a, d_raw, time_aug, lead_lag, d, time_step);
+                const T p1 = aug_point(x, t + 1, a, d_raw, time_aug, lead_lag, d, time_step);
+                ua[u] = T(0.5) * (p0 + p1) - x0a;
+            }
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) {
+                const int c = (cg * kDeg2Cols + j) * 16 + li;
+                zb[u][j] = T(0);
+                if (t_ok && c < d)
+                    zb[u][j] = aug_point(x, t + 1, c, d_raw, time_aug, lead_lag, d, time_step) -
+                               aug_point(x, t, c, d_raw, time_aug, lead_lag, d, time_step);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kDeg2Unroll; ++u) {
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j)
+                if (j < nb) acc[j] = M::mma(ua[u], zb[u][j], acc[j]);
+        }
+    }
+
+    T chk = T(0);
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) {
+        const int c = (cg * kDeg2Cols + j) * 16 + li;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = ta * 16 + M::row(lk, r);
+            if (row < d && c < d) {
+                T* dst = o + d + int64_t(row) * d + c;
+                if (slices > 1) dev_add(dst, acc[j][r]);
+                else *dst = acc[j][r];
+                chk = fmadd(acc[j][r], T(0), chk);
+            }
+        }
+    }
+    // level 1 and the scalar: written once per path
+    if (cg == 0 && slice == 0 && lk == 0 && a_ok) {
+        const T s1 = aug_point(x, L, a, d_raw, time_aug, lead_lag, d, time_step) - x0a;
+        o[a] = s1;
+        chk = fmadd(s1, T(0), chk);
+        if (scalar && a == 0) o[-1] = T(1);
+    }
+    if (nonfinite && !(chk == T(0))) *nonfinite = 1;
+}
+
+// Slices of one path accumulate with atomics: a sum of finite parts can still overflow, so the flag is set from the
+// finished rows.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void finite_rows_kernel(const T* __restrict__ rows, int64_t total, int* __restrict__ nonfinite)
+{
+    T chk = T(0);
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock)
+        chk = fmadd(rows[e], T(0), chk);
+    if (!(chk == T(0))) *nonfinite = 1;
+}
+
+// h[b][c] = G1[c] + sum_e G2[c][e] * S1[e]
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_h_kernel(
+    const T* __restrict__ path, const T* __restrict__ gsig, T* __restrict__ h, int64_t batch, int64_t len_raw, int d_raw,
+    int time_aug, int lead_lag, T time_step, int64_t sig_stride, int scalar)
+{
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < batch * d; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / d;
+        const int c = int(e - b * d);
+        const T* x = path + b * len_raw * d_raw;
+        const T* g = gsig + b * sig_stride + scalar;
+        T s0 = g[c], s1 = T(0);
+        int k = 0;
+        for (; k + 2 <= d; k += 2) {
+            const T v0 = aug_point(x, L, k, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k, d_raw, time_aug, lead_lag, d, time_step);
+            const T v1 = aug_point(x, L, k + 1, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k + 1, d_raw, time_aug, lead_lag, d, time_step);
+            s0 = fmadd(g[d + int64_t(c) * d + k], v0, s0);
+            s1 = fmadd(g[d + int64_t(c) * d + k + 1], v1, s1);
+        }
+        if (k < d)
+            s0 = fmadd(g[d + int64_t(c) * d + k],
+                       aug_point(x, L, k, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k, d_raw, time_aug, lead_lag, d, time_step), s0);
+        h[e] = s0 + s1;
+    }
+}
+
+// Backward: dz[b][t][c] = h[b][c] + sum_a U_t[a] * (G2[a][c] - G2[c][a]).  One wave per (path, 16 steps, group of
+// kDeg2Cols column tiles); the product runs over the channels a in steps of 4.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_bwd_kernel(
+    const T* __restrict__ path, const T* __restrict__ gsig, const T* __restrict__ h, T* __restrict__ dz, int64_t batch,
+    int64_t len_raw, int d_raw, int time_aug, int lead_lag, T time_step, int64_t sig_stride, int scalar, int64_t time_tiles,
+    int col_groups)
+{
+    using M = Mfma16<T>;
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    const int64_t per_path = time_tiles * col_groups;
+    const int64_t b = wave / per_path;
+    if (b >= batch) return;
+    const int64_t w = wave - b * per_path;
+    const int cg = int(w % col_groups);
+    const int64_t tt = w / col_groups;
+    const T* x = path + b * len_raw * d_raw;
+    const T* g2 = gsig + b * sig_stride + scalar + d;
+
+    const int li = lane & 15, lk = lane >> 4;
+    const int tiles = (d + 15) / 16;
+    const int nb = tiles - cg * kDeg2Cols < kDeg2Cols ? tiles - cg * kDeg2Cols : kDeg2Cols;     // column tiles in use
+    const int64_t t = tt * 16 + li;                  // step this lane feeds as a row of U
+    const bool t_ok = t < L;
+    typename M::Acc acc[kDeg2Cols];
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) acc[j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+
+    for (int a0 = 0; a0 < d; a0 += 4) {
+        const int a = a0 + lk;
+        const bool a_ok = a < d;
+        T ua = T(0);
+        if (t_ok && a_ok) {
+            const T p0 = aug_point(x, t, a, d_raw, time_aug, lead_lag, d, time_step);
+            const T p1 = aug_point(x, t + 1, a, d_raw, time_aug, lead_lag, d, time_step);
+            ua = T(0.5) * (p0 + p1) - aug_point(x, 0, a, d_raw, time_aug, lead_lag, d, time_step);
+        }
+#pragma unroll
+        for (int j = 0; j < kDeg2Cols; ++j) {
+            const int c = (cg * kDeg2Cols + j) * 16 + li;
+            T anti = T(0);
+            if (a_ok && c < d) anti = g2[int64_t(a) * d + c] - g2[int64_t(c) * d + a];
+            if (j < nb) acc[j] = M::mma(ua, anti, acc[j]);
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) {
+        const int c = (cg * kDeg2Cols + j) * 16 + li;
+        if (c >= d) continue;
+        const T hc = h[b * d + c];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t row = tt * 16 + M::row(lk, r);
+            if (row < L) dz[(b * L + row) * d + c] = acc[j][r] + hc;
+        }
+    }
+}
+
+}  // namespace sigamd

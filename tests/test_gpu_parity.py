@@ -433,6 +433,47 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
     assert level_rel_err(P.sig(dev(xa), min(deg, 3), **aug).cpu().numpy(), refa, da, min(deg, 3)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("shape,aug", [
+    ((3, 9, 2, 2), {}), ((2, 30, 5, 2), {}), ((4, 17, 16, 2), {}), ((2, 21, 17, 2), dict(time_aug=True)),
+    ((2, 13, 31, 2), dict(lead_lag=True)), ((3, 12, 33, 2), dict(time_aug=True, lead_lag=True)), ((1, 2, 70, 2), {}),
+    ((2, 700, 20, 2), {}),                      # few long paths: time slices adding into the output
+    ((1, 1500, 7, 2), dict(lead_lag=True)), ((70, 6, 65, 2), {}), ((2, 5, 130, 2), dict(time_aug=True))])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
+    """Degree 2 has a closed form in the path (S2 = U^T Z, pullback through the antisymmetric part of the level-2
+    gradient) that runs on the matrix cores; forced on for every dimension here and compared with the oracle's sweep."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_degree2.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_degree2.restype = None
+    b, length, d, deg = shape
+    rng = np.random.default_rng(b * 1000 + d * 10 + length)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (1.0 / np.sqrt(length))).astype(dtype)
+    d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    try:
+        # forced on, then forced off (the sweep kernels of degree 2 stay covered)
+        for mode, scalar_term in ((1, False), (1, True), (0, True)):
+            L.CUSIG.cusig_amd_force_degree2(mode)
+            ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+            off = 1 if scalar_term else 0
+            with warnings.catch_warnings():
+                warnings.simplefilter("error", RuntimeWarning)       # a finite result must not be reported as overflow
+                got = P.sig(dev(x), deg, scalar_term=scalar_term, **aug).cpu().numpy()
+            if scalar_term:
+                np.testing.assert_array_equal(got[:, 0], 1.0)
+            assert level_rel_err(got[:, off:], ref[:, off:], d_aug, deg) <= TOL[dtype], (shape, aug, scalar_term)
+            g = rng.standard_normal(ref.shape).astype(dtype)
+            want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+            got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+            assert bwd_rel_err(got_b, want) <= TOL[dtype], (shape, aug, scalar_term)
+        big = x.copy()
+        big[0] *= 1e200 if dtype == np.float64 else 1e30
+        with pytest.warns(RuntimeWarning):
+            P.sig(dev(big), deg, **aug)
+    finally:
+        L.CUSIG.cusig_amd_force_degree2(-1)
+
+
 def test_wide_degree_one(P):
     x = torch.randn(3, 2, 200000, dtype=torch.float32, device=DEV)
     torch.testing.assert_close(P.sig(x, 1), x[:, 1] - x[:, 0])
