@@ -23,10 +23,11 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 # known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
 # reports null instead of a stale figure.
 TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5_lds": 53.0e6,
-    "bwd_f64_d10_n5_t2_k5_lds": 152.0e6,
-    "fwd_f64_d3_n12_t4_k3": 462.6e6,
-    "fwd_f32_d17_n4_t1_k17": 323.0e6,
+    "fwd_f64_d10_n5_t2_k5_lds": 53.2e6,
+    "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
+    "fwd_f32_d5_n7_t4_k1_lds": 64.0e6,
+    "fwd_f64_d3_n12_t4_k3": 491.0e6,
+    "fwd_f32_d17_n4_t1_k17": 323.4e6,
 }
 
 
@@ -296,6 +297,29 @@ def main():
                                   "kernel_ms": kms, "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS[r.dtype]}
             del r
             torch.cuda.empty_cache()
+        # degree 2 on paths of many channels: closed form on the matrix cores (not a BASELINE workload)
+        db, dl, dd = 2048, 256, 64
+        xp = (torch.randn((db, dl, dd), dtype=torch.float32, device="cuda:0").cumsum(1) * 0.05).contiguous()
+        sg = torch.empty((db, dd + dd * dd), dtype=torch.float32, device="cuda:0")
+        gg = torch.randn_like(sg)
+        gx = torch.empty_like(xp)
+        fp = ctypes.POINTER(ctypes.c_float)
+
+        def d2_fwd():
+            loader.CUSIG_SIGNATURE["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), db, dd, dl, 2,
+                                              False, False, 1.0, True, False, None, 0, 0, 0)
+
+        def d2_bwd():
+            loader.CUSIG_SIG_BACKPROP["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(gx.data_ptr(), fp),
+                                                 ctypes.cast(gg.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), db, dd, dl,
+                                                 2, False, False, 1.0, False, None, 0, 0, 0)
+
+        mm_flops = 2.0 * db * (dl - 1) * dd * dd        # one (d x L)(L x d) resp. (L x d)(d x d) product per path
+        for tag, fn in (("D2 fwd f32 (2048,256,64) deg 2", d2_fwd), ("D2 bwd f32 (2048,256,64) deg 2", d2_bwd)):
+            wall, kms, name = time_calls(fn, torch, loader, 2, max(5, min(args.steps, 50)))
+            configs[tag] = {"signatures_per_s": db / wall, "call_ms": wall * 1e3, "kernel": name, "kernel_ms": kms,
+                            "tflops": mm_flops / (kms * 1e-3) / 1e12, "bound": "mfma",
+                            "roofline_frac": mm_flops / (kms * 1e-3) / 1e12 / PEAK_TFLOPS["float32"]}
 
     line = {
         "metric": "signatures/sec, (32,1000,10) deg 5 fwd+bwd, fp64, 1 GPU",
