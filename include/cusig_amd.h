@@ -219,6 +219,9 @@ CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: the closed-form degree-2 kernels (matrix cores): -1 automatic, 0 never, 1 whenever the degree is 2. */
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) CUSIG_AMD_NOEXCEPT;
+/* Tuning hook: 0 makes the degree-2 kernels build their operands straight from global memory instead of staging
+ * them through LDS (the path taken anyway when a chunk of all channels does not fit). */
+CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: with a forced partition, shapes served by a run-time-dimension kernel take its wide-layout variant. */
 CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: prefer the compiled lane partition (tail, k) where a shape has several; tail = 0 restores

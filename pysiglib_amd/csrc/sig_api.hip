@@ -354,6 +354,7 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
 // degree 2 in closed form (matrix cores): taken for paths of many channels, where no specialised sweep exists
 // ---------------------------------------------------------------------------
 static int g_force_degree2 = -1;    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
+static int g_degree2_staged = 1;    // tuning hook: 0 keeps the operands of the degree-2 products out of LDS
 
 // Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
 // forward from about 12 channels on and for small dimensions whenever the sweeps cannot fill the chip.
@@ -478,14 +479,32 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         if (slices > 1)
             hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
                                int64_t(batch * s.stride));
-        const int64_t total = waves * slices;
-        const int64_t blocks = (total + kWavesPerBlock - 1) / kWavesPerBlock;
-        if (blocks > 2147483647LL) throw std::runtime_error("signature_cuda: launch too large");
         const T time_step = end_time / T(s.len_aug - 1);
-        MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_fwd_f64" : "degree2_fwd_f32");
-        hipLaunchKernelGGL((degree2_fwd_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), 0, stream, path, out, int64_t(batch),
-                           int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, tiles,
-                           col_groups, int(slices), slice_len, slices > 1 ? nullptr : flag);
+        // operands staged through LDS: two slabs of `chunk` steps by 64 channels
+        const size_t row_bytes = size_t(kDeg2SlabStride) * sizeof(T) * 2;
+        int chunk = sizeof(T) == 8 ? 32 : 64;
+        while (chunk > 8 && chunk / 2 >= slice_len) chunk /= 2;
+        // with fewer than four row tiles some of a block's waves would idle and its slabs be mostly padding (measured:
+        // d = 64..256 1.4-1.5x faster staged, d <= 32 up to 3x slower)
+        const bool staged = g_degree2_staged != 0 && tiles >= kWavesPerBlock;
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? (staged ? "degree2_fwd_f64_lds" : "degree2_fwd_f64")
+                                                     : (staged ? "degree2_fwd_f32_lds" : "degree2_fwd_f32"));
+        if (staged) {
+            const int64_t row_groups = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
+            const int64_t blocks = int64_t(batch) * row_groups * col_groups * slices;
+            if (blocks > 2147483647LL) throw std::runtime_error("signature_cuda: launch too large");
+            hipLaunchKernelGGL((degree2_fwd_staged_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), chunk * row_bytes, stream, path,
+                               out, int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
+                               int64_t(s.stride), sc, tiles, col_groups, int(slices), slice_len, chunk,
+                               slices > 1 ? nullptr : flag);
+        } else {
+            const int64_t total = waves * slices;
+            const int64_t blocks = (total + kWavesPerBlock - 1) / kWavesPerBlock;
+            if (blocks > 2147483647LL) throw std::runtime_error("signature_cuda: launch too large");
+            hipLaunchKernelGGL((degree2_fwd_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), 0, stream, path, out, int64_t(batch),
+                               int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc,
+                               tiles, col_groups, int(slices), slice_len, slices > 1 ? nullptr : flag);
+        }
         timer.stop();
         if (slices > 1 && flag)
             hipLaunchKernelGGL((finite_rows_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
@@ -780,6 +799,8 @@ CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
 
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) noexcept { g_force_degree2 = mode; }
+
+CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) noexcept { g_degree2_staged = enabled; }
 
 CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { g_force_run_time_wide = enabled; }
 

@@ -139,6 +139,113 @@ __global__ __launch_bounds__(kBlock) void degree2_fwd_kernel(
     if (nonfinite && !(chk == T(0))) *nonfinite = 1;
 }
 
+// Forward, operands staged through LDS.  A block serves one (path, time slice, group of four 16-row tiles, group of
+// kDeg2Cols column tiles): its four waves own one row tile each and share the column group.  Per chunk of `chunk`
+// steps the block writes the U values of its 64 row channels and the Z values of its 64 column channels to LDS
+// (coalesced reads of the path, every element computed once per block), then every wave feeds its products from
+// LDS.  Slab rows are 80 words long so that the four step rows a fragment read touches fall into different banks.
+constexpr int kDeg2Slab = 16 * kDeg2Cols;       // channels per slab (64)
+constexpr int kDeg2SlabStride = kDeg2Slab + 16;
+static_assert(kBlock % kDeg2Slab == 0 && kWavesPerBlock == kDeg2Cols, "staging assumes 4 waves and 64-channel slabs");
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_fwd_staged_kernel(
+    const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int d_raw, int time_aug, int lead_lag,
+    T time_step, int64_t out_stride, int scalar, int tiles, int col_groups, int slices, int64_t slice_len, int chunk,
+    int* __restrict__ nonfinite)
+{
+    using M = Mfma16<T>;
+    extern __shared__ double lds_raw_d2[];
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    T* lds_u = reinterpret_cast<T*>(lds_raw_d2);
+    T* lds_z = lds_u + int64_t(chunk) * kDeg2SlabStride;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int row_groups = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int64_t per_path = int64_t(row_groups) * col_groups * slices;
+    const int64_t b = int64_t(blockIdx.x) / per_path;          // grid = batch * per_path: every block has a path
+    int64_t w = int64_t(blockIdx.x) - b * per_path;
+    const int slice = int(w % slices);
+    w /= slices;
+    const int cg = int(w % col_groups);
+    const int rg = int(w / col_groups);
+    const int ta = rg * kWavesPerBlock + wave;                  // this wave's row tile
+    const bool has_task = ta < tiles;
+    const T* x = path + b * len_raw * d_raw;
+    T* o = out + b * out_stride + scalar;
+
+    const int li = lane & 15, lk = lane >> 4;
+    typename M::Acc acc[kDeg2Cols];
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) acc[j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+    const int nb = tiles - cg * kDeg2Cols < kDeg2Cols ? tiles - cg * kDeg2Cols : kDeg2Cols;
+
+    // staging: a thread keeps one slab column and walks the chunk's rows
+    const int sc_col = threadIdx.x % kDeg2Slab, sc_row0 = threadIdx.x / kDeg2Slab;
+    const int cu = rg * kDeg2Slab + sc_col, cz = cg * kDeg2Slab + sc_col;
+    const T x0u = cu < d ? aug_point(x, 0, cu, d_raw, time_aug, lead_lag, d, time_step) : T(0);
+
+    const int64_t t_begin = int64_t(slice) * slice_len;
+    const int64_t t_end = t_begin + slice_len < L ? t_begin + slice_len : L;
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += chunk) {
+        __syncthreads();        // the previous chunk has been consumed
+        for (int r = sc_row0; r < chunk; r += kBlock / kDeg2Slab) {
+            const int64_t t = t0 + r;
+            T u = T(0), z = T(0);
+            if (t < t_end) {
+                if (cu < d)
+                    u = T(0.5) * (aug_point(x, t, cu, d_raw, time_aug, lead_lag, d, time_step) +
+                                  aug_point(x, t + 1, cu, d_raw, time_aug, lead_lag, d, time_step)) - x0u;
+                if (cz < d)
+                    z = aug_point(x, t + 1, cz, d_raw, time_aug, lead_lag, d, time_step) -
+                        aug_point(x, t, cz, d_raw, time_aug, lead_lag, d, time_step);
+            }
+            lds_u[r * kDeg2SlabStride + sc_col] = u;
+            lds_z[r * kDeg2SlabStride + sc_col] = z;
+        }
+        __syncthreads();
+        if (has_task) {
+            const T* pu = lds_u + lk * kDeg2SlabStride + wave * 16 + li;
+            const T* pz = lds_z + lk * kDeg2SlabStride + li;
+            for (int r0 = 0; r0 < chunk; r0 += 4) {
+                const T ua = pu[r0 * kDeg2SlabStride];
+                T zb[kDeg2Cols];
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) zb[j] = j < nb ? pz[r0 * kDeg2SlabStride + j * 16] : T(0);
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j)
+                    if (j < nb) acc[j] = M::mma(ua, zb[j], acc[j]);
+            }
+        }
+    }
+    if (!has_task) return;
+
+    T chk = T(0);
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) {
+        const int c = (cg * kDeg2Cols + j) * 16 + li;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = ta * 16 + M::row(lk, r);
+            if (row < d && c < d) {
+                T* dst = o + d + int64_t(row) * d + c;
+                if (slices > 1) dev_add(dst, acc[j][r]);
+                else *dst = acc[j][r];
+                chk = fmadd(acc[j][r], T(0), chk);
+            }
+        }
+    }
+    const int a = ta * 16 + li;
+    if (cg == 0 && slice == 0 && lk == 0 && a < d) {
+        const T s1 = aug_point(x, L, a, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, a, d_raw, time_aug, lead_lag, d, time_step);
+        o[a] = s1;
+        chk = fmadd(s1, T(0), chk);
+        if (scalar && a == 0) o[-1] = T(1);
+    }
+    if (nonfinite && !(chk == T(0))) *nonfinite = 1;
+}
+
 // Slices of one path accumulate with atomics: a sum of finite parts can still overflow, so the flag is set from the
 // finished rows.
 template <typename T>

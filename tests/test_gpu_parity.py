@@ -437,6 +437,7 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
     ((3, 9, 2, 2), {}), ((2, 30, 5, 2), {}), ((4, 17, 16, 2), {}), ((2, 21, 17, 2), dict(time_aug=True)),
     ((2, 13, 31, 2), dict(lead_lag=True)), ((3, 12, 33, 2), dict(time_aug=True, lead_lag=True)), ((1, 2, 70, 2), {}),
     ((2, 700, 20, 2), {}),                      # few long paths: time slices adding into the output
+    ((2, 600, 50, 2), {}), ((1, 300, 36, 2), dict(lead_lag=True)),      # the same with operands staged through LDS
     ((1, 1500, 7, 2), dict(lead_lag=True)), ((70, 6, 65, 2), {}), ((2, 5, 130, 2), dict(time_aug=True))])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
@@ -450,10 +451,14 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
     rng = np.random.default_rng(b * 1000 + d * 10 + length)
     x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (1.0 / np.sqrt(length))).astype(dtype)
     d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    L.CUSIG.cusig_amd_set_degree2_staged.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_degree2_staged.restype = None
     try:
-        # forced on, then forced off (the sweep kernels of degree 2 stay covered)
-        for mode, scalar_term in ((1, False), (1, True), (0, True)):
+        # forced on (operands staged through LDS where that applies, then straight from memory), then forced off
+        # (the sweep kernels of degree 2 stay covered)
+        for mode, scalar_term, staged in ((1, False, 1), (1, True, 0), (0, True, 1)):
             L.CUSIG.cusig_amd_force_degree2(mode)
+            L.CUSIG.cusig_amd_set_degree2_staged(staged)
             ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
             off = 1 if scalar_term else 0
             with warnings.catch_warnings():
@@ -472,6 +477,7 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
             P.sig(dev(big), deg, **aug)
     finally:
         L.CUSIG.cusig_amd_force_degree2(-1)
+        L.CUSIG.cusig_amd_set_degree2_staged(1)
 
 
 def test_wide_degree_one(P):
