@@ -20,10 +20,10 @@ MAX_GENERIC_N = 16
 GENERIC_K = 4
 # Paths of many channels (beyond the specialised dimensions) at low degree: run-time-dimension kernels with more
 # letters per lane, (D, K) per direction; D = -1 is the wide layout.  Measured on MI355X for d = 18 .. 100:
-# forward: wide K 8 is fastest wherever it applies except for d close to 32, where packed K 32 wastes no lane;
-# backward: packed K 16.
+# forward: wide K 8 is fastest wherever it applies (degree >= 3; degree 2 of that many channels runs in closed
+# form); backward: packed K 16.
 MANY_CHANNELS_MAX_N = 5
-MANY_CHANNELS = {"fwd": ((0, 32), (-1, 8)), "bwd": ((0, 16),)}
+MANY_CHANNELS = {"fwd": ((-1, 8),), "bwd": ((0, 16),)}
 
 # value budgets (signature values held per lane); backward holds state + adjoint
 BUDGET = {("f64", "fwd"): 100, ("f64", "bwd"): 60, ("f32", "fwd"): 170, ("f32", "bwd"): 100}
@@ -53,10 +53,14 @@ EXTRA = {
 
 def spec_shapes():
     """(D, N) pairs that get specialised kernels."""
-    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 5, 8: 5, 9: 4, 10: 5, 11: 4, 12: 4, 13: 3, 14: 3, 15: 3, 16: 4, 17: 4}
+    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 5, 8: 5, 9: 5, 10: 5, 11: 5, 12: 5}
+    caps.update({d: 4 for d in range(13, 33)})
+    caps.update({d: 3 for d in range(33, 49)})
     out = []
     for d, nmax in sorted(caps.items()):
         for n in range(2, nmax + 1):
+            if n == 2 and d >= 18:
+                continue        # degree 2 of that many channels always runs in closed form on the matrix cores
             out.append((d, n))
     return out
 

@@ -398,7 +398,8 @@ def test_extreme_shapes(P, oracle, shape, dtype):
 
 @pytest.mark.parametrize("shape", [
     (3, 9, 13, 4), (2, 12, 20, 3), (5, 7, 30, 2), (2, 6, 32, 3), (3, 8, 50, 2), (4, 9, 40, 2), (2, 5, 18, 5), (2, 6, 100, 2),
-    (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2)])
+    (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2),
+    (2, 6, 50, 3), (1, 5, 34, 4), (2, 5, 13, 5), (3, 40, 49, 3)])        # beyond the specialised table: run-time dimension
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_many_channel_shapes(P, oracle, shape, dtype):
     """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
@@ -478,6 +479,47 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
     finally:
         L.CUSIG.cusig_amd_force_degree2(-1)
         L.CUSIG.cusig_amd_set_degree2_staged(1)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_every_specialised_dimension_above_12(P, oracle, dtype):
+    """One small forward + backward per compiled (dimension, degree) instance that the grid above does not reach:
+    dimensions 13..48 at degree 3, 13..32 at degree 4, 9..12 at degree 5."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    C = L.CUSIG
+    C.cusig_amd_force_partition.argtypes = (ctypes.c_int, ctypes.c_int)
+    C.cusig_amd_force_partition.restype = None
+    rng = np.random.default_rng(5)
+    shapes = [(d, 3) for d in range(13, 49)] + [(d, 4) for d in range(13, 33)] + [(d, 5) for d in range(9, 13)]
+    tail, k, spec = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+
+    def pin(backward, d, deg):
+        # tiny batches would be handed to the run-time-dimension kernel: pin the instance's own partition
+        C.cusig_amd_force_partition(0, 0)
+        assert C.cusig_amd_kernel_choice(int(backward), int(dtype == np.float64), d, deg, tail, k, spec) == 1
+        assert spec.value == 1, (d, deg)
+        C.cusig_amd_force_partition(tail.value, k.value)
+
+    try:
+        C.cusig_amd_set_profiling(1)
+        for (d, deg) in shapes:
+            b, length = (2, 4) if d ** deg < 200000 else (1, 3)
+            x = (rng.standard_normal((b, length, d)) * 0.5).astype(dtype)
+            ref = oracle.signature(x, deg, n_jobs=-1)
+            pin(False, d, deg)
+            got = P.sig(dev(x), deg).cpu().numpy()
+            assert ("_d%d_n%d_" % (d, deg)) in C.cusig_amd_last_kernel_name().decode()
+            assert level_rel_err(got, ref, d, deg) <= TOL[dtype], (d, deg)
+            g = rng.standard_normal(ref.shape).astype(dtype)
+            want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
+            pin(True, d, deg)
+            got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+            assert ("_d%d_n%d_" % (d, deg)) in C.cusig_amd_last_kernel_name().decode()
+            assert bwd_rel_err(got_b, want) <= TOL[dtype], (d, deg)
+    finally:
+        C.cusig_amd_force_partition(0, 0)
+        C.cusig_amd_set_profiling(0)
 
 
 def test_wide_degree_one(P):
