@@ -53,9 +53,10 @@ EXTRA = {
 
 def spec_shapes():
     """(D, N) pairs that get specialised kernels."""
-    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 5, 8: 5, 9: 5, 10: 5, 11: 5, 12: 5}
-    caps.update({d: 4 for d in range(13, 33)})
-    caps.update({d: 3 for d in range(33, 49)})
+    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 6, 8: 6}
+    caps.update({d: 5 for d in range(9, 17)})
+    caps.update({d: 4 for d in range(17, 33)})
+    caps.update({d: 3 for d in range(33, 65)})
     out = []
     for d, nmax in sorted(caps.items()):
         for n in range(2, nmax + 1):

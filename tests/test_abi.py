@@ -84,8 +84,8 @@ def test_kernel_table(lib):
         for f64 in (0, 1):
             for (d, n) in ((10, 5), (5, 7), (3, 12), (17, 4)):
                 assert fn(bwd, f64, d, n, tail, k, spec) == 1 and spec.value == 1 and 1 <= tail.value < n
-            assert fn(bwd, f64, 37, 3, tail, k, spec) == 1 and spec.value == 1      # the table reaches d = 48 at degree 3
-            assert fn(bwd, f64, 57, 3, tail, k, spec) == 1 and spec.value == 0      # run-time-dimension kernel
+            assert fn(bwd, f64, 37, 3, tail, k, spec) == 1 and spec.value == 1      # the table reaches d = 64 at degree 3
+            assert fn(bwd, f64, 70, 3, tail, k, spec) == 1 and spec.value == 0      # run-time-dimension kernel
             assert fn(bwd, f64, 2, 40, tail, k, spec) == 0                           # beyond the compiled degrees
 
 

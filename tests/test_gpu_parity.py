@@ -399,7 +399,7 @@ def test_extreme_shapes(P, oracle, shape, dtype):
 @pytest.mark.parametrize("shape", [
     (3, 9, 13, 4), (2, 12, 20, 3), (5, 7, 30, 2), (2, 6, 32, 3), (3, 8, 50, 2), (4, 9, 40, 2), (2, 5, 18, 5), (2, 6, 100, 2),
     (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2),
-    (2, 6, 50, 3), (1, 5, 34, 4), (2, 5, 13, 5), (3, 40, 49, 3)])        # beyond the specialised table: run-time dimension
+    (2, 6, 70, 3), (1, 5, 34, 4), (2, 5, 17, 5), (3, 40, 65, 3)])        # beyond the specialised table: run-time dimension
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_many_channel_shapes(P, oracle, shape, dtype):
     """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
@@ -484,14 +484,15 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_every_specialised_dimension_above_12(P, oracle, dtype):
     """One small forward + backward per compiled (dimension, degree) instance that the grid above does not reach:
-    dimensions 13..48 at degree 3, 13..32 at degree 4, 9..12 at degree 5."""
+    dimensions 13..64 at degree 3, 13..32 at degree 4, 9..16 at degree 5, 7..8 at degree 6."""
     import ctypes
     from pysiglib_amd import _loader as L
     C = L.CUSIG
     C.cusig_amd_force_partition.argtypes = (ctypes.c_int, ctypes.c_int)
     C.cusig_amd_force_partition.restype = None
     rng = np.random.default_rng(5)
-    shapes = [(d, 3) for d in range(13, 49)] + [(d, 4) for d in range(13, 33)] + [(d, 5) for d in range(9, 13)]
+    shapes = ([(d, 3) for d in range(13, 65)] + [(d, 4) for d in range(13, 33)] + [(d, 5) for d in range(9, 17)] +
+              [(7, 6), (8, 6)])
     tail, k, spec = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
 
     def pin(backward, d, deg):
