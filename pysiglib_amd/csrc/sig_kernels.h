@@ -413,12 +413,15 @@ struct RedPlan {
     static constexpr int NG = D > 0 ? (D + K - 1) / K : 0;
     static constexpr bool PAIR = ZL && D > 0 && NG <= 3 && TAIL >= 2 && sizeof(T) == 8;
     static constexpr int kRows = int(16384 / (kRedStride * sizeof(T)));       // 31 (f64) / 63 (f32)
+    // Wider paths get a tile of their own size holding a single step (up to 64 rows f64 / 128 rows f32, 33 KB per
+    // wave): without it every lane of a wave would add into the same few LDS words.
+    static constexpr int kRowsWide = 2 * kRows + 2;
     __host__ __device__ static constexpr int rows_per_step(int d) { return PAIR ? (d + 1) / 2 : d; }
     // steps per chunk of the tile; 0: the path is too wide for the tile
     __host__ __device__ static constexpr int steps(int d)
     {
         const int r = rows_per_step(d);
-        return r > kRows ? 0 : (kRows / r > 8 ? 8 : kRows / r);
+        return r > kRowsWide ? 0 : r > kRows ? 1 : (kRows / r > 8 ? 8 : kRows / r);
     }
     __host__ __device__ static constexpr int64_t tile_elems(int d) { return int64_t(steps(d)) * rows_per_step(d) * kRedStride; }
 };
@@ -524,8 +527,8 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     // banks; own column: no atomic ever collides).  When the chunk is full each (row, column segment) is
     // summed by one lane and added to dz[path][step][letter] in HBM.  Column segments: the lanes of one path
     // when several whole paths share the wave, else two halves of the wave.  Paths too wide for the tile
-    // (d > 31 in f64, d > 63 in f32) fall back to a per-wave accumulator updated with LDS atomics, whose
-    // collisions are rare exactly because d is large.
+    // (d > 64 in f64, d > 128 in f32; up to half of that the tile holds several steps, beyond it a single one) fall
+    // back to a per-wave accumulator updated with LDS atomics.
     const int lane = threadIdx.x & (kWave - 1);
     const int wave_in_block = threadIdx.x >> 6;
     constexpr bool WIDE = Cx::WIDE;
