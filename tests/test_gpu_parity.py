@@ -523,6 +523,57 @@ def test_every_specialised_dimension_above_12(P, oracle, dtype):
         C.cusig_amd_set_profiling(0)
 
 
+def test_randomised_shapes(P, oracle):
+    """400 seeded random draws over the whole instance table: dimension, degree, batch, length, augmentations,
+    dtype, scalar term and forced time splits of both sweeps, each against the oracle."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    C = L.CUSIG
+    C.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    C.cusig_amd_force_bwd_segments.argtypes = (ctypes.c_int,)
+    C.cusig_amd_force_bwd_segments.restype = None
+    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 6, 8: 6}
+    caps.update({d: 5 for d in range(9, 17)})
+    caps.update({d: 4 for d in range(17, 33)})
+    caps.update({d: 3 for d in range(33, 70)})
+    rng = np.random.default_rng(2024)
+    try:
+        for it in range(400):
+            time_aug, lead_lag = bool(rng.integers(0, 4) == 0), bool(rng.integers(0, 4) == 0)
+            d = int(rng.choice(list(caps.keys())))
+            if lead_lag:
+                d = max(1, d // 2)
+            d_aug = (2 * d if lead_lag else d) + (1 if time_aug else 0)
+            deg = int(rng.integers(2, caps.get(d_aug, 3) + 1))
+            while d_aug ** deg > 3_000_000 and deg > 2:
+                deg -= 1
+            b = int(rng.choice([1, 2, 3, 5, 17, 70]))
+            length = int(rng.choice([2, 3, 5, 9, 33, 70, 131, 300]))
+            if d_aug ** deg * b * length > 60_000_000:
+                b, length = 1, min(length, 5)
+            dtype = np.float64 if rng.integers(0, 2) else np.float32
+            scalar_term = bool(rng.integers(0, 2))
+            segments = int(rng.choice([0, 0, 2, 3, 5]))
+            case = (it, b, length, d, deg, np.dtype(dtype).name, time_aug, lead_lag, scalar_term, segments)
+            x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (0.7 / np.sqrt(length))).astype(dtype)
+            aug = dict(time_aug=time_aug, lead_lag=lead_lag)
+            ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+            g = rng.standard_normal(ref.shape).astype(dtype)
+            want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+            C.cusig_amd_force_segments(segments)
+            C.cusig_amd_force_bwd_segments(segments)
+            got = P.sig(dev(x), deg, scalar_term=scalar_term, **aug).cpu().numpy()
+            got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+            off = 1 if scalar_term else 0
+            if scalar_term:
+                np.testing.assert_array_equal(got[:, 0], 1.0)
+            assert level_rel_err(got[:, off:], ref[:, off:], d_aug, deg) <= TOL[dtype], case
+            assert bwd_rel_err(got_b, want) <= TOL[dtype], case
+    finally:
+        C.cusig_amd_force_segments(0)
+        C.cusig_amd_force_bwd_segments(0)
+
+
 def test_wide_degree_one(P):
     x = torch.randn(3, 2, 200000, dtype=torch.float32, device=DEV)
     torch.testing.assert_close(P.sig(x, 1), x[:, 1] - x[:, 0])
