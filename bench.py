@@ -297,7 +297,7 @@ def main():
                                   "kernel_ms": kms, "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS[r.dtype]}
             del r
             torch.cuda.empty_cache()
-        # degree 2 on paths of many channels: closed form on the matrix cores (not a BASELINE workload)
+        # degree 2 on paths of many channels: closed form on the matrix cores (not one of the five benchmark workloads)
         db, dl, dd = 2048, 256, 64
         xp = (torch.randn((db, dl, dd), dtype=torch.float32, device="cuda:0").cumsum(1) * 0.05).contiguous()
         sg = torch.empty((db, dd + dd * dd), dtype=torch.float32, device="cuda:0")
