@@ -347,4 +347,105 @@ __global__ __launch_bounds__(kBlock) void degree2_bwd_kernel(
     }
 }
 
+// anti[b][a][c] = G2[a][c] - G2[c][a]: written once per call so that the staged backward reads it row-wise
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_anti_kernel(
+    const T* __restrict__ gsig, T* __restrict__ anti, int64_t batch, int d, int64_t sig_stride, int scalar)
+{
+    const int64_t dd = int64_t(d) * d;
+    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < batch * dd; e += int64_t(gridDim.x) * kBlock) {
+        const int64_t b = e / dd;
+        const int64_t r = e - b * dd;
+        const int a = int(r / d), c = int(r - int64_t(a) * d);
+        const T* g2 = gsig + b * sig_stride + scalar + d;
+        anti[e] = g2[r] - g2[int64_t(c) * d + a];
+    }
+}
+
+// Backward, operands staged through LDS.  A block serves one (path, 64 steps, group of kDeg2Cols column tiles): its
+// four waves own 16 steps each and share the column group.  The product runs over the channels a in chunks of 64: per
+// chunk the block writes U[64 steps][64 channels] and anti[64 channels][64 columns] to LDS, then every wave feeds its
+// products from there.  Row strides are chosen so that fragment reads are bank-conflict free: the U fragment walks
+// rows with its 16 lanes (stride 66 words f32 / 65 f64), the anti fragment walks columns (stride 80).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree2_bwd_staged_kernel(
+    const T* __restrict__ path, const T* __restrict__ anti, const T* __restrict__ h, T* __restrict__ dz, int64_t batch,
+    int64_t len_raw, int d_raw, int time_aug, int lead_lag, T time_step, int64_t time_groups, int col_groups)
+{
+    using M = Mfma16<T>;
+    extern __shared__ double lds_raw_d2b[];
+    constexpr int SU = sizeof(T) == 8 ? 65 : 66;
+    constexpr int SA = kDeg2SlabStride;
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    T* lds_u = reinterpret_cast<T*>(lds_raw_d2b);
+    T* lds_a = lds_u + kDeg2Slab * SU;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t per_path = time_groups * col_groups;
+    const int64_t b = int64_t(blockIdx.x) / per_path;           // grid = batch * per_path
+    const int64_t w = int64_t(blockIdx.x) - b * per_path;
+    const int cg = int(w % col_groups);
+    const int64_t tg = w / col_groups;
+    const T* x = path + b * len_raw * d_raw;
+    const T* an = anti + b * int64_t(d) * d;
+
+    const int li = lane & 15, lk = lane >> 4;
+    const int tiles = (d + 15) / 16;
+    const int nb = tiles - cg * kDeg2Cols < kDeg2Cols ? tiles - cg * kDeg2Cols : kDeg2Cols;
+    typename M::Acc acc[kDeg2Cols];
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) acc[j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+
+    const int sc_col = threadIdx.x % kDeg2Slab, sc_row0 = threadIdx.x / kDeg2Slab;
+    const int64_t t_base = tg * kDeg2Slab;
+    for (int a0 = 0; a0 < d; a0 += kDeg2Slab) {
+        __syncthreads();        // the previous chunk has been consumed
+        {
+            // U: rows are steps, columns channels a0 + sc_col
+            const int a = a0 + sc_col;
+            const T x0 = a < d ? aug_point(x, 0, a, d_raw, time_aug, lead_lag, d, time_step) : T(0);
+            for (int r = sc_row0; r < kDeg2Slab; r += kBlock / kDeg2Slab) {
+                const int64_t t = t_base + r;
+                T u = T(0);
+                if (t < L && a < d)
+                    u = T(0.5) * (aug_point(x, t, a, d_raw, time_aug, lead_lag, d, time_step) +
+                                  aug_point(x, t + 1, a, d_raw, time_aug, lead_lag, d, time_step)) - x0;
+                lds_u[r * SU + sc_col] = u;
+            }
+            // anti: rows are channels a0 + r, columns cg * 64 + sc_col
+            const int c = cg * kDeg2Slab + sc_col;
+            for (int r = sc_row0; r < kDeg2Slab; r += kBlock / kDeg2Slab) {
+                const int aa = a0 + r;
+                lds_a[r * SA + sc_col] = (aa < d && c < d) ? an[int64_t(aa) * d + c] : T(0);
+            }
+        }
+        __syncthreads();
+        const T* pu = lds_u + (wave * 16 + li) * SU + lk;
+        const T* pa = lds_a + lk * SA + li;
+        const int kmax = d - a0 < kDeg2Slab ? d - a0 : kDeg2Slab;
+        for (int k0 = 0; k0 < kmax; k0 += 4) {
+            const T ua = pu[k0];
+            T ab[kDeg2Cols];
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) ab[j] = j < nb ? pa[k0 * SA + j * 16] : T(0);
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j)
+                if (j < nb) acc[j] = M::mma(ua, ab[j], acc[j]);
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < kDeg2Cols; ++j) {
+        const int c = (cg * kDeg2Cols + j) * 16 + li;
+        if (c >= d) continue;
+        const T hc = h[b * d + c];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t row = t_base + wave * 16 + M::row(lk, r);
+            if (row < L) dz[(b * L + row) * d + c] = acc[j][r] + hc;
+        }
+    }
+}
+
 }  // namespace sigamd
