@@ -156,16 +156,33 @@ CUSIG_AMD_API int sig_coef_backprop_cuda_d(const double* path, double* out, cons
                                            const uint64_t* multi_idx, uint64_t num_multi_idx, const uint64_t* degrees,
                                            uint64_t batch_size, uint64_t dimension, uint64_t length) CUSIG_AMD_NOEXCEPT;
 
-/* Expanded (tensor) logarithm of each signature; same row layout in and out, scalar slot of the result 0.
- * method 0 only: methods 1 and 2 (Lyndon coordinates) return status 10.
- * Replaces: sig_to_log_sig_cuda_{f,d} (decl siglib/cusig/cusig.h:407-409; arithmetic siglib/cpsig/cp_tensor_log.h:40-125),
+/* Logarithm of each signature.  method 0: expanded (tensor) logarithm, same row layout in and out, scalar slot of
+ * the result 0.  method 1: its coefficients at the Lyndon words, method 2: its coordinates in the Lyndon basis; both
+ * write rows of log_sig_length(dimension, degree) values (no scalar slot) and need prepare_log_sig_cuda first
+ * (status 5 otherwise).
+ * Replaces: sig_to_log_sig_cuda_{f,d} (decl siglib/cusig/cusig.h:407-409; arithmetic siglib/cpsig/cp_tensor_log.h:40-170),
  * bound by pysiglib/load_siglib.py (CUSIG_SIG_TO_LOG_SIG), called from pysiglib/log_sig.py:223-311. */
 CUSIG_AMD_API int sig_to_log_sig_cuda_f(const float* sig, float* out, uint64_t batch_size, uint64_t dimension, uint64_t degree,
                                         int method, bool scalar_term) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API int sig_to_log_sig_cuda_d(const double* sig, double* out, uint64_t batch_size, uint64_t dimension,
                                         uint64_t degree, int method, bool scalar_term) CUSIG_AMD_NOEXCEPT;
 
-/* Gradient w.r.t. the signature given dF/d(log signature) (method 0 layout); scalar slot of the result 0.
+/* Prepares the tables of methods 1 and 2 for (dimension, degree) on the current device; preparing method 2 also
+ * serves method 1; method 0 needs nothing; method 3 (BCH) returns status 10.  use_disk is accepted and ignored.
+ * Replaces: prepare_log_sig_cuda (siglib/cusig/cusig.h:447; tables of siglib/shared/preparation/log_sig/lyndon_words.cpp),
+ * bound by pysiglib/load_siglib.py:166-167, called from pysiglib/log_sig.py:93-187. */
+CUSIG_AMD_API int prepare_log_sig_cuda(uint64_t dimension, uint64_t degree, int method, bool use_disk) CUSIG_AMD_NOEXCEPT;
+/* Host-only view of the tables prepare_log_sig_cuda builds (needs no GPU; no counterpart in the reference's ABI): call
+ * with null arrays for the sizes, then with `count` indices (positions of the Lyndon words in a scalar-free signature
+ * row), `count + 1` row offsets and `nnz` columns / values of the strictly lower part of the inverse projection
+ * (unit diagonal implicit; empty for method 1). */
+CUSIG_AMD_API int cusig_amd_lyndon_tables(uint64_t dimension, uint64_t degree, int method, uint64_t* count, uint64_t* nnz,
+                                          uint64_t* index, uint64_t* row_ptr, uint32_t* col, int32_t* val) CUSIG_AMD_NOEXCEPT;
+/* Drops every prepared table.  Replaces: clear_cache_cuda (siglib/cusig/cusig.h:626), bound by
+ * pysiglib/load_siglib.py:169-170, called from pysiglib/log_sig.py:190-240. */
+CUSIG_AMD_API int clear_cache_cuda(bool use_disk) CUSIG_AMD_NOEXCEPT;
+
+/* Gradient w.r.t. the signature given dF/d(log signature) (rows in the layout of `method`); scalar slot of the result 0.
  * Replaces: sig_to_log_sig_backprop_cuda_{f,d} (decl siglib/cusig/cusig.h:429-431; arithmetic
  * siglib/cpsig/cp_tensor_log.h:164-221), bound by pysiglib/load_siglib.py (CUSIG_SIG_TO_LOG_SIG_BACKPROP), called from
  * pysiglib/log_sig_backprop.py:30-137. */

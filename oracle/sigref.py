@@ -308,8 +308,14 @@ def sig_coef_backprop(path, words, coefs, derivs, time_aug=False, lead_lag=False
     return out[0] if single else out
 
 
-def sig_to_log_sig(sig, dimension, degree):
-    """Oracle expanded (method 0) log signature; ``dimension`` is the augmented dimension."""
+def sig_to_log_sig(sig, dimension, degree, method=0):
+    """Oracle log signature; ``dimension`` is the augmented dimension.  method 0: expanded (same width as ``sig``);
+    1: its coefficients at the Lyndon words; 2: coordinates in the Lyndon basis (oracle/lyndon.py)."""
+    if method:
+        from . import lyndon
+        full = sig_to_log_sig(sig, dimension, degree, 0)
+        off = 1 if np.asarray(sig).shape[-1] == sig_length(dimension, degree) else 0
+        return np.ascontiguousarray(lyndon.compress(full[..., off:], dimension, degree, method))
     sig = np.asarray(sig)
     suf, real = _suffix(sig.dtype)
     a = _rows(sig, sig.dtype)
@@ -323,7 +329,13 @@ def sig_to_log_sig(sig, dimension, degree):
     return out.reshape(sig.shape)
 
 
-def sig_to_log_sig_backprop(sig, derivs, dimension, degree):
+def sig_to_log_sig_backprop(sig, derivs, dimension, degree, method=0):
+    if method:
+        from . import lyndon
+        expanded = lyndon.compress_backprop(derivs, dimension, degree, method)
+        if np.asarray(sig).shape[-1] == sig_length(dimension, degree):
+            expanded = np.concatenate([np.zeros(expanded.shape[:-1] + (1,), dtype=expanded.dtype), expanded], axis=-1)
+        return sig_to_log_sig_backprop(sig, np.ascontiguousarray(expanded), dimension, degree, 0)
     sig = np.asarray(sig)
     suf, real = _suffix(sig.dtype)
     a, g = _rows(sig, sig.dtype), _rows(derivs, sig.dtype)

@@ -27,6 +27,10 @@ CUSIG.cusig_shutdown.argtypes = ()
 CUSIG.cusig_shutdown.restype = None
 CUSIG.cusig_amd_sig_length.argtypes = (c_uint64, c_uint64)
 CUSIG.cusig_amd_sig_length.restype = c_uint64
+CUSIG.prepare_log_sig_cuda.argtypes = (c_uint64, c_uint64, c_int, c_bool)
+CUSIG.prepare_log_sig_cuda.restype = c_int
+CUSIG.clear_cache_cuda.argtypes = (c_bool,)
+CUSIG.clear_cache_cuda.restype = c_int
 CUSIG.cusig_amd_last_sig_nonfinite.argtypes = ()
 CUSIG.cusig_amd_last_sig_nonfinite.restype = c_int
 CUSIG.cusig_amd_set_profiling.argtypes = (c_int,)

@@ -798,7 +798,11 @@ CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const dou
 
 CUSIG_AMD_API const char* cusig_last_error_message(void) noexcept { return g_last_error; }
 
-CUSIG_AMD_API void cusig_shutdown(void) noexcept { release_workspaces(); }
+CUSIG_AMD_API void cusig_shutdown(void) noexcept
+{
+    release_workspaces();
+    clear_lyndon_tables();
+}
 
 CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree) noexcept
 {

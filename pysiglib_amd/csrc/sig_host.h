@@ -14,9 +14,12 @@ namespace sigamd {
 extern thread_local char g_last_error[4096];
 
 // Grow-only device buffers, one per (current device, slot), released by cusig_shutdown(); hold g_ws_mutex while a
-// buffer is in use (defined in sig_api.hip).  Slots 0-3: signature sweeps; 4-5: sig_join_backprop; 6: word tables of sig_coef; 7: tensor logarithm.
+// buffer is in use (defined in sig_api.hip).  Slots 0-3: signature sweeps; 4-5: sig_join_backprop; 6: word tables of sig_coef; 7, 14, 15: tensor logarithm; 8-11: time-split backward; 12-13: degree-2 backward.
 extern std::mutex g_ws_mutex;
 void* workspace(int slot, size_t bytes);
+
+// drops the prepared Lyndon tables of every device (defined in sig_log.hip; also called by cusig_shutdown)
+void clear_lyndon_tables() noexcept;
 
 inline void clear_last_error() { g_last_error[0] = 0; }
 inline void set_last_error(const char* msg) { std::snprintf(g_last_error, sizeof g_last_error, "%s", msg ? msg : ""); }
@@ -35,12 +38,21 @@ struct HipFailure : std::runtime_error {
         if (e__ != hipSuccess) throw ::sigamd::HipFailure(e__, #call); \
     } while (0)
 
+// a runtime error that carries its own status code (siglib/shared/errors.h: 5 = prepared cache not found)
+struct CodedError : std::runtime_error {
+    int code;
+    CodedError(int code_, const char* what_) : std::runtime_error(what_), code(code_) {}
+};
+
 template <typename F>
 int guarded(F&& body) noexcept
 {
     clear_last_error();
     try {
         body();
+    } catch (const CodedError& e) {
+        set_last_error(e.what());
+        return e.code;
     } catch (const std::bad_alloc&) {
         set_last_error("Failed to allocate memory");
         return 1;

@@ -1,19 +1,27 @@
-// Expanded (tensor) logarithm of a signature and its backward pass, behind the reference's entry points
-//   sig_to_log_sig_cuda_{f,d}, sig_to_log_sig_backprop_cuda_{f,d} with method 0
-//   (decl siglib/cusig/cusig.h:391-431; arithmetic of siglib/cpsig/cp_tensor_log.h:40-113 forward, :164-221 backward).
-// Methods 1 and 2 (Lyndon coordinates) need the reference's prepared Lyndon tables and are not part of this build.
+// Logarithm of a signature and its backward pass, behind the reference's entry points
+//   sig_to_log_sig_cuda_{f,d}, sig_to_log_sig_backprop_cuda_{f,d}, prepare_log_sig_cuda, clear_cache_cuda
+//   (decl siglib/cusig/cusig.h:391-447, 616-626; arithmetic of siglib/cpsig/cp_tensor_log.h:40-113 forward,
+//   :140-170 Lyndon coordinates, :164-221 backward).
+// Method 0: expanded (tensor) logarithm.  Methods 1 and 2: its coordinates at the Lyndon words resp. in the Lyndon
+// basis, from tables prepared on the host per (device, dimension, degree) (sig_lyndon.h); as in the reference they
+// must have been prepared with prepare_log_sig_cuda (status 5 otherwise).  Method 3 (BCH) is not part of this build.
 //
 // With x = sig - 1:   log(1 + x) = P_1,   P_k = x / k - x (x) P_{k+1},   P_{N+1} = 0,
 // where P_k only needs levels <= N - k + 1.  One launch per k, one thread per coefficient.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <map>
 #include <mutex>
+#include <string>
+#include <tuple>
+#include <vector>
 
 #include "../../include/cusig_amd.h"
 #include "sig_chen_adjoint.h"
 #include "sig_host.h"
 #include "sig_kernels.h"
+#include "sig_lyndon.h"
 
 namespace sigamd {
 
@@ -89,9 +97,131 @@ __global__ __launch_bounds__(kBlock) void tensor_log_bwd_init_kernel(
 static void check_method(int method, const char* who)
 {
     if (method < 0 || method > 2) throw std::invalid_argument(std::string(who) + ": method must be 0, 1 or 2");
-    if (method != 0)
-        throw std::runtime_error(std::string(who) + ": methods 1 and 2 (Lyndon coordinates) are not implemented in this "
-                                 "build; use method 0 (expanded tensor logarithm)");
+}
+
+// ---------------------------------------------------------------------------
+// Lyndon coordinates: prepared tables on the device
+// ---------------------------------------------------------------------------
+struct CacheMissing : CodedError {
+    explicit CacheMissing(const char* what_) : CodedError(5, what_) {}
+};
+
+struct DeviceLyndon {
+    int method = 0;
+    uint64_t count = 0;                                  // Lyndon words
+    uint64_t* index = nullptr;                           // their positions in a scalar-free row
+    uint64_t *row_ptr = nullptr, *t_row_ptr = nullptr;   // strictly lower part of M^-1 and of its transpose (CSR)
+    uint32_t *col = nullptr, *t_col = nullptr;
+    int32_t *val = nullptr, *t_val = nullptr;
+    void release() noexcept
+    {
+        for (void* p : {(void*)index, (void*)row_ptr, (void*)t_row_ptr, (void*)col, (void*)t_col, (void*)val, (void*)t_val})
+            if (p) (void)hipFree(p);
+        *this = DeviceLyndon();
+    }
+};
+static std::mutex g_lyndon_mutex;
+static std::map<std::tuple<int, uint64_t, uint64_t>, DeviceLyndon> g_lyndon;       // (device, dimension, degree)
+
+template <typename V>
+static V* upload(const std::vector<V>& host)
+{
+    V* dev = nullptr;
+    SIG_HIP(hipMalloc(reinterpret_cast<void**>(&dev), std::max<size_t>(host.size(), 1) * sizeof(V)));
+    if (!host.empty()) SIG_HIP(hipMemcpy(dev, host.data(), host.size() * sizeof(V), hipMemcpyHostToDevice));
+    return dev;
+}
+
+static void prepare_lyndon(uint64_t dimension, uint64_t degree, int method)
+{
+    if (method == 0) return;
+    if (method == 3) throw std::runtime_error("prepare_log_sig_cuda: method 3 (BCH) is not implemented in this build");
+    if (method < 0 || method > 3) throw std::invalid_argument("log signature method must be 1, 2, or 3");
+    int dev = 0;
+    SIG_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_lyndon_mutex);
+    DeviceLyndon& slot = g_lyndon[std::make_tuple(dev, dimension, degree)];
+    if (slot.method >= method) return;                   // preparing for method 2 also serves method 1
+    const LyndonTables t = build_lyndon_tables(dimension, degree, method);
+    DeviceLyndon fresh;
+    try {
+        fresh.method = method;
+        fresh.count = t.index.size();
+        fresh.index = upload(t.index);
+        if (method == 2) {
+            fresh.row_ptr = upload(t.row_ptr);
+            fresh.t_row_ptr = upload(t.t_row_ptr);
+            fresh.col = upload(t.col);
+            fresh.t_col = upload(t.t_col);
+            fresh.val = upload(t.val);
+            fresh.t_val = upload(t.t_val);
+        }
+    } catch (...) {
+        fresh.release();
+        throw;
+    }
+    slot.release();
+    slot = fresh;
+}
+
+void clear_lyndon_tables() noexcept
+{
+    std::lock_guard<std::mutex> lk(g_lyndon_mutex);
+    int cur = 0;
+    const bool have = hipGetDevice(&cur) == hipSuccess;
+    for (auto& kv : g_lyndon) {
+        if (have && hipSetDevice(std::get<0>(kv.first)) == hipSuccess) kv.second.release();
+    }
+    if (have) (void)hipSetDevice(cur);
+    g_lyndon.clear();
+    (void)hipGetLastError();
+}
+
+static DeviceLyndon find_lyndon(uint64_t dimension, uint64_t degree, int method)
+{
+    int dev = 0;
+    SIG_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_lyndon_mutex);
+    auto it = g_lyndon.find(std::make_tuple(dev, dimension, degree));
+    if (it == g_lyndon.end() || it->second.method < method) throw CacheMissing("Could not find prepared cache");
+    return it->second;
+}
+
+// out[b][i] = x[b][index[i]] (method 1) plus sum_k val[k] * x[b][index[col[k]]] over the row's entries (method 2)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lyndon_compress_kernel(
+    const T* __restrict__ expanded, T* __restrict__ out, int64_t batch, int64_t count, int64_t stride, int off,
+    const uint64_t* __restrict__ index, const uint64_t* __restrict__ row_ptr, const uint32_t* __restrict__ col,
+    const int32_t* __restrict__ val)
+{
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* x = expanded + b * stride + off;
+        for (int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x; i < count; i += int64_t(gridDim.x) * kBlock) {
+            T acc = x[index[i]];
+            if (row_ptr)
+                for (uint64_t k = row_ptr[i]; k < row_ptr[i + 1]; ++k) acc = fmadd(T(val[k]), x[index[col[k]]], acc);
+            out[b * count + i] = acc;
+        }
+    }
+}
+
+// the transpose: dx[b][index[j]] = g[b][j] + sum_k t_val[k] * g[b][t_col[k]]; every other entry of dx must be zero
+// beforehand
+template <typename T>
+__global__ __launch_bounds__(kBlock) void lyndon_expand_kernel(
+    const T* __restrict__ g, T* __restrict__ dx, int64_t batch, int64_t count, int64_t stride, int off,
+    const uint64_t* __restrict__ index, const uint64_t* __restrict__ t_row_ptr, const uint32_t* __restrict__ t_col,
+    const int32_t* __restrict__ t_val)
+{
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* gb = g + b * count;
+        for (int64_t j = int64_t(blockIdx.x) * kBlock + threadIdx.x; j < count; j += int64_t(gridDim.x) * kBlock) {
+            T acc = gb[j];
+            if (t_row_ptr)
+                for (uint64_t k = t_row_ptr[j]; k < t_row_ptr[j + 1]; ++k) acc = fmadd(T(t_val[k]), gb[t_col[k]], acc);
+            dx[b * stride + off + index[j]] = acc;
+        }
+    }
 }
 
 // number of coefficients of levels 1 .. t
@@ -124,11 +254,13 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
     check_method(method, "sig_to_log_sig_cuda");
     const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_cuda");
     if (batch == 0) return;
+    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     const uint64_t bytes = checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
     SIG_HIP(hipDeviceSynchronize());
     hipStream_t stream = nullptr;
     if (s.n_coef == 0) {
-        if (scalar_term) hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch));
+        // degree 0: the compressed forms are empty, the expanded one holds the scalar slot
+        if (scalar_term && !method) hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch));
         SIG_HIP(hipGetLastError());
         SIG_HIP(hipStreamSynchronize(stream));
         return;
@@ -136,7 +268,17 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     T* ws = degree >= 2 ? static_cast<T*>(workspace(7, checked_mul(bytes, 2, "workspace"))) : nullptr;
     const uint64_t elems = batch * s.stride;
-    run_tensor_log<T>(sig, out, batch, dimension, degree, s, stream, [&](uint64_t k) { return ws + (k & 1) * elems; });
+    // Lyndon coordinates are read off the expanded logarithm, which then lives in a scratch copy
+    T* expanded = method ? static_cast<T*>(workspace(14, bytes)) : out;
+    run_tensor_log<T>(sig, expanded, batch, dimension, degree, s, stream, [&](uint64_t k) { return ws + (k & 1) * elems; });
+    if (method) {
+        launch_indexed(0, lyn.count, batch, [&](auto, dim3 grid) {
+            hipLaunchKernelGGL((lyndon_compress_kernel<T>), grid, dim3(kBlock), 0, stream, (const T*)expanded, out, int64_t(batch),
+                               int64_t(lyn.count), int64_t(s.stride), s.off, (const uint64_t*)lyn.index,
+                               (const uint64_t*)(method == 2 ? lyn.row_ptr : nullptr), (const uint32_t*)lyn.col,
+                               (const int32_t*)lyn.val);
+        });
+    }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
 }
@@ -148,6 +290,7 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
     check_method(method, "sig_to_log_sig_backprop_cuda");
     const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_backprop_cuda");
     if (batch == 0) return;
+    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     const uint64_t bytes = checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
     SIG_HIP(hipDeviceSynchronize());
     hipStream_t stream = nullptr;
@@ -159,6 +302,18 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
     }
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     const uint64_t elems = batch * s.stride;
+    if (method) {
+        // gradient w.r.t. the expanded logarithm: the transposed coordinate map, zero off the Lyndon words
+        T* dexp = static_cast<T*>(workspace(15, bytes));
+        hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(elems)), dim3(kBlock), 0, stream, dexp, int64_t(elems));
+        launch_indexed(0, lyn.count, batch, [&](auto, dim3 grid) {
+            hipLaunchKernelGGL((lyndon_expand_kernel<T>), grid, dim3(kBlock), 0, stream, derivs, dexp, int64_t(batch),
+                               int64_t(lyn.count), int64_t(s.stride), s.off, (const uint64_t*)lyn.index,
+                               (const uint64_t*)(method == 2 ? lyn.t_row_ptr : nullptr), (const uint32_t*)lyn.t_col,
+                               (const int32_t*)lyn.t_val);
+        });
+        derivs = dexp;
+    }
     // P_1 (discarded), P_2 .. P_N, two adjoint buffers, two product-adjoint buffers
     T* ws = degree >= 2 ? static_cast<T*>(workspace(7, checked_mul(bytes, degree + 4, "workspace"))) : nullptr;
     launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
@@ -222,6 +377,38 @@ CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_d(const double* sig, double* out,
     return guarded([&] {
         sig_to_log_sig_backprop_impl<double>(sig, out, log_sig_derivs, batch_size, dimension, degree, method, scalar_term);
     });
+}
+
+/* Replaces prepare_log_sig_cuda (siglib/cusig/cusig.h:447): builds and uploads the Lyndon tables of (dimension, degree) for
+ * the current device.  use_disk is accepted and ignored: tables are rebuilt in memory (milliseconds for the sizes
+ * a signature of that shape allows). */
+CUSIG_AMD_API int prepare_log_sig_cuda(uint64_t dimension, uint64_t degree, int method, bool) noexcept
+{
+    return guarded([&] { prepare_lyndon(dimension, degree, method); });
+}
+
+/* Host-only view of the tables prepare_log_sig_cuda uploads (needs no GPU): first call with null arrays for the sizes,
+ * then with arrays of `count` indices, `count + 1` row offsets and `nnz` columns / values (strictly lower part of the
+ * inverse projection; empty for method 1). */
+CUSIG_AMD_API int cusig_amd_lyndon_tables(uint64_t dimension, uint64_t degree, int method, uint64_t* count, uint64_t* nnz,
+                                          uint64_t* index, uint64_t* row_ptr, uint32_t* col, int32_t* val) noexcept
+{
+    return guarded([&] {
+        if (method != 1 && method != 2) throw std::invalid_argument("cusig_amd_lyndon_tables: method must be 1 or 2");
+        const LyndonTables t = build_lyndon_tables(dimension, degree, method);
+        if (count) *count = t.index.size();
+        if (nnz) *nnz = t.col.size();
+        if (index) std::copy(t.index.begin(), t.index.end(), index);
+        if (row_ptr) std::copy(t.row_ptr.begin(), t.row_ptr.end(), row_ptr);
+        if (col) std::copy(t.col.begin(), t.col.end(), col);
+        if (val) std::copy(t.val.begin(), t.val.end(), val);
+    });
+}
+
+/* Replaces clear_cache_cuda (siglib/cusig/cusig.h:626): drops every prepared table on every device. */
+CUSIG_AMD_API int clear_cache_cuda(bool) noexcept
+{
+    return guarded([&] { clear_lyndon_tables(); });
 }
 
 }  // extern "C"

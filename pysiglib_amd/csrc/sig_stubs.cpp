@@ -52,8 +52,6 @@ STUB_PAIR(log_sig_join_cuda)
 STUB_PAIR(log_sig_join_backprop_cuda)
 STUB_PAIR(logsig_to_sig_cuda)
 STUB_PAIR(logsig_to_sig_backprop_cuda)
-STUB_ONE(prepare_log_sig_cuda)
-STUB_ONE(clear_cache_cuda)
 STUB_ONE(set_cache_dir_cuda)
 STUB_ONE(prepare_branched_sig_cuda)
 STUB_ONE(prepare_branched_log_sig_cuda)

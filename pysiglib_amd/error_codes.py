@@ -6,6 +6,7 @@ _MESSAGES = {
     2: "Invalid argument",
     3: "Out of range",
     4: "Filesystem error",
+    5: "Could not find prepared cache. Please call the corresponding preparation function with the correct parameters.",
     10: "Runtime error",
     11: "Unknown exception",
 }

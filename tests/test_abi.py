@@ -23,7 +23,7 @@ branched_sig_combine_cuda branched_sig_to_log_sig_cuda branched_sig_to_log_sig_b
 branched_log_sig_join_backprop_cuda branched_log_sig_from_path_cuda branched_log_sig_from_path_backprop_cuda
 branched_sig_combine_backprop_cuda branched_sig_backprop_cuda linear_sig_cuda log_sig_join_cuda
 log_sig_join_backprop_cuda logsig_to_sig_cuda logsig_to_sig_backprop_cuda""".split()
-LOADER_SINGLES = ["prepare_log_sig_cuda", "clear_cache_cuda", "set_cache_dir_cuda", "prepare_branched_sig_cuda",
+LOADER_SINGLES = ["prepare_log_sig_cuda", "clear_cache_cuda", "set_cache_dir_cuda", "cusig_amd_lyndon_tables", "prepare_branched_sig_cuda",
                   "prepare_branched_log_sig_cuda", "prepare_branched_sig_coef_cuda", "cusig_shutdown",
                   "cusig_last_error_message"]
 
@@ -54,7 +54,39 @@ def test_out_of_scope_symbols_report_not_implemented(lib):
     lib.cusig_last_error_message.restype = ctypes.c_char_p
     assert lib.sig_kernel_cuda_d(None, None, None, 0, 0, 0) == 10
     assert b"not implemented" in lib.cusig_last_error_message()
-    assert lib.prepare_log_sig_cuda(2, 2, 0, False) == 10
+    assert lib.set_cache_dir_cuda(None) == 10
+
+
+@pytest.mark.parametrize("d,deg", [(2, 7), (3, 5), (5, 4), (1, 3), (8, 3)])
+def test_lyndon_tables_match_the_oracle(lib, d, deg):
+    """The host code behind prepare_log_sig_cuda against the oracle's Lyndon words and bracket projection."""
+    import numpy as np
+    from oracle import lyndon
+    fn = lib.cusig_amd_lyndon_tables
+    u64p, u32p, i32p = ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_int32)
+    fn.argtypes = (ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int, u64p, u64p, u64p, u64p, u32p, i32p)
+    count, nnz = ctypes.c_uint64(), ctypes.c_uint64()
+    words = lyndon.lyndon_words(d, deg)
+    for method in (1, 2):
+        assert fn(d, deg, method, ctypes.byref(count), ctypes.byref(nnz), None, None, None, None) == 0
+        assert count.value == len(words)
+        index = np.zeros(count.value, dtype=np.uint64)
+        row_ptr = np.zeros(count.value + 1, dtype=np.uint64)
+        col = np.zeros(max(nnz.value, 1), dtype=np.uint32)
+        val = np.zeros(max(nnz.value, 1), dtype=np.int32)
+        assert fn(d, deg, method, None, None, index.ctypes.data_as(u64p), row_ptr.ctypes.data_as(u64p),
+                  col.ctypes.data_as(u32p), val.ctypes.data_as(i32p)) == 0
+        assert list(index) == [lyndon.word_index(w, d) for w in words]
+        if method == 1:
+            assert nnz.value == 0
+            continue
+        inv = np.eye(len(words))
+        for i in range(len(words)):
+            for k in range(int(row_ptr[i]), int(row_ptr[i + 1])):
+                assert col[k] < i
+                inv[i, col[k]] = val[k]
+        np.testing.assert_allclose(inv @ lyndon.projection_matrix(d, deg), np.eye(len(words)), rtol=0, atol=1e-9)
+    assert fn(d, deg, 3, None, None, None, None, None, None) == 2
 
 
 def test_sig_length(lib, kats):

@@ -590,10 +590,13 @@ def test_log_sig_identities_shapes_and_errors(P):
                                rtol=1e-14, atol=1e-14)
     empty = torch.empty((0, P.sig_length(d, deg)), dtype=torch.float64, device=DEV)
     assert P.sig_to_log_sig(empty, d, deg, method=0).shape == empty.shape
-    with pytest.raises(NotImplementedError):
-        P.sig_to_log_sig(s, d, deg)                     # the reference's default, method=1, needs Lyndon tables
+    P.clear_cache()
+    with pytest.raises(Exception, match="Could not find prepared cache"):
+        P.sig_to_log_sig(s, d, deg)                     # the reference's default, method=1, needs prepare_log_sig
     with pytest.raises(NotImplementedError):
         P.log_sig(x, deg, method=3)
+    with pytest.raises(ValueError):
+        P.sig_to_log_sig(s, d, deg, method=3)
     with pytest.raises(ValueError):
         P.sig_to_log_sig(s, d, deg, method=7)
     with pytest.raises(ValueError):
@@ -603,6 +606,67 @@ def test_log_sig_identities_shapes_and_errors(P):
     from pysiglib_amd import _loader as L
     pd = lambda t: ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_double))
     o = torch.empty_like(s)
-    assert L.CUSIG_SIG_TO_LOG_SIG["float64"](pd(s), pd(o), 3, d, deg, 1, True) == 10
-    assert "not implemented" in L.last_error_message()
+    assert L.CUSIG_SIG_TO_LOG_SIG["float64"](pd(s), pd(o), 3, d, deg, 1, True) == 5
+    assert "prepared cache" in L.last_error_message()
     assert L.CUSIG_SIG_TO_LOG_SIG["float64"](pd(s), pd(o), 3, d, deg, 5, True) == 2
+    assert L.CUSIG.prepare_log_sig_cuda(d, deg, 3, False) == 10
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_log_sig_lyndon_golden(P, fixtures, deg, dtype):
+    """tests/test_log_sig.py:143-203 and tests/test_log_sig_backprop.py of the reference: signatory's Lyndon-word
+    coordinates and iisignature's Lyndon-basis coordinates of the fixture paths, forward and path gradients."""
+    tol = 1e-10 if dtype == torch.float64 else 1e-4
+    try:
+        P.clear_cache()
+        x = dev(fixtures["path"]).to(dtype)
+        with pytest.raises(Exception, match="Could not find prepared cache"):
+            P.log_sig(x, deg, method=1)
+        P.prepare_log_sig(3, deg, 1)
+        np.testing.assert_allclose(P.log_sig(x, deg, method=1).cpu().numpy(), fixtures["logsig_words__d%d" % deg], rtol=0, atol=tol)
+        np.testing.assert_allclose(P.log_sig(x[0], deg).cpu().numpy(), fixtures["logsig_words__d%d" % deg][0], rtol=0, atol=tol)
+        with pytest.raises(Exception, match="Could not find prepared cache"):
+            P.log_sig(x, deg, method=2)                  # prepared for method 1 only
+        P.prepare_log_sig(3, deg, 2)
+        np.testing.assert_allclose(P.log_sig(x, deg, method=2).cpu().numpy(), fixtures["logsig_basis__d%d" % deg], rtol=0, atol=tol)
+        np.testing.assert_allclose(P.log_sig(x, deg, method=1, scalar_term=True).cpu().numpy(),
+                                   fixtures["logsig_words__d%d" % deg], rtol=0, atol=tol)
+        for name, method in (("words", 1), ("basis", 2)):
+            xr = torch.tensor(fixtures["path"], dtype=dtype, device=DEV, requires_grad=True)
+            ls = P.torch_api.log_sig(xr, deg, method=method)
+            ls.backward(torch.tensor(fixtures["logsig_bp_%s_derivs__d%d" % (name, deg)], dtype=dtype, device=DEV))
+            np.testing.assert_allclose(xr.grad.cpu().numpy(), fixtures["logsig_bp_%s_expected__d%d" % (name, deg)], rtol=0,
+                                       atol=1e-5 if dtype == torch.float64 else 1e-4)
+    finally:
+        P.clear_cache()
+
+
+@pytest.mark.parametrize("d,deg,batch", [(2, 7, 5), (3, 4, 70), (5, 4, 4), (1, 5, 3), (4, 1, 2), (8, 3, 33), (6, 5, 2), (20, 2, 3)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_sig_to_log_sig_lyndon_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+    rng = np.random.default_rng(5 * d + deg)
+    n = oracle.sig_length(d, deg) - 1
+    scale = np.concatenate([np.full(d ** k, 0.5 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
+    a = (rng.standard_normal((batch, n)) * scale).astype(dtype)       # arbitrary tensors, not group-like
+    if scalar_term:
+        a = np.hstack([np.ones((batch, 1), dtype=dtype), a])
+    m = P.log_sig_length(d, deg)
+    g = rng.standard_normal((batch, m)).astype(dtype)
+    try:
+        P.prepare_log_sig(d, deg, 2)
+        for method in (1, 2):
+            want = oracle.sig_to_log_sig(a, d, deg, method=method)
+            got = P.sig_to_log_sig(dev(a), d, deg, method=method).cpu().numpy()
+            assert got.shape == (batch, m) and got.dtype == dtype
+            assert row_rel_err(got, want) < TOL[dtype]
+            wantb = oracle.sig_to_log_sig_backprop(a, g, d, deg, method=method)
+            gotb = P.sig_to_log_sig_backprop(dev(a), dev(g), d, deg, method=method).cpu().numpy()
+            assert gotb.shape == wantb.shape
+            if scalar_term:
+                assert np.all(gotb[:, 0] == 0)
+            off = 1 if scalar_term else 0
+            assert row_rel_err(gotb[:, off:], wantb[:, off:]) < TOL[dtype] * (1 if dtype == np.float64 else 10)
+    finally:
+        P.clear_cache()

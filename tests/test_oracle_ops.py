@@ -409,6 +409,91 @@ def test_log_sig_backprop_golden(fixtures, deg):
         np.testing.assert_allclose(got, fixtures["%s_expected__d%d" % (key, deg)], rtol=0, atol=1e-5)
 
 
+# ---- compressed log signatures: Lyndon words (method 1) and Lyndon basis (method 2) -----------------------------
+
+def _witt(d, n):
+    """Number of Lyndon words of length n over d letters (necklace polynomial)."""
+    def mobius(k):
+        res, p = 1, 2
+        while p * p <= k:
+            if k % p == 0:
+                k //= p
+                if k % p == 0:
+                    return 0
+                res = -res
+            p += 1
+        return -res if k > 1 else res
+    return sum(mobius(n // x) * d ** x for x in range(1, n + 1) if n % x == 0) // n
+
+
+@pytest.mark.parametrize("d,deg", [(2, 7), (3, 5), (5, 4), (1, 4), (7, 3)])
+def test_lyndon_words(d, deg):
+    from oracle import lyndon
+    words = lyndon.lyndon_words(d, deg)
+    # counts by the necklace polynomial; every word strictly smaller than its proper suffixes; sorted inside a length
+    for n in range(1, deg + 1):
+        level = [w for w in words if len(w) == n]
+        assert len(level) == _witt(d, n)
+        assert level == sorted(level)
+        for w in level:
+            assert all(w < w[i:] for i in range(1, n))
+    assert [len(w) for w in words] == sorted(len(w) for w in words)
+    # brute force: nothing is missing
+    if d ** deg <= 3000:
+        import itertools
+        brute = [w for n in range(1, deg + 1) for w in itertools.product(range(d), repeat=n)
+                 if all(w < w[i:] for i in range(1, n))]
+        assert set(brute) == set(words)
+    # the projection is unit lower triangular and couples only words made of the same letters
+    m = lyndon.projection_matrix(d, deg)
+    assert np.all(np.diag(m) == 1) and np.all(np.triu(m, 1) == 0)
+    for i, j in zip(*np.nonzero(m)):
+        assert sorted(words[i]) == sorted(words[j])
+
+
+@pytest.mark.parametrize("deg", range(1, 6))
+def test_log_sig_lyndon_golden(fixtures, deg):
+    # signatory's "words" mode and iisignature's "s" (Lyndon basis) coordinates, held by the reference's fixture
+    x = fixtures["path"]
+    s = sigref.signature(x, deg)
+    np.testing.assert_allclose(sigref.sig_to_log_sig(s, 3, deg, method=1), fixtures["logsig_words__d%d" % deg], rtol=0, atol=1e-12)
+    np.testing.assert_allclose(sigref.sig_to_log_sig(s, 3, deg, method=2), fixtures["logsig_basis__d%d" % deg], rtol=0, atol=1e-12)
+    one = np.hstack([np.ones((len(s), 1)), s])
+    for method in (1, 2):
+        np.testing.assert_array_equal(sigref.sig_to_log_sig(one, 3, deg, method=method), sigref.sig_to_log_sig(s, 3, deg, method=method))
+    # path gradients through the compressed coordinates
+    for name, method, tol in (("words", 1, 1e-10), ("basis", 2, 1e-5)):
+        ds = sigref.sig_to_log_sig_backprop(s, fixtures["logsig_bp_%s_derivs__d%d" % (name, deg)], 3, deg, method=method)
+        got = sigref.sig_backprop(x, s, ds, deg)
+        np.testing.assert_allclose(got, fixtures["logsig_bp_%s_expected__d%d" % (name, deg)], rtol=0, atol=tol)
+
+
+@pytest.mark.parametrize("d,deg", [(2, 6), (3, 4), (4, 3)])
+def test_log_sig_lyndon_basis_reconstructs(d, deg):
+    """The log signature of a path is a Lie element: expanding its Lyndon-basis coordinates through the brackets
+    must give back the whole expanded log signature, not only its Lyndon-word coefficients; and the backward passes
+    of both methods are the transposes of the forward maps."""
+    from oracle import lyndon
+    rng = np.random.default_rng(d + deg)
+    x = np.cumsum(rng.standard_normal((3, 12, d)), axis=1) * 0.3
+    s = sigref.signature(x, deg)
+    expanded = sigref.sig_to_log_sig(s, d, deg)
+    beta = sigref.sig_to_log_sig(s, d, deg, method=2)
+    words = lyndon.lyndon_words(d, deg)
+    poly = lyndon._bracket_polynomials(words)
+    rebuilt = np.zeros_like(expanded)
+    for j, w in enumerate(words):
+        for word, c in poly[w].items():
+            rebuilt[:, lyndon.word_index(word, d)] += c * beta[:, j]
+    np.testing.assert_allclose(rebuilt, expanded, rtol=0, atol=1e-12)
+    n = expanded.shape[1]
+    for method in (1, 2):
+        m = len(words)
+        fwd = np.stack([lyndon.compress(e, d, deg, method) for e in np.eye(n)], axis=1)          # (m, n) matrix
+        bwd = np.stack([lyndon.compress_backprop(e, d, deg, method) for e in np.eye(m)], axis=0)  # (m, n) as well
+        np.testing.assert_allclose(bwd, fwd, rtol=0, atol=1e-13)
+
+
 @pytest.mark.parametrize("d,deg", [(2, 6), (3, 4), (5, 3), (1, 5), (4, 1), (3, 2)])
 def test_log_sig_vs_power_series_and_autograd(d, deg):
     rng = np.random.default_rng(d * 7 + deg)
