@@ -28,6 +28,9 @@ TRAFFIC_BYTES = {
     "fwd_f32_d5_n7_t4_k1_lds": 64.0e6,
     "fwd_f64_d3_n12_t4_k3": 491.0e6,
     "fwd_f32_d17_n4_t1_k17": 323.4e6,
+    # re-tuned partitions of the same workloads: filled in from the traffic profile
+    "fwd_f64_d3_n12_t5_k1": None,
+    "fwd_f32_d17_n4_t2_k6_lds": None,
 }
 
 

@@ -32,8 +32,8 @@ BUDGET = {("f64", "fwd"): 100, ("f64", "bwd"): 60, ("f32", "fwd"): 170, ("f32", 
 OVERRIDES = {
     # measured on MI355X (kernel ms at the benchmark workloads, see profiles/)
     ("f32", 5, 7, "fwd"): (4, 1),
-    ("f64", 3, 12, "fwd"): (4, 3),
-    ("f32", 17, 4, "fwd"): (1, 17),
+    ("f64", 3, 12, "fwd"): (5, 1),      # 24.1 ms; (4, 3) 25.3, (3, 3) and (4, 1) 31.7
+    ("f32", 17, 4, "fwd"): (2, 6),      # staged 0.66 ms; (1, 17) direct 0.96, (2, 9) staged 0.79, (2, 3) staged 0.91
 }
 
 
@@ -41,7 +41,7 @@ OVERRIDES = {
 # 1 always staged, 2 never staged.  Measured on MI355X at the benchmark workloads.
 STAGE_POLICY = {
     ("f32", 5, 7, "fwd"): 1,
-    ("f32", 17, 4, "fwd"): 2,
+    ("f32", 17, 4, "fwd"): 1,
     ("f64", 3, 12, "fwd"): 2,
 }
 
@@ -135,7 +135,8 @@ def main():
                                           if (tl, kk) != (tail, K)]
                 for (tl, kk, pref) in parts:
                     insts.append((T, D, N, tl, kk, direction, pref, 0))
-                    if D ** (N - tl) >= 48 and D <= 31:       # wide layout: also the LDS-staged variant
+                    # wide layout: also the LDS-staged variant (the backward gains nothing from it beyond ~13 channels)
+                    if D ** (N - tl) >= 48 and D <= (64 if direction == "fwd" else 31):
                         insts.append((T, D, N, tl, kk, direction, pref, 1))
         for N in range(2, MAX_GENERIC_N + 1):
             for direction in ("fwd", "bwd"):

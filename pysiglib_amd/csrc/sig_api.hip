@@ -343,15 +343,20 @@ static int choose_bwd_segments(int64_t waves, int64_t L, uint64_t sig_bytes_all_
 }
 
 // With at most two waves per SIMD the LDS-staged twin (all-VGPR FMAs, HBM latency hidden by a chunk of
-// arithmetic) is the faster way to feed increments; with more resident waves the scalar path costs nothing.
+// arithmetic) is the faster way to feed increments.  With more resident waves it depends (measured over d = 4..24,
+// degrees 4..6, 3-9 waves per SIMD): the f32 forward is always faster staged (1.2-1.8x: SGPR-operand FMAs issue
+// slower than all-VGPR ones), the f32 backward up to 13 channels and both f64 sweeps up to 8 (1.05-1.3x), while with
+// more channels the ring's LDS reads cost them 3-30 % (f64 at 10-12 channels is mixed).
 static int g_force_staged = -1;   // tuning hook: -1 automatic, 0 never, 1 whenever compiled
 
 static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, int64_t waves)
 {
+    const bool small_dim = base->D > 0 && base->D <= (base->is_f64 ? 8 : 13);
     const bool want = g_force_staged >= 0 ? g_force_staged != 0
                       : base->stage_policy == 1 ? true
                       : base->stage_policy == 2 ? false
-                                                : waves <= 2 * int64_t(simd_count());
+                                                : waves <= 2 * int64_t(simd_count()) || small_dim ||
+                                                      (!backward && !base->is_f64);
     if (!want) return base;
     const KernelEntry* twin = staged_twin(backward, base);
     return twin ? twin : base;
