@@ -37,18 +37,40 @@ OVERRIDES = {
 }
 
 
-# which twin (scalar-load or LDS-staged increments) a shape launches: 0 decide by occupancy at run time,
-# 1 always staged, 2 never staged.  Measured on MI355X at the benchmark workloads.
+# which twin (scalar-load or LDS-staged increments) a shape launches: 0 the general rules at run time, 1 always
+# staged, 2 never staged, 3 staged only when the launch leaves SIMDs under-filled.  Measured on MI355X.
 STAGE_POLICY = {
     ("f32", 5, 7, "fwd"): 1,
     ("f32", 17, 4, "fwd"): 1,
     ("f64", 3, 12, "fwd"): 2,
 }
 
+# Partitions and feeds found by a sweep on MI355X (every partition within the register budget whose lane count and
+# letter waste are reasonable, both feeds, at a throughput workload: batch ~3e7 / d^N paths of 128 points): entries
+# that beat the model's choice by at least 12 %.  "staged": 1 always, 3 only when the launch is under-filled.
+# "ms": kernel time of the model's choice and of the entry.  Hand entries above take precedence.
+_TUNED = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuned_partitions.json")
+if os.path.exists(_TUNED):
+    import json
+    with open(_TUNED) as _f:
+        for _k, _v in json.load(_f).items():
+            _dt, _d, _n, _dir = _k.split(",")
+            _key = (_dt, int(_d), int(_n), _dir)
+            if _key not in OVERRIDES:
+                OVERRIDES[_key] = tuple(_v["partition"])
+                STAGE_POLICY[_key] = int(_v["staged"])
+
 # additional partitions compiled next to the default one (selectable through
 # cusig_amd_force_partition; used for tuning sweeps): (dtype, D, N, dir) -> [(TAIL, K), ...]
 EXTRA = {
 }
+# tuning sweeps: SIGAMD_EXTRA_PARTITIONS names a JSON file {"f32,17,4,fwd": [[2, 6], [2, 9]], ...} of more of them
+if os.environ.get("SIGAMD_EXTRA_PARTITIONS"):
+    import json
+    with open(os.environ["SIGAMD_EXTRA_PARTITIONS"]) as _f:
+        for _k, _v in json.load(_f).items():
+            _dt, _d, _n, _dir = _k.split(",")
+            EXTRA[(_dt, int(_d), int(_n), _dir)] = [tuple(x) for x in _v]
 
 
 def spec_shapes():

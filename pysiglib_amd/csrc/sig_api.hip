@@ -355,6 +355,7 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
     const bool want = g_force_staged >= 0 ? g_force_staged != 0
                       : base->stage_policy == 1 ? true
                       : base->stage_policy == 2 ? false
+                      : base->stage_policy == 3 ? waves <= 2 * int64_t(simd_count())
                                                 : waves <= 2 * int64_t(simd_count()) || small_dim ||
                                                       (!backward && !base->is_f64);
     if (!want) return base;

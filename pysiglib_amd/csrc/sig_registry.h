@@ -44,7 +44,7 @@ struct KernelEntry {
     const char* name;
     int preferred;   // default partition of its shape
     int (*waves_per_simd)();   // register-limited residency of the kernel
-    int stage_policy;          // which twin to launch: 0 by occupancy, 1 always the staged one, 2 never
+    int stage_policy;          // which twin to launch: 0 general rules, 1 always the staged one, 2 never, 3 only when under-filled
 };
 
 // every generated instance file contributes one array
