@@ -26,11 +26,8 @@ TRAFFIC_BYTES = {
     "fwd_f64_d10_n5_t2_k5_lds": 53.2e6,
     "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
     "fwd_f32_d5_n7_t4_k1_lds": 64.0e6,
-    "fwd_f64_d3_n12_t4_k3": 491.0e6,
-    "fwd_f32_d17_n4_t1_k17": 323.4e6,
-    # re-tuned partitions of the same workloads: filled in from the traffic profile
-    "fwd_f64_d3_n12_t5_k1": None,
-    "fwd_f32_d17_n4_t2_k6_lds": None,
+    "fwd_f64_d3_n12_t5_k1": 546.3e6,
+    "fwd_f32_d17_n4_t2_k6_lds": 182.8e6,
 }
 
 
