@@ -23,11 +23,11 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 # known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
 # reports null instead of a stale figure.
 TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5_lds": 53.2e6,
+    "fwd_f64_d10_n5_t2_k5_lds": 35.6e6,
     "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
-    "fwd_f32_d5_n7_t4_k1_lds": 64.0e6,
-    "fwd_f64_d3_n12_t5_k1": 546.3e6,
-    "fwd_f32_d17_n4_t2_k6_lds": 182.8e6,
+    "fwd_f32_d5_n7_t4_k1_lds": 55.5e6,
+    "fwd_f64_d3_n12_t5_k1": 477.9e6,
+    "fwd_f32_d17_n4_t2_k6_lds": 113.7e6,
 }
 
 

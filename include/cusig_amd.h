@@ -221,6 +221,10 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
+/* Tuning hook: 0 makes every forward sweep read increments computed by a kernel of their own; 1 (default) lets
+ * the LDS-staged sweeps of plain paths (no time or lead-lag augmentation) of at most 16 channels take the
+ * differences of consecutive points while they stage them. */
+CUSIG_AMD_API void cusig_amd_set_point_fed(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: how increments reach the waves: -1 automatic, 0 scalar loads, 1 LDS-staged where compiled. */

@@ -192,7 +192,7 @@ def main():
             zs = "true" if zl else "false"
             if direction == "fwd":
                 lines.append("template __global__ void tree_fwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, %s*, int64_t, "
-                             "int64_t, int, int64_t, int, int, int64_t, int*);" % (T, D, N, tail, K, zs, T, T))
+                             "int64_t, int, int64_t, int, int, int64_t, int*, int);" % (T, D, N, tail, K, zs, T, T))
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
                              "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))

@@ -297,6 +297,7 @@ static int* nonfinite_flag()
 // time segmentation of the forward sweep
 // ---------------------------------------------------------------------------
 static int g_force_segments = 0;   // tuning hook (0 = automatic)
+static int g_point_fed = 1;        // tuning hook: 0 always computes the increments in a kernel of their own
 
 static int simd_count()
 {
@@ -527,10 +528,6 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         if (!e)
             throw std::runtime_error("signature_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
-        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
-        const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;    // staged sweeps read whole chunks past either end
-        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
-        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
         // Few paths cannot fill the chip with whole-path sweeps: split every path into time segments,
         // sweep all (path, segment) pairs concurrently and fold the pieces with Chen's identity.
         const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
@@ -540,7 +537,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                                                batch * (s.full_len - 1) * sizeof(T));
         const uint64_t n_coef = s.full_len - 1;
         FwdParams p;
-        p.inc = inc; p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
+        p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
         p.lseg = (int64_t(s.L) + nseg - 1) / nseg;
         nseg = int((int64_t(s.L) + p.lseg - 1) / p.lseg);      // drop segments the rounding left empty
         p.nseg = nseg;
@@ -560,6 +557,17 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             p.out = segs; p.out_stride = int64_t(n_coef); p.scalar = 0;
         }
         e = pick_variant(false, e, total_waves(geom, p.batch));
+        // staged sweeps of plain narrow paths form the increments themselves while staging the points
+        if (e->staged && !time_aug && !lead_lag && e->D > 0 && e->D <= kPointFedMaxDim && g_point_fed) {
+            p.inc = path;
+            p.from_points = 1;
+        } else {
+            const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+            const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;    // staged sweeps read whole chunks past either end
+            T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
+            compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+            p.inc = inc;
+        }
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->fwd(p));
         timer.stop();
@@ -822,6 +830,7 @@ CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
 
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
+CUSIG_AMD_API void cusig_amd_set_point_fed(int on) noexcept { g_point_fed = on; }
 
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force_bwd_segments = segments; }
 

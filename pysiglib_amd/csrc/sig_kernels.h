@@ -79,11 +79,11 @@ struct LaneCtx {
     int p[M];
     int a0;
 
-    __device__ __forceinline__ void init(int d_rt, int64_t batch)
+    __device__ __forceinline__ void init(int d_rt, int64_t batch, bool xcd = true)
     {
         d = D > 0 ? D : d_rt;
         G = make_geom(d, M, K, D != 0);
-        id = lane_id<WIDE>(G, batch);
+        id = lane_id<WIDE>(G, batch, xcd);
         // idle lanes shadow a valid lane so that every load stays in bounds;
         // they never store and never contribute
         if constexpr (WIDE) {
@@ -190,9 +190,14 @@ struct IncRing {
     {
         return DIR > 0 ? parity * CHUNK : D + (1 - parity) * CHUNK;
     }
+    // The ring can also be fed from the points of a plain path (no augmentation): element e of a chunk is then
+    // x[e + D] - x[e], the two loads travel in `regs` and `ahead` and are subtracted when the chunk is committed.
+    // Only narrow paths get the second register set.
+    static constexpr bool kPoints = NREG <= 4;
     T* lds;
     int lane;
     T regs[NREG];
+    T ahead[kPoints ? NREG : 1];
 
     __device__ __forceinline__ void issue(const T* __restrict__ g)
     {
@@ -202,17 +207,35 @@ struct IncRing {
             regs[i] = ((i + 1) * kWave <= CHUNK || e < CHUNK) ? g[e] : T(0);
         }
     }
-    __device__ __forceinline__ void commit(int parity)
+    // g: the point whose increment is element 0 of the chunk; elements outside [lo, hi) are not read and count as 0
+    // (nothing before the first or after the last point of the swept range is touched)
+    __device__ __forceinline__ void issue_points(const T* __restrict__ g, int lo, int hi)
+    {
+        if constexpr (kPoints) {
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) {
+                const int e = lane + kWave * i;
+                const bool ok = e >= lo && e < hi;
+                regs[i] = ok ? g[e] : T(0);
+                ahead[i] = ok ? g[e + D] : T(0);
+            }
+        }
+    }
+    __device__ __forceinline__ void commit(int parity, bool points = false)
     {
         T* dst = lds + base(parity);
 #pragma unroll
         for (int i = 0; i < NREG; ++i) {
             const int e = lane + kWave * i;
             if ((i + 1) * kWave <= CHUNK || e < CHUNK) {
-                dst[e] = regs[i];
+                T v = regs[i];
+                if constexpr (kPoints) {
+                    if (points) v = ahead[i] - v;
+                }
+                dst[e] = v;
                 if (parity == 0) {
-                    if (DIR > 0) { if (e < D) lds[2 * CHUNK + e] = regs[i]; }
-                    else { if (e >= CHUNK - D) lds[e - (CHUNK - D)] = regs[i]; }
+                    if (DIR > 0) { if (e < D) lds[2 * CHUNK + e] = v; }
+                    else { if (e >= CHUNK - D) lds[e - (CHUNK - D)] = v; }
                 }
             }
         }
@@ -254,9 +277,11 @@ __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__
 }
 
 // staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0
+// points (wave-uniform; forward sweeps of plain paths only): `row` is the path point of the first step instead of an
+// increment row, and the ring takes differences of consecutive points.
 template <int DIR, int G0, typename Tr, typename Cx, typename T, typename StepFn>
 __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
-                                             T* lds_wave, StepFn&& step)
+                                             T* lds_wave, StepFn&& step, bool points = false)
 {
     constexpr int D = Tr::DD;
     using Ring = IncRing<T, D, DIR>;
@@ -285,16 +310,25 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
         for (int l = 0; l < Tr::M; ++l) in.pz[l] = lp[cx.p[l]];
     };
 
-    ring.issue(chunk_src(0));
-    ring.commit(0);
-    if (nchunks > 1) ring.issue(chunk_src(1));
+    // chunk k holds the elements [k * CHUNK, (k + 1) * CHUNK) of the range; count * D of them exist
+    auto issue = [&](int64_t k) {
+        if (DIR > 0 && Ring::kPoints && points) {
+            const int64_t left = count * D - k * Ring::CHUNK;
+            ring.issue_points(chunk_src(k), 0, left < Ring::CHUNK ? int(left) : Ring::CHUNK);
+        } else {
+            ring.issue(chunk_src(k));
+        }
+    };
+    issue(0);
+    ring.commit(0, points);
+    if (nchunks > 1) issue(1);
     typename Tr::Inc za, zb;
     load_row(za, ring.lds + Ring::base(0) + (DIR > 0 ? 0 : (CS - 1) * D));
     int64_t done = 0;
     for (int64_t k = 0; k < nchunks; ++k) {
         const int parity = int(k & 1);
-        if (k + 1 < nchunks) ring.commit(parity ^ 1);            // chunk k+1 becomes readable
-        if (k + 2 < nchunks) ring.issue(chunk_src(k + 2));       // two chunks ahead of use
+        if (k + 1 < nchunks) ring.commit(parity ^ 1, points);    // chunk k+1 becomes readable
+        if (k + 2 < nchunks) issue(k + 2);                       // two chunks ahead of use
         // the row pointer is made opaque so that row reads use small immediate offsets from one VGPR
         const T* lp = opaque_lds(ring.lds + Ring::base(parity) + (DIR > 0 ? 0 : (CS - 1) * D));
         const int nk = int((count - done < CS) ? count - done : CS);
@@ -319,9 +353,11 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d_rt,
-    int64_t out_stride, int scalar, int nseg, int64_t lseg, int* __restrict__ nonfinite)
+    int64_t out_stride, int scalar, int nseg, int64_t lseg, int* __restrict__ nonfinite, int from_points)
 {
     // `nonfinite` (may be null): set to 1 when any stored value is NaN or infinite.
+    // `from_points` (staged kernels of narrow paths only): `inc` is the plain path [batch][L + 1][d] itself and the
+    // increments are formed while they are staged.
     // `batch` counts (path, time segment) pairs: item vb = path * nseg + segment sweeps the
     // increments [segment * lseg, min(L, (segment + 1) * lseg)) and stores the signature of
     // that piece in row vb of `out`.  nseg == 1 is the plain whole-path sweep.
@@ -343,20 +379,22 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const int64_t seg = cx.id.b % nseg;
     const int64_t t0 = seg * lseg;
     const int64_t ns = (L - t0 < lseg) ? L - t0 : lseg;      // steps of this segment (>= 1)
-    const T* row = inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;     // row of the segment's first step
+    // row of the segment's first step (increments: [batch][L + 2][d] with a zero row at either end)
+    const T* row = from_points ? inc + ((cx.id.b / nseg) * (L + 1) + t0) * d : inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;
     auto step = [&](const typename Tr::Inc& z, int64_t, auto) { S.fwd_step(z); };
     if constexpr (ZL) {
         static_assert(LaneCtx<T, D, N, TAIL, K>::WIDE, "staged increments need the wide layout");
         extern __shared__ double lds_raw_f[];
         T* lds_wave = reinterpret_cast<T*>(lds_raw_f) + (threadIdx.x >> 6) * IncRing<T, Tr::DD, 1>::ELEMS;
         constexpr int NG = (Tr::DD + K - 1) / K;
+        const bool points = IncRing<T, Tr::DD, 1>::kPoints && from_points != 0;
         if constexpr (NG <= 3) {
             static_for<0, NG - 1>([&](auto gc) {
                 if (cx.id.g == decltype(gc)::value)
-                    sweep_staged<1, decltype(gc)::value * K, Tr>(cx, row, t0, ns, lds_wave, step);
+                    sweep_staged<1, decltype(gc)::value * K, Tr>(cx, row, t0, ns, lds_wave, step, points);
             });
         } else {
-            sweep_staged<1, -1, Tr>(cx, row, t0, ns, lds_wave, step);
+            sweep_staged<1, -1, Tr>(cx, row, t0, ns, lds_wave, step, points);
         }
     } else {
         sweep_direct<1, true, LaneCtx<T, D, N, TAIL, K>, typename Tr::Inc>(cx, row, t0, ns, step);
@@ -462,6 +500,15 @@ __device__ __forceinline__ void dev_add(T* p, T v)
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The forward sweep numbers its blocks per XCD (xcd_block): its HBM reads drop to the size of the path.  The backward
+// keeps the dispatch order: with all waves of a path behind one L2 the atomic adds into a gradient row queue up in
+// one cache channel instead of eight, which costs more (0.5 % of the sweep at batch 32, length 1000, d = 10, degree 5)
+// than the saved re-reads of the increment rows give back.  -DSIGAMD_BWD_XCD=1 switches it on for measurements.
+#ifndef SIGAMD_BWD_XCD
+#define SIGAMD_BWD_XCD 0
+#endif
+constexpr bool kBwdXcd = SIGAMD_BWD_XCD != 0;
+
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
@@ -482,7 +529,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     T* lds = reinterpret_cast<T*>(lds_raw);
 
     Cx cx;
-    cx.init(d_rt, batch);
+    cx.init(d_rt, batch, kBwdXcd);
     if constexpr (Cx::WIDE) {
         if (cx.id.b >= batch) return;
     }
@@ -548,7 +595,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     }
     int64_t b_first;
     {
-        const int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + wave_in_block;
+        const int64_t wave = xcd_block(kBwdXcd) * kWavesPerBlock + wave_in_block;
         b_first = (slots > 1) ? wave * slots : (wave / cx.G.wpp);
     }
     // path and first step of an item (whole paths skip the divisions)

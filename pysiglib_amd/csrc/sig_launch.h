@@ -26,6 +26,9 @@ hipError_t launch_tree_fwd(const FwdParams& p)
     const int64_t waves = total_waves(g, p.batch);
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
+    static_assert(!ZL || D <= 0 || IncRing<T, (D > 0 ? D : 1), 1>::kPoints == (D <= kPointFedMaxDim),
+                  "the ring's point-fed mode and the host's limit must agree");
+    if (p.from_points && !(ZL && D > 0 && D <= kPointFedMaxDim)) return hipErrorInvalidConfiguration;
     size_t lds = 0;
     if (ZL) {
         if (!g.wide) return hipErrorInvalidConfiguration;
@@ -35,7 +38,7 @@ hipError_t launch_tree_fwd(const FwdParams& p)
     }
     hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
-                       p.out_stride, p.scalar, p.nseg, p.lseg, p.nonfinite);
+                       p.out_stride, p.scalar, p.nseg, p.lseg, p.nonfinite, (ZL && D > 0 && D <= kPointFedMaxDim) ? p.from_points : 0);
     return hipGetLastError();
 }
 

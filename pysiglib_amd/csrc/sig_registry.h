@@ -16,7 +16,9 @@ struct FwdParams {
     int nseg;        // time segments per path; batch counts (path, segment) items
     int64_t lseg;    // increments per segment
     int* nonfinite = nullptr;   // device-visible flag set when a stored value is NaN or infinite (may be null)
+    int from_points = 0;        // staged kernels of at most kPointFedMaxDim channels: inc is the plain path [batch][L + 1][d]
 };
+constexpr int kPointFedMaxDim = 16;
 
 struct BwdParams {
     const void* inc;

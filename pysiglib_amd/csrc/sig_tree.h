@@ -93,12 +93,25 @@ struct LaneId {
     bool active;
 };
 
+// The dispatcher deals the blocks of a grid to the 8 XCDs in turn (block p runs on XCD p % 8), and every XCD has an
+// L2 of its own.  Renumbering the blocks so that each XCD works on one contiguous range keeps the waves of a path
+// (which read the same increment rows and add into the same gradient rows) behind one L2: the rows are fetched from
+// HBM once instead of once per XCD, and the atomics of a row meet in one cache.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ int64_t xcd_block(bool on = true)
+{
+    const uint32_t nb = gridDim.x, p = blockIdx.x;
+    if (!on) return p;
+    const uint32_t x = p % kXcds, base = nb / kXcds, rem = nb % kXcds;
+    return int64_t(x) * base + (x < rem ? x : rem) + p / kXcds;
+}
+
 template <bool WIDE>
-__device__ __forceinline__ LaneId lane_id(const TreeGeom& G, int64_t batch)
+__device__ __forceinline__ LaneId lane_id(const TreeGeom& G, int64_t batch, bool xcd)
 {
     LaneId id;
     const int lane = threadIdx.x & (kWave - 1);
-    int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    int64_t wave = xcd_block(xcd) * kWavesPerBlock + (threadIdx.x >> 6);
     id.slot = 0;
     if constexpr (WIDE) {
         // wave-uniform quantities are forced into SGPRs

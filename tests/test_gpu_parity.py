@@ -209,6 +209,50 @@ def test_batch_dims_views_and_warnings(P, oracle):
         P.sig(torch.full((1, 3, 2), 1e200, dtype=torch.float64, device=DEV).cumsum(1), 3)
 
 
+def test_point_fed_staging(P):
+    """Staged forward sweeps of plain paths of at most 16 channels difference the points while staging them; the
+    result must equal, bit for bit, the sweep fed by the increments kernel (same subtractions, same order), for
+    lengths around the 16-step chunk, forced time segments and the last path of the batch (whose final chunk must
+    not read past the end of the path buffer)."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_point_fed.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_point_fed.restype = None
+    L.CUSIG.cusig_amd_force_staged.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_staged.restype = None
+    rng = np.random.default_rng(4242)
+    fed = 0
+    try:
+        L.CUSIG.cusig_amd_force_staged(1)
+        for (d, n) in ((10, 5), (5, 7), (4, 8), (16, 4), (17, 4), (12, 4), (6, 6)):
+            for length in (2, 3, 16, 17, 18, 33, 100):
+                for segments in (0, 3):
+                    for dtype in (torch.float64, torch.float32):
+                        x = torch.as_tensor(rng.standard_normal((48, length, d)), dtype=dtype, device=DEV)
+                        L.CUSIG.cusig_amd_force_segments(segments)
+                        L.CUSIG.cusig_amd_set_point_fed(0)
+                        ref = P.sig(x, n)
+                        L.CUSIG.cusig_amd_set_point_fed(1)
+                        L.CUSIG.cusig_amd_set_profiling(1)
+                        out = P.sig(x, n)
+                        name = L.CUSIG.cusig_amd_last_kernel_name().decode()
+                        L.CUSIG.cusig_amd_set_profiling(0)
+                        fed += name.endswith("_lds") and d <= 16
+                        assert torch.equal(out, ref), (d, n, length, segments, dtype, name)
+        # augmented paths keep the increments kernel: same answers either way
+        x = torch.as_tensor(rng.standard_normal((3, 20, 4)), dtype=torch.float64, device=DEV)
+        L.CUSIG.cusig_amd_set_point_fed(0)
+        ref = P.sig(x, 4, time_aug=True, lead_lag=True)
+        L.CUSIG.cusig_amd_set_point_fed(1)
+        assert torch.equal(P.sig(x, 4, time_aug=True, lead_lag=True), ref)
+    finally:
+        L.CUSIG.cusig_amd_force_segments(0)
+        L.CUSIG.cusig_amd_set_point_fed(1)
+        L.CUSIG.cusig_amd_force_staged(-1)
+    assert fed > 100     # the staged kernels did run
+
+
 def test_overflow_report(P):
     """The kernels that store the signature flag NaN / Inf themselves (the reference scans the result,
     pysiglib/sig.py:299-310): the report must agree with a scan on every forward route."""
