@@ -65,8 +65,8 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_init_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, T* __restrict__ dB, int64_t batch, I init_len, int64_t stride, int off,
     int identity, int64_t dc_share, int64_t dc_stride, int dc_off, int families)
 {
-    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < init_len; r += I(gridDim.x) * kBlock) {
+    for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
+        for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < init_len; r += I(gridDim.x) * kBlock) {
             const T v = identity ? dC[(b / dc_share) * dc_stride + dc_off + r] : T(0);
             dA[b * stride + off + r] = v;
             if (families > 1) dB[b * stride + off + r] = v;
@@ -81,9 +81,9 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
     int64_t dc_share, int64_t dc_stride, int dc_off, int families)
 {
     const int N = plan.degree;
-    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+    for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         const T* g = dC + (b / dc_share) * dc_stride + dc_off;
-        for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < I(families) * plan.items; it += I(gridDim.x) * kBlock) {
+        for (I it = I(xcd_block_2d().x) * kBlock + threadIdx.x; it < I(families) * plan.items; it += I(gridDim.x) * kBlock) {
             const bool fam_b = it >= plan.items;
             const I i2 = fam_b ? it - plan.items : it;
             int t = 1;
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
             const I x0 = q * kCombChunk;
             const I x1 = x0 + kCombChunk < s_t ? x0 + kCombChunk : s_t;
             const T* other = (fam_b ? A : B) + b * stride + off;      // the factor the sum runs over
-            T s0 = T(0), s1 = T(0);
+            T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
             for (int m = 1; m <= N - t; ++m) {
                 const I seg0 = plan.lo[m] > x0 ? plan.lo[m] : x0;
                 const I seg1 = plan.lo[m + 1] < x1 ? plan.lo[m + 1] : x1;
@@ -105,25 +105,35 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
                 if (!fam_b) {
                     const T* blockp = up + w * (plan.lo[m + 1] - plan.lo[m]) - plan.lo[m];    // words w v
                     I x = seg0;
-                    for (; x + 2 <= seg1; x += 2) {
-                        s0 = fmadd(blockp[x], other[x], s0);
-                        s1 = fmadd(blockp[x + 1], other[x + 1], s1);
+                    for (; x + 4 <= seg1; x += 4) {      // all eight loads are issued before the first product needs one
+                        const T g0 = blockp[x], g1 = blockp[x + 1], g2 = blockp[x + 2], g3 = blockp[x + 3];
+                        const T o0 = other[x], o1 = other[x + 1], o2 = other[x + 2], o3 = other[x + 3];
+                        s0 = fmadd(g0, o0, s0);
+                        s1 = fmadd(g1, o1, s1);
+                        s2 = fmadd(g2, o2, s2);
+                        s3 = fmadd(g3, o3, s3);
                     }
-                    if (x < seg1) s0 = fmadd(blockp[x], other[x], s0);
+                    for (; x < seg1; ++x) s0 = fmadd(blockp[x], other[x], s0);
                 } else {
                     const T* strided = up + w;                         // words u w: index u * d^t + w
                     I x = seg0;
-                    for (; x + 2 <= seg1; x += 2) {
-                        s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
-                        s1 = fmadd(strided[(x + 1 - plan.lo[m]) * sz_t], other[x + 1], s1);
+                    for (; x + 4 <= seg1; x += 4) {
+                        const T* sp = strided + (x - plan.lo[m]) * sz_t;
+                        const T g0 = sp[0], g1 = sp[sz_t], g2 = sp[2 * sz_t], g3 = sp[3 * sz_t];
+                        const T o0 = other[x], o1 = other[x + 1], o2 = other[x + 2], o3 = other[x + 3];
+                        s0 = fmadd(g0, o0, s0);
+                        s1 = fmadd(g1, o1, s1);
+                        s2 = fmadd(g2, o2, s2);
+                        s3 = fmadd(g3, o3, s3);
                     }
-                    if (x < seg1) s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
+                    for (; x < seg1; ++x) s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
                 }
             }
             const I r = plan.lo[t] + w;
             T* dst = (fam_b ? dB : dA) + b * stride + off + r;
-            if (plan.parts[t] == 1) *dst = (identity ? g[r] : T(0)) + (s0 + s1);
-            else dev_add(dst, s0 + s1);
+            const T sum = (s0 + s1) + (s2 + s3);
+            if (plan.parts[t] == 1) *dst = (identity ? g[r] : T(0)) + sum;
+            else dev_add(dst, sum);
             if (off && it == 0) {
                 dA[b * stride] = T(0);
                 if (families > 1) dB[b * stride] = T(0);

@@ -33,11 +33,11 @@ __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
     T inv_k, int64_t stride, int off, int64_t out_stride, int final)
 {
     const I d = I(dv.d);
-    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+    for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         const T* x = X + b * stride + off;
         const T* pin = Pin + b * stride + off;
         T* po = Pout + b * out_stride + off;
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < count; r += I(gridDim.x) * kBlock) {
+        for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < count; r += I(gridDim.x) * kBlock) {
             const WordPos<I> p = word_pos<I>(r, d);
             T acc = T(0);
             I pre = p.w, suf = 0, pw = 1;

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
     const I d = I(dv.d);
     // `copies` private sets of d accumulators, chosen by lane: few letters mean many lanes adding to one word
     T* mine = acc + (threadIdx.x % copies) * d;
-    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+    for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         if (use_lds) {
             __syncthreads();
             for (I j = threadIdx.x; j < I(copies) * d; j += kBlock) acc[j] = T(0);
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
         const T* z = disp + b * int64_t(d);
         const T* g = dE + b * stride + off;
         T* out = dz + b * int64_t(d);
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
+        for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
             const WordPos<I> p = word_pos<I>(r, d);
             T suf[kExpMaxDegree];       // suf[i] = dE[w] / t! * z[w_{i+2}] ... z[w_t]   (0-based position i)
             I let[kExpMaxDegree];

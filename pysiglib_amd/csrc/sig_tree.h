@@ -106,6 +106,20 @@ __device__ __forceinline__ int64_t xcd_block(bool on = true)
     return int64_t(x) * base + (x < rem ? x : rem) + p / kXcds;
 }
 
+// The same for 2-D grids (x: work inside a row, y: rows), which are dispatched x-fastest: each XCD takes whole rows
+// one after the other, so a row that several blocks read again and again is fetched into one L2 only.
+struct Block2 {
+    uint32_t x, y;
+};
+__device__ __forceinline__ Block2 xcd_block_2d()
+{
+    const uint32_t gx = gridDim.x;
+    const uint64_t nb = uint64_t(gx) * gridDim.y, p = uint64_t(blockIdx.y) * gx + blockIdx.x;
+    const uint64_t x = p % kXcds, base = nb / kXcds, rem = nb % kXcds;
+    const uint64_t l = x * base + (x < rem ? x : rem) + p / kXcds;
+    return Block2{uint32_t(l % gx), uint32_t(l / gx)};
+}
+
 template <bool WIDE>
 __device__ __forceinline__ LaneId lane_id(const TreeGeom& G, int64_t batch, bool xcd)
 {
