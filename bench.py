@@ -294,7 +294,10 @@ def main():
             wall, kms, name = time_calls(r.forward, torch, loader, 1, n)
             tf = r.flops_fwd / (kms * 1e-3) / 1e12
             configs["C%d" % k] = {"signatures_per_s": r.c["batch"] / wall, "call_ms": wall * 1e3, "kernel": name,
-                                  "kernel_ms": kms, "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS[r.dtype]}
+                                  "kernel_ms": kms, "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS[r.dtype],
+                                  # the whole call (sweep plus, when the paths were cut in time, the Chen folds)
+                                  "call_roofline_frac": r.flops_fwd / wall / 1e12 / PEAK_TFLOPS[r.dtype],
+                                  "time_segments": int(loader.CUSIG.cusig_amd_last_segments())}
             del r
             torch.cuda.empty_cache()
         # degree 2 on paths of many channels: closed form on the matrix cores (not one of the five benchmark workloads)

@@ -221,6 +221,8 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
+/* Number of time segments per path in the last forward sweep on this thread (0 if no sweep kernel ran). */
+CUSIG_AMD_API int cusig_amd_last_segments(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: 0 makes every forward sweep read increments computed by a kernel of their own; 1 (default) lets
  * the LDS-staged sweeps of plain paths (no time or lead-lag augmentation) of at most 16 channels take the
  * differences of consecutive points while they stage them. */

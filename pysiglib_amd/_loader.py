@@ -35,6 +35,8 @@ CUSIG.cusig_amd_last_sig_nonfinite.argtypes = ()
 CUSIG.cusig_amd_last_sig_nonfinite.restype = c_int
 CUSIG.cusig_amd_set_profiling.argtypes = (c_int,)
 CUSIG.cusig_amd_set_profiling.restype = None
+CUSIG.cusig_amd_last_segments.argtypes = ()
+CUSIG.cusig_amd_last_segments.restype = c_int
 CUSIG.cusig_amd_last_kernel_ms.argtypes = ()
 CUSIG.cusig_amd_last_kernel_ms.restype = c_float
 CUSIG.cusig_amd_last_kernel_name.argtypes = ()

@@ -253,10 +253,17 @@ struct MainKernelTimer {
         std::snprintf(g_last_name, sizeof g_last_name, "%s", name);
         SIG_HIP(hipEventRecord(g_ev0, s));
     }
-    void stop()
+    // defer: only mark the end; read() fetches the duration later, so that kernels enqueued after the timed one do
+    // not wait for a host round trip
+    void stop(bool defer = false)
     {
         if (!on) return;
         SIG_HIP(hipEventRecord(g_ev1, s));
+        if (!defer) read();
+    }
+    void read()
+    {
+        if (!on) return;
         SIG_HIP(hipEventSynchronize(g_ev1));
         SIG_HIP(hipEventElapsedTime(&g_last_ms, g_ev0, g_ev1));
     }
@@ -297,6 +304,7 @@ static int* nonfinite_flag()
 // time segmentation of the forward sweep
 // ---------------------------------------------------------------------------
 static int g_force_segments = 0;   // tuning hook (0 = automatic)
+static thread_local int tl_last_segments = 0;   // pieces per path of the last forward sweep on this thread (0: no sweep ran)
 static int g_point_fed = 1;        // tuning hook: 0 always computes the increments in a kernel of their own
 
 static int simd_count()
@@ -311,18 +319,50 @@ static int simd_count()
     return cached;
 }
 
-// Splitting costs one extra signature write per segment plus the Chen folds, so it only pays when whole-path
-// sweeps leave more than half of the SIMDs without a wave.  Then aim at two waves per SIMD (never more than the
-// kernel's registers allow), with segments of at least 48 increments and at most 256 MB of segment signatures.
-static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_t sig_bytes_all_paths)
+// Cutting every path into g pieces of 1/g of the steps multiplies the waves and divides the chain of dependent
+// steps; it costs one signature write per piece plus the Chen folds.  Two situations pay:
+//  * under-filled: whole-path sweeps leave SIMDs without a wave (few paths);
+//  * unevenly filled: a few waves per SIMD, and the fullest SIMD holds one more than most (1280 waves on 1024 SIMDs
+//    that hold two each run as long as 2048 would); the launch lasts as long as its fullest SIMD needs, and shorter
+//    pieces even the load out.
+// A small model picks g: the fullest SIMD works through its waves `waves_per_simd` at a time, a SIMD with two or
+// more resident waves issuing `pair_rate` times as fast as with one; a step of a lone wave takes 2.4 ns per
+// instruction of lane_step_cost, and at least 240 ns when its increments come straight from memory instead of the
+// LDS ring (lane_step(g) says which, for the launch g pieces make); the folds cost a fixed 8 us, 10 us per launch
+// and 2.2 signature sets of traffic per piece at 4 TB/s (measured: d = 12, degree 4, 48 paths of 300 steps: whole
+// 92 us, 2 pieces 77, 3: 76, 4: 94, 6: 101 us).  Pieces keep at least 48 steps and 256 MB of segment signatures at most, and a
+// split must promise 7 % (batch 128, length 1024, d = 5, degree 7, f32: 0.587 -> 0.523 ms with three pieces).
+template <typename LaneStep>
+static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_t sig_bytes_all_paths, LaneStep&& lane_step,
+                           bool f64)
 {
     const int64_t simds = simd_count();
-    if (waves <= 0 || waves * 2 > simds) return 1;
-    int64_t g = int64_t(std::min(waves_per_simd, 2)) * simds / waves;
-    g = std::min<int64_t>(g, 32);
-    g = std::min<int64_t>(g, L / 48);
-    if (sig_bytes_all_paths > 0) g = std::min<int64_t>(g, int64_t((uint64_t(256) << 20) / sig_bytes_all_paths));
-    return int(std::max<int64_t>(g, 1));
+    if (waves <= 0 || sig_bytes_all_paths == 0) return 1;
+    const int occ = std::max(1, waves_per_simd);
+    if (waves > 4 * simds * occ) return 1;
+    const double pair_rate = f64 ? 1.2 : 1.35;
+    auto estimate = [&](int g) {
+        const int64_t fullest = (waves * g + simds - 1) / simds;          // waves of the fullest SIMD
+        const int64_t rounds = fullest / occ, rest = fullest % occ;
+        double steps = double(rounds) * occ / (occ > 1 ? pair_rate : 1.0);
+        if (rest) steps += double(rest) / (rest > 1 ? pair_rate : 1.0);
+        double t = double((L + g - 1) / g) * lane_step(g) * steps;
+        if (g > 1) {
+            int launches = 0;
+            for (int m = g; m > 1; m = (m + 1) / 2) ++launches;
+            t += 8e-6 + 10e-6 * launches + 2.2 * g * double(sig_bytes_all_paths) / 4e12;
+        }
+        return t;
+    };
+    int best = 1;
+    double best_t = estimate(1);
+    const double whole = best_t;
+    for (int g : {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32}) {
+        if (L / g < 48 || uint64_t(g) * sig_bytes_all_paths > (uint64_t(256) << 20)) break;
+        const double t = estimate(g);
+        if (t < best_t) { best = g; best_t = t; }
+    }
+    return best_t < 0.93 * whole ? best : 1;
 }
 
 // The backward sweep can be cut in time as well: the state at the end of segment g is the Chen product of the
@@ -534,13 +574,20 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         int nseg = g_force_segments > 0
                              ? int(std::min<uint64_t>(uint64_t(g_force_segments), s.L))
                              : choose_segments(total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
-                                               batch * (s.full_len - 1) * sizeof(T));
+                                               batch * (s.full_len - 1) * sizeof(T),
+                                               [&](int g) {
+                                                   const double c = lane_step_cost(int(s.d_aug), e->N, e->tail, e->k) * 2.4e-9;
+                                                   const bool ring = pick_variant(false, e, total_waves(geom, int64_t(batch)) * g)->staged;
+                                                   return ring ? c : std::max(c, 240e-9);
+                                               },
+                                               sizeof(T) == 8);
         const uint64_t n_coef = s.full_len - 1;
         FwdParams p;
         p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
         p.lseg = (int64_t(s.L) + nseg - 1) / nseg;
         nseg = int((int64_t(s.L) + p.lseg - 1) / p.lseg);      // drop segments the rounding left empty
         p.nseg = nseg;
+        tl_last_segments = nseg;
         p.batch = int64_t(batch) * nseg;
         T* segs = nullptr;
         T* folds = nullptr;
@@ -570,7 +617,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         }
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->fwd(p));
-        timer.stop();
+        timer.stop(/*defer=*/true);
         if (nseg > 1) {
             // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches
             const T* src = segs;
@@ -579,11 +626,15 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                 const bool last = m == 2;
                 const int half = (m + 1) / 2;
                 T* dst = last ? out : next;
-                launch_indexed(n_coef, n_coef, batch * uint64_t(half), [&](auto ix, dim3 grid) {
-                    using I = decltype(ix);
-                    hipLaunchKernelGGL((chen_fold_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, src, dst, int64_t(batch), m,
-                                       last ? int64_t(s.stride) : int64_t(n_coef) * half, last ? sc : 0, DivBy<I>(s.d_aug),
-                                       I(n_coef), last ? flag : nullptr);
+                with_chen_fan(s.d_aug, [&](auto fan) {
+                    constexpr int FAN = decltype(fan)::value;
+                    const uint64_t items = chen_items(s.d_aug, degree, FAN);
+                    launch_indexed(n_coef, items, batch * uint64_t(half), [&](auto ix, dim3 grid) {
+                        using I = decltype(ix);
+                        hipLaunchKernelGGL((chen_fold_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, src, dst,
+                                           int64_t(batch), m, last ? int64_t(s.stride) : int64_t(n_coef) * half, last ? sc : 0,
+                                           DivBy<I>(s.d_aug), I(n_coef), I(items), last ? flag : nullptr);
+                    });
                 });
                 SIG_HIP(hipGetLastError());
                 src = dst;
@@ -591,6 +642,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             }
         }
         exit_sync(stream);
+        timer.read();
         if (flag) tl_sig_nonfinite = *g_flag_host;
         return;
     }
@@ -726,10 +778,15 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                 const bool last = k == steps - 1;
                 T* xdst = last ? left : scratch + uint64_t(k & 1) * 2 * buf;
                 T* zdst = last ? right : scratch + (uint64_t(k & 1) * 2 + 1) * buf;
-                launch_indexed(n_coef, n_coef, 2 * rows, [&](auto ix, dim3 grid) {
-                    using I = decltype(ix);
-                    hipLaunchKernelGGL((chen_scan_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, xsrc, zsrc, xdst, zdst,
-                                       int64_t(batch), nseg, 1 << k, k == 0 ? 1 : 0, DivBy<I>(s.d_aug), I(n_coef));
+                with_chen_fan(s.d_aug, [&](auto fan) {
+                    constexpr int FAN = decltype(fan)::value;
+                    const uint64_t items = chen_items(s.d_aug, degree, FAN);
+                    launch_indexed(n_coef, items, 2 * rows, [&](auto ix, dim3 grid) {
+                        using I = decltype(ix);
+                        hipLaunchKernelGGL((chen_scan_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, xsrc, zsrc, xdst,
+                                           zdst, int64_t(batch), nseg, 1 << k, k == 0 ? 1 : 0, DivBy<I>(s.d_aug), I(n_coef),
+                                           I(items));
+                    });
                 });
                 xsrc = xdst;
                 zsrc = zdst;
@@ -830,6 +887,7 @@ CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; 
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
 
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
+CUSIG_AMD_API int cusig_amd_last_segments(void) noexcept { return tl_last_segments; }
 CUSIG_AMD_API void cusig_amd_set_point_fed(int on) noexcept { g_point_fed = on; }
 
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force_bwd_segments = segments; }

@@ -27,34 +27,19 @@ namespace sigamd {
 
 // P_out[r] = inv_k * x[r] - sum_{l=1..t-1} x_l[w_1..w_l] * P_in_{t-l}[w_{l+1}..w_t]   for the `count` coefficients of
 // levels <= top.  x and the P buffers share one row layout (stride, off); `final` also clears the scalar slot.
-template <typename T, typename I>
+template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
-    const T* __restrict__ X, const T* __restrict__ Pin, T* __restrict__ Pout, int64_t batch, DivBy<I> dv, I count,
-    T inv_k, int64_t stride, int off, int64_t out_stride, int final)
+    const T* __restrict__ X, const T* __restrict__ Pin, T* __restrict__ Pout, int64_t batch, DivBy<I> dv,
+    I items /* chen_items(d, levels, FAN) */, T inv_k, int64_t stride, int off, int64_t out_stride, int final)
 {
-    const I d = I(dv.d);
     for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         const T* x = X + b * stride + off;
         const T* pin = Pin + b * stride + off;
         T* po = Pout + b * out_stride + off;
-        for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < count; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T acc = T(0);
-            I pre = p.w, suf = 0, pw = 1;
-            I a_lo = p.lo, a_sz = p.size;
-            I b_lo = 0;
-            for (int l = p.t - 1; l >= 1; --l) {        // split after l letters, as in the Chen product kernel
-                const I q = dv.quot(pre);
-                suf += (pre - q * d) * pw;
-                pw *= d;
-                pre = q;
-                a_sz = dv.quot(a_sz);
-                a_lo -= a_sz;
-                acc = fmadd(x[a_lo + pre], pin[b_lo + suf], acc);
-                b_lo += pw;
-            }
-            po[r] = inv_k * x[r] - acc;
-            if (final && off && r == 0) po[-off] = T(0);
+        for (I it = I(xcd_block_2d().x) * kBlock + threadIdx.x; it < items; it += I(gridDim.x) * kBlock) {
+            // the splits after l = 1 .. t-1 letters, several first letters per thread as in the Chen product kernels
+            chen_fan<T, I, FAN>(x, pin, it, dv, [&](I r, T sum) { po[r] = inv_k * x[r] - sum; });
+            if (final && off && it == 0) po[-off] = T(0);
         }
     }
 }
@@ -239,9 +224,14 @@ static void run_tensor_log(const T* sig, T* out, uint64_t batch, uint64_t dimens
             const uint64_t count = coef_count(dimension, degree - k + 1);
             const T* pin = k == degree ? sig : p_of(k + 1);       // unused when k == degree: only level 1 is computed
             T* pout = k == 1 ? out : p_of(k);
-            launch_indexed(0, count, batch, [&](auto, dim3 grid) {
-                hipLaunchKernelGGL((tensor_log_step_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig, pin, pout, int64_t(batch),
-                                   dv, I(count), T(1) / T(k), int64_t(s.stride), s.off, int64_t(s.stride), int(k == 1));
+            with_chen_fan(dimension, [&](auto fan) {
+                constexpr int FAN = decltype(fan)::value;
+                const uint64_t items = chen_items(dimension, degree - k + 1, FAN);
+                launch_indexed(0, items, batch, [&](auto, dim3 grid) {
+                    hipLaunchKernelGGL((tensor_log_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig, pin, pout,
+                                       int64_t(batch), dv, I(items), T(1) / T(k), int64_t(s.stride), s.off, int64_t(s.stride),
+                                       int(k == 1));
+                });
             });
         }
     });

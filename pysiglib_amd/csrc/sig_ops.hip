@@ -252,11 +252,15 @@ static void sig_combine_impl(const T* sig1, const T* sig2, T* out, uint64_t batc
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((sig_combine_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig1, sig2, out, int64_t(batch),
-                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), int64_t(s.stride), int64_t(s.stride),
-                               s.off, s.off, s.off);
+        with_chen_fan(dimension, [&](auto fan) {
+            constexpr int FAN = decltype(fan)::value;
+            const uint64_t items = chen_items(dimension, degree, FAN);
+            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+                using I = decltype(ix);
+                hipLaunchKernelGGL((sig_combine_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig1, sig2, out, int64_t(batch),
+                                   DivBy<I>(dimension), I(items), int64_t(s.stride), int64_t(s.stride), int64_t(s.stride),
+                                   s.off, s.off, s.off);
+            });
         });
     }
     SIG_HIP(hipGetLastError());

@@ -642,7 +642,7 @@ def test_config_forward_full_size(P, oracle, k):
 
 def test_config3_forward(P, oracle):
     """(64, 4096, 3) degree 12: the oracle checks the first 6 paths; all 64 are checked through
-    size-independent properties (level 1 = total increment, level-2 shuffle identity, batch invariance)."""
+    size-independent properties (level 1 = total increment, level-2 shuffle identity, batch invariance up to rounding)."""
     c = C.CONFIGS[3]
     x = C.make_path(3)
     xt = dev(x)
@@ -654,8 +654,9 @@ def test_config3_forward(P, oracle):
     np.testing.assert_allclose(l1, x[:, -1] - x[:, 0], rtol=1e-12, atol=1e-14)
     l2 = got[:, 3:12].cpu().numpy().reshape(64, 3, 3)
     np.testing.assert_allclose(l2 + l2.transpose(0, 2, 1), l1[:, :, None] * l1[:, None, :], rtol=1e-10, atol=1e-13)
+    # a smaller batch may be cut into time segments (a different order of additions): equal up to rounding
     again = P.sig(xt[40:47].clone(), 12)
-    assert torch.equal(again, got[40:47])
+    assert level_rel_err(again.cpu().numpy(), got[40:47].cpu().numpy(), 3, 12) <= 1e-12
     del got, again
     torch.cuda.empty_cache()
 
