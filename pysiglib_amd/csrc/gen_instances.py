@@ -209,8 +209,8 @@ def main():
                 lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))
             else:
-                lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, nullptr, %d},'
-                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, pol))
+                lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, &bwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
+                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))
         lines.append("};")
         lines.append("extern const EntryList kList_%02d = {kEntries_%02d, %d};" % (fi, fi, len(bucket)))
         lines.append("#endif")

@@ -368,19 +368,47 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
 // The backward sweep can be cut in time as well: the state at the end of segment g is the Chen product of the
 // segment signatures up to g, and the adjoint of that state is the upstream gradient pulled back through the product
 // with the remaining segments.  That costs a segmented forward sweep, two chains of Chen products and one product
-// adjoint, all over (path, segment) rows, so it is only taken when whole-path sweeps leave at least half of the
-// SIMDs idle and the paths are long; the aim is two waves per SIMD.
+// adjoint, all over (path, segment) rows.
 static int g_force_bwd_segments = 0;   // tuning hook (0 = automatic)
 
-static int choose_bwd_segments(int64_t waves, int64_t L, uint64_t sig_bytes_all_paths)
+// g pieces are chosen by the same kind of model as for the forward sweep (fullest SIMD, `pair_rate`, lane_step(g) =
+// seconds per step of a lone wave).  The extra work is larger here: the segmented forward sweep (a third of the
+// backward's arithmetic), 2 ceil(log2 g) + 2 launches of about 10 us each on top of a fixed 30 us, and the
+// traffic of the scans and of the product adjoint over g rows per path, fitted at 4.2 + 0.64 ceil(log2 g) ps per
+// byte of segment signatures (48 paths of 300 steps, d = 12, degree 4, f64: whole 0.225 ms, 2 pieces 0.270,
+// 8: 0.578, 64: 4.65 ms; 8 paths of 4000 steps, d = 6, degree 4, f32: whole 3.42 ms, 32 pieces 0.249 ms).
+template <typename LaneStep>
+static int choose_bwd_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_t sig_bytes_all_paths, LaneStep&& lane_step,
+                               bool f64)
 {
     const int64_t simds = simd_count();
-    if (waves <= 0 || waves * 2 > simds) return 1;
-    int64_t g = 2 * simds / waves;
-    g = std::min<int64_t>(g, 64);
-    g = std::min<int64_t>(g, L / 32);
-    if (sig_bytes_all_paths > 0) g = std::min<int64_t>(g, int64_t((uint64_t(64) << 20) / sig_bytes_all_paths));
-    return int(std::max<int64_t>(g, 1));
+    if (waves <= 0 || sig_bytes_all_paths == 0) return 1;
+    const int occ = std::max(1, waves_per_simd);
+    if (waves > 2 * simds * occ) return 1;
+    const double pair_rate = f64 ? 1.2 : 1.35;
+    auto estimate = [&](int g) {
+        const int64_t fullest = (waves * g + simds - 1) / simds;
+        const int64_t rounds = fullest / occ, rest = fullest % occ;
+        double steps = double(rounds) * occ / (occ > 1 ? pair_rate : 1.0);
+        if (rest) steps += double(rest) / (rest > 1 ? pair_rate : 1.0);
+        double t = double((L + g - 1) / g) * lane_step(g) * steps;
+        if (g > 1) {
+            int lg = 0;
+            while ((1 << lg) < g) ++lg;
+            t *= 1.31;
+            t += 30e-6 + 10e-6 * (2 * lg + 2) + double(g) * double(sig_bytes_all_paths) * (4.2e-12 + 0.64e-12 * lg);
+        }
+        return t;
+    };
+    int best = 1;
+    double best_t = estimate(1);
+    const double whole = best_t;
+    for (int g : {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64}) {
+        if (L / g < 32 || uint64_t(g) * sig_bytes_all_paths > (uint64_t(64) << 20)) break;
+        const double t = estimate(g);
+        if (t < best_t) { best = g; best_t = t; }
+    }
+    return best_t < 0.93 * whole ? best : 1;
 }
 
 // With at most two waves per SIMD the LDS-staged twin (all-VGPR FMAs, HBM latency hidden by a chunk of
@@ -743,8 +771,16 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         const KernelEntry* ef = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch, s.L);
         int nseg = (!ef || degree > uint64_t(kCombMaxLevels)) ? 1
                    : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
-                                              : choose_bwd_segments(total_waves(geom, int64_t(batch)), int64_t(s.L),
-                                                                    batch * n_coef * sizeof(T));
+                                              : choose_bwd_segments(
+                                                    total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
+                                                    batch * n_coef * sizeof(T),
+                                                    [&](int g) {
+                                                        // a backward step issues about 3.2 times the forward's instructions
+                                                        const double c = lane_step_cost(int(s.d_aug), e->N, e->tail, e->k) * 7.7e-9;
+                                                        const bool ring = pick_variant(true, e, total_waves(geom, int64_t(batch)) * g)->staged;
+                                                        return ring ? c : std::max(c, 700e-9);
+                                                    },
+                                                    sizeof(T) == 8);
         if (nseg > 1) {
             const int64_t lseg = (int64_t(s.L) + nseg - 1) / nseg;
             nseg = int((int64_t(s.L) + lseg - 1) / lseg);

@@ -54,6 +54,18 @@ int fwd_waves_per_simd()
     return blocks < 1 ? 1 : blocks;
 }
 
+// resident waves per SIMD of the backward kernel (register-limited; its LDS tiles never limit below that)
+template <typename T, int D, int N, int TAIL, int K, bool ZL>
+int bwd_waves_per_simd()
+{
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, tree_bwd_kernel<T, D, N, TAIL, K, ZL>, kBlock, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return 1;
+    }
+    return blocks < 1 ? 1 : blocks;
+}
+
 template <typename T, int D, int N, int TAIL, int K, bool ZL>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
