@@ -1018,24 +1018,40 @@ inline uint64_t chen_items(uint64_t d, uint64_t top, int fan)
     }
     return (d + fan - 1) / fan * words;
 }
+// work item -> level t, the start `lo` of that level in a scalar-free row, size = d^(t-1), the first letter a0 of the
+// item's group and the index `rest` of the remaining t - 1 letters
+template <typename I>
+struct FanItem {
+    int t;
+    I lo, size, a0, rest;
+};
+template <typename I, int FAN>
+__device__ __forceinline__ FanItem<I> fan_item(I item, I d)
+{
+    const I groups = (d + FAN - 1) / FAN;
+    FanItem<I> it{1, 0, 1, 0, 0};
+    I first = 0;                        // first item of level t
+    while (item >= first + groups * it.size) {
+        first += groups * it.size;
+        it.lo += it.size * d;
+        it.size *= d;
+        ++it.t;
+    }
+    const I local = item - first;
+    const I g = local / it.size;
+    it.rest = local - g * it.size;
+    it.a0 = g * FAN;
+    return it;
+}
+
 template <typename T, typename I, int FAN, typename F>
 __device__ __forceinline__ void chen_fan(const T* __restrict__ a, const T* __restrict__ bb, I item, const DivBy<I>& dv, F&& f)
 {
     constexpr int kChenFan = FAN;
     const I d = I(dv.d);
-    const I groups = (d + kChenFan - 1) / kChenFan;
-    int t = 1;
-    I first = 0, size = 1, lo = 0;      // first item of level t, d^(t-1), start of level t in a scalar-free row
-    while (item >= first + groups * size) {
-        first += groups * size;
-        lo += size * d;
-        size *= d;
-        ++t;
-    }
-    const I local = item - first;
-    const I g = local / size;
-    const I rest = local - g * size;
-    const I a0 = g * kChenFan;
+    const FanItem<I> fi = fan_item<I, FAN>(item, d);
+    const int t = fi.t;
+    const I lo = fi.lo, size = fi.size, a0 = fi.a0, rest = fi.rest;
     T acc[kChenFan];
 #pragma unroll
     for (int i = 0; i < kChenFan; ++i) acc[i] = T(0);

@@ -87,36 +87,43 @@ template <typename T>
 __device__ __forceinline__ T rcp_of(int k) { return k <= kExpMaxDegree ? T(kRcp[k]) : T(1) / T(k); }
 
 // Signature of a straight line: exp(z)_t[w] = z[w_1] ... z[w_t] / t!   (siglib/cpsig/cp_sig_join.h:36-60)
-template <typename T, typename I>
+// A thread writes the words (a, rest) for FAN consecutive first letters a: the product over `rest` is shared
+// (work items as in the Chen product kernels, chen_items).
+template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void linear_sig_kernel(
-    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I sig_len, int64_t stride, int off)
+    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I items, int64_t stride, int off)
 {
     const I d = I(dv.d);
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* z = disp + b * int64_t(d);
         T* o = out + b * stride;
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T v = T(1);
-            I idx = p.w;
-            for (int k = p.t; k >= 1; --k) {        // letters from the right
+        for (I item = I(blockIdx.x) * kBlock + threadIdx.x; item < items; item += I(gridDim.x) * kBlock) {
+            const FanItem<I> fi = fan_item<I, FAN>(item, d);
+            T v = rcp_of<T>(fi.t);
+            I idx = fi.rest;
+            for (int k = fi.t - 1; k >= 1; --k) {        // letters of rest from the right
                 const I q = dv.quot(idx);
                 v *= z[idx - q * d] * rcp_of<T>(k);
                 idx = q;
             }
-            o[off + r] = v;
-            if (off && r == 0) o[0] = T(1);
+#pragma unroll
+            for (int i = 0; i < FAN; ++i)
+                if (fi.a0 + i < d) o[off + fi.lo + (fi.a0 + i) * fi.size + fi.rest] = v * z[fi.a0 + i];
+            if (off && item == 0) o[0] = T(1);
         }
     }
 }
 
-// out = A (x) exp(z) (append) or exp(z) (x) A (prepend), one thread per output coefficient:
+// out = A (x) exp(z) (append) or exp(z) (x) A (prepend):
 //   append : out_t[w] = sum_{k=0..t} A_{t-k}[w_1..w_{t-k}] * z[w_{t-k+1}] ... z[w_t] / k!
 //   prepend: out_t[w] = sum_{k=0..t} z[w_1] ... z[w_k] / k! * A_{t-k}[w_{k+1}..w_t]          (A_0 = 1)
-// (siglib/cpsig/cp_sig_join.h:107-160)
-template <typename T, typename I>
+// (siglib/cpsig/cp_sig_join.h:107-160).  A thread computes the words (a, rest) for FAN consecutive first letters a.
+// append: the products of trailing letters are shared, the prefixes (a, head of rest) differ by d^(t-k-1) per letter;
+// prepend: every term with k >= 1 carries the factor z[a] and otherwise depends on `rest` only, so
+//   out_t[(a, rest)] = A_t[(a, rest)] + z[a] * C(rest),   C = sum_{k=1..t} z[r_1] .. z[r_{k-1}] / k! * A_{t-k}[r_k .. r_{t-1}].
+template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void sig_join_kernel(
-    const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I sig_len,
+    const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I items,
     int64_t stride, int off, int prepend)
 {
     const I d = I(dv.d);
@@ -124,43 +131,76 @@ __global__ __launch_bounds__(kBlock) void sig_join_kernel(
         const T* a = A + b * stride + off;
         const T* z = disp + b * int64_t(d);
         T* o = out + b * stride;
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T acc = a[p.lo + p.w];
-            T ek = T(1);
-            I lo = p.lo, size = p.size;       // level t-k of A
+        for (I item = I(blockIdx.x) * kBlock + threadIdx.x; item < items; item += I(gridDim.x) * kBlock) {
+            const FanItem<I> fi = fan_item<I, FAN>(item, d);
+            const int t = fi.t;
+            T acc[FAN];
             if (!prepend) {
-                I idx = p.w;
-                for (int k = 1; k <= p.t; ++k) {
-                    const I q = dv.quot(idx);
-                    ek *= z[idx - q * d] * rcp_of<T>(k);
-                    idx = q;
-                    size = dv.quot(size);
-                    lo -= size;
-                    acc = fmadd(k < p.t ? a[lo + idx] : T(1), ek, acc);
+#pragma unroll
+                for (int i = 0; i < FAN; ++i) acc[i] = T(0);
+                T ek = T(1);                       // z[w_{t-k+1}] .. z[w_t] / k!
+                I head = fi.rest;                  // first t-1-k letters of rest
+                I lev = fi.size * d, lo = fi.lo;   // size and start of level t-k+1 of A
+                for (int k = 1; k <= t - 1; ++k) {
+                    const I q = dv.quot(head);
+                    ek *= z[head - q * d] * rcp_of<T>(k);
+                    head = q;
+                    lev = dv.quot(lev);            // d^(t-k)
+                    lo -= lev;
+                    const I st = dv.quot(lev);     // d^(t-k-1): distance between the prefixes of consecutive first letters
+                    const T* ap = a + lo + head;
+#pragma unroll
+                    for (int i = 0; i < FAN; ++i) {
+                        const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
+                        acc[i] = fmadd(ap[letter * st], ek, acc[i]);
+                    }
+                }
+                // k = t: the empty prefix (A_0 = 1) and the whole word's product
+                const T et = ek * rcp_of<T>(t);
+#pragma unroll
+                for (int i = 0; i < FAN; ++i) {
+                    const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
+                    acc[i] = fmadd(et, z[letter], acc[i]);
                 }
             } else {
-                // letters from the left: reverse the word once (the letters come out of the divisions right to left)
-                I idx = p.w, rev = 0;
-                for (int k = 0; k < p.t; ++k) {
+                // letters of rest from the left: reverse it once (the divisions deliver letters right to left)
+                I idx = fi.rest, rev = 0;
+                for (int k = 0; k < t - 1; ++k) {
                     const I q = dv.quot(idx);
                     rev = rev * d + (idx - q * d);
                     idx = q;
                 }
-                I rem = p.w;
-                for (int k = 1; k <= p.t; ++k) {
-                    const I q = dv.quot(rev);
-                    const I letter = rev - q * d;      // w_k
-                    rev = q;
-                    size = dv.quot(size);              // d^(t-k)
-                    ek *= z[letter] * rcp_of<T>(k);
-                    rem -= letter * size;              // w_{k+1} .. w_t
-                    lo -= size;
-                    acc = fmadd(k < p.t ? a[lo + rem] : T(1), ek, acc);
+                // C = sum_{k=1..t} P_{k-1} / k! * A_{t-k}[suffix], P_j = z[r_1] .. z[r_j]
+                T c = T(0);
+                T pk = T(1);                       // P_{k-1} / k!
+                I rem = fi.rest, size = fi.size, lo = fi.lo;      // suffix r_k .. r_{t-1}, d^(t-k), start of level t-k+1
+                for (int k = 1; k <= t; ++k) {
+                    pk *= rcp_of<T>(k);
+                    lo -= size;                    // start of level t-k
+                    c = fmadd(k < t ? a[lo + rem] : T(1), pk, c);
+                    if (k < t) {
+                        const I q = dv.quot(rev);
+                        const I letter = rev - q * d;          // r_k
+                        rev = q;
+                        size = dv.quot(size);                  // d^(t-k-1)
+                        pk *= z[letter];
+                        rem -= letter * size;
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < FAN; ++i) {
+                    const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
+                    acc[i] = z[letter] * c;
                 }
             }
-            o[off + r] = acc;
-            if (off && r == 0) o[0] = T(1);
+#pragma unroll
+            for (int i = 0; i < FAN; ++i) {
+                if (fi.a0 + i < d) {
+                    const I r = fi.lo + (fi.a0 + i) * fi.size + fi.rest;
+                    o[off + r] = a[r] + acc[i];
+                }
+            }
+            if (off && item == 0) o[0] = T(1);
         }
     }
 }
@@ -302,10 +342,14 @@ static void linear_sig_impl(const T* disp, T* out, uint64_t batch, uint64_t dime
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((linear_sig_kernel<T, I>), grid, dim3(kBlock), 0, stream, disp, out, int64_t(batch),
-                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off);
+        with_chen_fan(dimension, [&](auto fan) {
+            constexpr int FAN = decltype(fan)::value;
+            const uint64_t items = chen_items(dimension, degree, FAN);
+            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+                using I = decltype(ix);
+                hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, out, int64_t(batch),
+                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+            });
         });
     }
     SIG_HIP(hipGetLastError());
@@ -326,10 +370,14 @@ static void sig_join_impl(const T* sig, const T* disp, T* out, uint64_t batch, u
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((sig_join_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig, disp, out, int64_t(batch),
-                               DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off, int(prepend));
+        with_chen_fan(dimension, [&](auto fan) {
+            constexpr int FAN = decltype(fan)::value;
+            const uint64_t items = chen_items(dimension, degree, FAN);
+            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+                using I = decltype(ix);
+                hipLaunchKernelGGL((sig_join_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig, disp, out, int64_t(batch),
+                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, int(prepend));
+            });
         });
     }
     SIG_HIP(hipGetLastError());
@@ -357,10 +405,14 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     T* E = static_cast<T*>(workspace(4, bytes));
     T* dE = static_cast<T*>(workspace(5, bytes));
-    launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-        using I = decltype(ix);
-        hipLaunchKernelGGL((linear_sig_kernel<T, I>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
-                           DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off);
+    with_chen_fan(dimension, [&](auto fan) {
+        constexpr int FAN = decltype(fan)::value;
+        const uint64_t items = chen_items(dimension, degree, FAN);
+        launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
+                               DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+        });
     });
     // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
     if (prepend) launch_combine_bwd<T>(d_out, dE, d_sig, (const T*)E, sig, batch, dimension, degree, s, stream);
