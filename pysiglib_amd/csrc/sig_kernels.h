@@ -136,6 +136,16 @@ __device__ __forceinline__ void loads_issued()
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// All LDS operations of this wave have completed (vector-memory counters untouched).  Placed before the ring reads
+// of the next step it replaces the compiler's waits before every first use of the current step's values (read a
+// whole step ago): a wait that does not stall still takes one of a lone wave's issue slots.
+__device__ __forceinline__ void wait_lds()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);     // lgkmcnt(0), vmcnt and expcnt at their maxima
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // all outstanding vector- and scalar-memory loads have landed
 __device__ __forceinline__ void wait_all_loads()
 {
@@ -334,9 +344,12 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
         const int nk = int((count - done < CS) ? count - done : CS);
         int i = 0;
         for (; i + 2 <= nk; i += 2) {
+            // forward only: the backward's steps end with LDS adds into the reduction tile, which such a wait would sit out
+            if constexpr (DIR > 0) wait_lds();
             load_row(zb, lp + DIR * D);
             loads_issued();
             step(za, first + DIR * (done + i), IntC<G0>{});
+            if constexpr (DIR > 0) wait_lds();
             load_row(za, lp + 2 * DIR * D);                      // may be row 0 of the next chunk (contiguous or wrap copy)
             loads_issued();
             step(zb, first + DIR * (done + i + 1), IntC<G0>{});
