@@ -638,6 +638,9 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const int64_t wave_base = lane_base;
     int cs = 0;                     // steps already written into the current chunk
     int64_t t_chunk = count - 1;    // local step held by chunk slot 0
+    // The tile is flushed when `limit` steps sit in it.  The first chunk takes the remainder of count / CH, so that
+    // all later chunks are full and the last flush falls on the last step: the test is one 32-bit compare per step.
+    int limit = tiled ? (count % CH == 0 ? CH : int(count % CH)) : 0;
 
     auto reduce_chunk = [&](int n_slots) {
         wave_lds_sync();
@@ -731,10 +734,11 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 for (int l = 0; l < M; ++l) lds_add(&col[cx.p[l] * kRedStride], dz.dc[l]);
             }
             ++cs;
-            if (cs == CH || t == 0) {
+            if (cs == limit) {
                 reduce_chunk(cs);
+                t_chunk -= cs;
                 cs = 0;
-                t_chunk = t - 1;
+                limit = CH;
             }
         } else {
             T* grow_t = dzinc + lane_base + t * d;
