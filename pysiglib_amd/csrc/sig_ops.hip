@@ -206,12 +206,17 @@ __global__ __launch_bounds__(kBlock) void sig_join_kernel(
 }
 
 // Adjoint of z -> exp(z): dz[j] = sum_t 1/t! sum_{w in d^t} dE_t[w] sum_{i : w_i = j} prod_{m != i} z[w_m]
-// (closed form of the level recursion in siglib/cpsig/cp_sig_combine.h:232-263).  One thread per coefficient,
-// per-block partial sums in LDS (or straight to HBM for very wide paths), dz zeroed beforehand.
+// (closed form of the level recursion in siglib/cpsig/cp_sig_combine.h:232-263).  A thread takes the words (a, rest)
+// for FAN consecutive first letters a (work items as in the Chen product kernels): the first position gives
+// dz[a] += dE[(a, rest)] * prod(rest) / t!, and for a letter r_i of `rest` the terms of all a collapse into
+// dz[r_i] += (sum_a z[a] dE[(a, rest)]) * prod_{m != i} z[r_m] / t!  - FAN + t - 1 additions instead of FAN * t.
+// The letters and suffix products of `rest` sit in arrays of TMAX entries that every loop walks with compile-time
+// bounds, so that they stay in registers (TMAX >= degree - 1; 64: rolled loops, arrays in scratch memory).
+// Per-block partial sums in LDS (or straight to HBM for very wide paths), dz zeroed beforehand.
 constexpr int kExpAccMax = 4096;
-template <typename T, typename I>
+template <typename T, typename I, int FAN, int TMAX>
 __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
-    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int64_t batch, DivBy<I> dv, I sig_len,
+    const T* __restrict__ dE, const T* __restrict__ disp, T* __restrict__ dz, int64_t batch, DivBy<I> dv, I items,
     int64_t stride, int off, int use_lds, int copies)
 {
     extern __shared__ double exp_lds_raw[];
@@ -228,26 +233,62 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
         const T* z = disp + b * int64_t(d);
         const T* g = dE + b * stride + off;
         T* out = dz + b * int64_t(d);
-        for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-            const WordPos<I> p = word_pos<I>(r, d);
-            T suf[kExpMaxDegree];       // suf[i] = dE[w] / t! * z[w_{i+2}] ... z[w_t]   (0-based position i)
-            I let[kExpMaxDegree];
-            I idx = p.w;
-            T run = g[r];
-            for (int k = 1; k <= p.t; ++k) run *= rcp_of<T>(k);
-            for (int i = p.t - 1; i >= 0; --i) {
-                const I q = dv.quot(idx);
-                let[i] = idx - q * d;
-                idx = q;
-                suf[i] = run;
-                run *= z[let[i]];
+        auto add = [&](I letter, T v) {
+            if (use_lds) lds_add_shared(&mine[letter], v);
+            else dev_add(&out[letter], v);
+        };
+        for (I item = I(xcd_block_2d().x) * kBlock + threadIdx.x; item < items; item += I(gridDim.x) * kBlock) {
+            const FanItem<I> fi = fan_item<I, FAN>(item, d);
+            const int n = fi.t - 1;         // letters of rest
+            T suf[TMAX];                    // suf[i] = z[r_{i+1}] .. z[r_{n-1}] / t!   (0-based position i in rest)
+            I let[TMAX];
+            T run = T(1);
+            for (int k = 1; k <= fi.t; ++k) run *= rcp_of<T>(k);
+            I idx = fi.rest;
+            if constexpr (TMAX < 64) {
+#pragma unroll
+                for (int i = TMAX - 1; i >= 0; --i) {
+                    if (i < n) {
+                        const I q = dv.quot(idx);
+                        let[i] = idx - q * d;
+                        idx = q;
+                        suf[i] = run;
+                        run *= z[let[i]];
+                    }
+                }
+            } else {
+                for (int i = n - 1; i >= 0; --i) {
+                    const I q = dv.quot(idx);
+                    let[i] = idx - q * d;
+                    idx = q;
+                    suf[i] = run;
+                    run *= z[let[i]];
+                }
             }
-            T pre = T(1);
-            for (int i = 0; i < p.t; ++i) {
-                const T c = pre * suf[i];
-                if (use_lds) lds_add_shared(&mine[let[i]], c);
-                else dev_add(&out[let[i]], c);
-                pre *= z[let[i]];
+            // run = prod(rest) / t!
+            T wsum = T(0);
+#pragma unroll
+            for (int i = 0; i < FAN; ++i) {
+                if (fi.a0 + i < d) {
+                    const T e = g[fi.lo + (fi.a0 + i) * fi.size + fi.rest];
+                    add(fi.a0 + i, e * run);
+                    wsum = fmadd(z[fi.a0 + i], e, wsum);
+                }
+            }
+            T pre = wsum;                   // wsum * z[r_0] .. z[r_{i-1}]
+            if constexpr (TMAX < 64) {
+#pragma unroll
+                for (int i = 0; i < TMAX; ++i) {
+                    if (i < n) {
+                        add(let[i], pre * suf[i]);
+                        pre *= z[let[i]];
+                    }
+                }
+            } else {
+                for (int i = 0; i < n; ++i) {
+                    add(let[i], pre * suf[i]);
+                    pre *= z[let[i]];
+                }
             }
         }
         if (use_lds) {
@@ -423,13 +464,24 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     } else {
         const int use_lds = dimension <= uint64_t(kExpAccMax);
         const int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(32, uint64_t(kExpAccMax) / dimension))) : 1;
-        // about 8 coefficients per thread, so that a block's LDS partial sums amortise their flush
-        launch_indexed(s.n_coef, (s.n_coef + 7) / 8, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((exp_pullback_kernel<T, I>), grid, dim3(kBlock),
-                               use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp,
-                               d_disp, int64_t(batch), DivBy<I>(dimension), I(s.n_coef), int64_t(s.stride), s.off, use_lds,
-                               copies);
+        with_chen_fan(dimension, [&](auto fan) {
+            constexpr int FAN = decltype(fan)::value;
+            const uint64_t items = chen_items(dimension, degree, FAN);
+            // a few items per thread, so that a block's LDS partial sums amortise their flush
+            launch_indexed(s.n_coef, (items + 3) / 4, batch, [&](auto ix, dim3 grid) {
+                using I = decltype(ix);
+                auto go = [&](auto tmax) {
+                    constexpr int TMAX = decltype(tmax)::value;
+                    hipLaunchKernelGGL((exp_pullback_kernel<T, I, FAN, TMAX>), grid, dim3(kBlock),
+                                       use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp,
+                                       d_disp, int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, use_lds,
+                                       copies);
+                };
+                if (degree <= 5) go(IntC<4>{});
+                else if (degree <= 9) go(IntC<8>{});
+                else if (degree <= 17) go(IntC<16>{});
+                else go(IntC<64>{});
+            });
         });
     }
     SIG_HIP(hipGetLastError());
