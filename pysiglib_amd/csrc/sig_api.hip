@@ -495,9 +495,13 @@ static void compute_increments(const T* path, T* inc, uint64_t batch, uint64_t d
                                T* zero_out = nullptr, uint64_t zero_count = 0)
 {
     const T time_step = s.len_aug > 1 ? end_time / T(s.len_aug - 1) : T(0);
-    hipLaunchKernelGGL((increments_kernel<T>), dim3(grid_for(batch * (s.L + 2) * s.d_aug)), dim3(kBlock), 0, stream,
-                       path, inc, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
-                       int(lead_lag), time_step, zero_out, int64_t(zero_count));
+    (void)zero_count;       // always the whole increment gradient of the batch: batch * L * d elements
+    const uint64_t per = (s.L + 2) * s.d_aug;
+    launch_indexed(per, (per + 1) / 2, batch, [&](auto ix, dim3 grid) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((increments_kernel<T, I>), grid, dim3(kBlock), 0, stream, path, inc, int64_t(batch), int64_t(length),
+                           int(dimension), int(time_aug), int(lead_lag), time_step, zero_out, DivBy<I>(s.d_aug));
+    });
     SIG_HIP(hipGetLastError());
 }
 

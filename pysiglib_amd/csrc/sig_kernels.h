@@ -21,51 +21,6 @@ __device__ __forceinline__ void static_for(F&& f)
 }
 
 // ---------------------------------------------------------------------------
-// Increment pre-pass: z[b][t][c] of the (virtually) augmented path.
-// lead-lag: even step moves the lead half, odd step the lag half; time is the
-// last channel with constant spacing end_time / (len_eff - 1)
-// (siglib/cpsig/cp_path.h:46-62,262-279; siglib/cusig/cu_signature.cu:146-166).
-// ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(kBlock) void increments_kernel(
-    const T* __restrict__ path, T* __restrict__ inc, int64_t batch, int64_t len_raw, int d_raw,
-    int time_aug, int lead_lag, T time_step, T* __restrict__ zero_out, int64_t zero_count)
-{
-    // zero_out (optional, zero_count <= number of increment elements): cleared in the same launch; the backward
-    // accumulates its increment gradient there with atomics.
-    // Layout [batch][L + 2][d]: row t + 1 holds the increment of step t; rows 0 and L + 1 are zero so
-    // that the sweeps may prefetch one row past either end of a path without a bounds test.
-    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
-    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
-    const int64_t rows = L + 2;
-    const int64_t total = batch * rows * d;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int c = int(e % d);
-        const int64_t row = (e / d) % rows;
-        const int64_t b = e / (int64_t(d) * rows);
-        const T* x = path + b * len_raw * d_raw;
-        T v;
-        if (row == 0 || row == rows - 1) {
-            v = T(0);
-        } else {
-            const int64_t t = row - 1;
-            if (time_aug && c == d - 1) {
-                v = T(t + 1) * time_step - T(t) * time_step;
-            } else if (!lead_lag) {
-                v = x[(t + 1) * d_raw + c] - x[t * d_raw + c];
-            } else {
-                const int64_t k = t >> 1;
-                const bool odd = t & 1;
-                if (c < d_raw) v = odd ? x[(k + 1) * d_raw + c] - x[k * d_raw + c] : T(0);
-                else v = odd ? T(0) : x[(k + 1) * d_raw + (c - d_raw)] - x[k * d_raw + (c - d_raw)];
-            }
-        }
-        inc[e] = v;
-        if (e < zero_count) zero_out[e] = T(0);
-    }
-}
-
-// ---------------------------------------------------------------------------
 // Lane set-up shared by both sweeps.
 // ---------------------------------------------------------------------------
 template <typename T, int D, int N, int TAIL, int K>
@@ -964,6 +919,55 @@ void launch_indexed(uint64_t max_index, uint64_t per_item, uint64_t batch, F&& f
     const dim3 grid{unsigned(gx), unsigned(gy), 1};
     if (max_index < (uint64_t(1) << 31) && !g_force_wide_index) f(uint32_t{}, grid);
     else f(uint64_t{}, grid);
+}
+
+// ---------------------------------------------------------------------------
+// Increment pre-pass: z[b][t][c] of the (virtually) augmented path.
+// lead-lag: even step moves the lead half, odd step the lag half; time is the
+// last channel with constant spacing end_time / (len_eff - 1)
+// (siglib/cpsig/cp_path.h:46-62,262-279; siglib/cusig/cu_signature.cu:146-166).
+// Grid: x over the (L + 2) * d elements of one path, y over the paths; the only division is by d.
+// ---------------------------------------------------------------------------
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void increments_kernel(
+    const T* __restrict__ path, T* __restrict__ inc, int64_t batch, int64_t len_raw, int d_raw,
+    int time_aug, int lead_lag, T time_step, T* __restrict__ zero_out, DivBy<I> dv)
+{
+    // zero_out (optional): the increment gradient [batch][L][d], cleared in the same launch; the backward
+    // accumulates into it with atomics.
+    // Layout [batch][L + 2][d]: row t + 1 holds the increment of step t; rows 0 and L + 1 are zero so
+    // that the sweeps may prefetch one row past either end of a path without a bounds test.
+    const I d = I(dv.d);
+    const I L = I((lead_lag ? 2 * len_raw - 1 : len_raw) - 1);
+    const I rows = L + 2;
+    const I per = rows * d;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* x = path + b * len_raw * d_raw;
+        T* o = inc + b * int64_t(per);
+        T* zo = zero_out ? zero_out + b * int64_t(L) * int64_t(d) : nullptr;
+        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
+            const I row = dv.quot(e);
+            const I c = e - row * d;
+            T v;
+            if (row == 0 || row == rows - 1) {
+                v = T(0);
+            } else {
+                const I t = row - 1;
+                if (time_aug && c == d - 1) {
+                    v = T(t + 1) * time_step - T(t) * time_step;
+                } else if (!lead_lag) {
+                    v = x[int64_t(t + 1) * d_raw + c] - x[int64_t(t) * d_raw + c];
+                } else {
+                    const I k = t >> 1;
+                    const bool odd = t & 1;
+                    if (c < I(d_raw)) v = odd ? x[int64_t(k + 1) * d_raw + c] - x[int64_t(k) * d_raw + c] : T(0);
+                    else v = odd ? T(0) : x[int64_t(k + 1) * d_raw + (c - d_raw)] - x[int64_t(k) * d_raw + (c - d_raw)];
+                }
+            }
+            o[e] = v;
+            if (zo && e < L * d) zo[e] = T(0);
+        }
+    }
 }
 
 // level t (1-based) of coefficient r of a scalar-free signature row, its index w inside the level, the start
