@@ -749,8 +749,11 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                                int64_t(s.stride), sc, time_tiles, col_groups);
         }
         timer.stop();
-        hipLaunchKernelGGL((path_grad_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, dzinc, out,
-                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+        launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, (const T*)dzinc, out, int64_t(batch),
+                               int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
+        });
         SIG_HIP(hipGetLastError());
         exit_sync(stream);      // the workspaces stay locked until the kernels are done
         return;
@@ -845,8 +848,11 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         MainKernelTimer timer(stream, e->name);
         SIG_HIP(e->bwd(p));
         timer.stop();
-        hipLaunchKernelGGL((path_grad_kernel<T>), dim3(grid_for(out_elems)), dim3(kBlock), 0, stream, dzinc, out,
-                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag));
+        launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, (const T*)dzinc, out, int64_t(batch),
+                               int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
+        });
         SIG_HIP(hipGetLastError());
         exit_sync(stream);
         return;

@@ -755,38 +755,6 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Increment gradient -> raw path gradient.  Point i of the raw path receives
-// +dz of every step that ends in it and -dz of every step that starts from it;
-// with lead-lag, step 2k moves the lead half and step 2k+1 the lag half of
-// raw segment k -> k+1; the time channel has no raw counterpart
-// (siglib/cpsig/cp_signature.h:1189-1201, siglib/cusig/cu_path_transforms.cu:129-147).
-// ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(kBlock) void path_grad_kernel(
-    const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, int d_raw,
-    int time_aug, int lead_lag)
-{
-    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
-    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
-    const int64_t total = batch * len_raw * d_raw;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < total; e += int64_t(gridDim.x) * kBlock) {
-        const int c = int(e % d_raw);
-        const int64_t i = (e / d_raw) % len_raw;
-        const int64_t b = e / (int64_t(d_raw) * len_raw);
-        const T* g = dzinc + b * L * d;
-        T v = T(0);
-        if (!lead_lag) {
-            if (i > 0) v += g[(i - 1) * d + c];
-            if (i < len_raw - 1) v -= g[i * d + c];
-        } else {
-            if (i > 0) v += g[(2 * (i - 1)) * d + d_raw + c] + g[(2 * (i - 1) + 1) * d + c];
-            if (i < len_raw - 1) v -= g[(2 * i) * d + d_raw + c] + g[(2 * i + 1) * d + c];
-        }
-        out[e] = v;
-    }
-}
-
-// ---------------------------------------------------------------------------
 // Closed forms (siglib/cpsig/cp_signature.h:748-784,845-851; backward :941-945).
 // ---------------------------------------------------------------------------
 template <typename T>
@@ -966,6 +934,42 @@ __global__ __launch_bounds__(kBlock) void increments_kernel(
             }
             o[e] = v;
             if (zo && e < L * d) zo[e] = T(0);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Increment gradient -> raw path gradient.  Point i of the raw path receives
+// +dz of every step that ends in it and -dz of every step that starts from it;
+// with lead-lag, step 2k moves the lead half and step 2k+1 the lag half of
+// raw segment k -> k+1; the time channel has no raw counterpart
+// (siglib/cpsig/cp_signature.h:1189-1201, siglib/cusig/cu_path_transforms.cu:129-147).
+// ---------------------------------------------------------------------------
+// Grid: x over the len_raw * d_raw elements of one path's gradient, y over the paths; the only division is by d_raw.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void path_grad_kernel(
+    const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, int time_aug, int lead_lag,
+    DivBy<I> dv)
+{
+    const I d_raw = I(dv.d);
+    const I d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    const I per = I(len_raw) * d_raw;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* g = dzinc + b * L * int64_t(d);
+        T* o = out + b * int64_t(per);
+        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
+            const int64_t i = int64_t(dv.quot(e));
+            const int64_t c = int64_t(e) - i * int64_t(d_raw);
+            T v = T(0);
+            if (!lead_lag) {
+                if (i > 0) v += g[(i - 1) * d + c];
+                if (i < len_raw - 1) v -= g[i * d + c];
+            } else {
+                if (i > 0) v += g[(2 * (i - 1)) * d + d_raw + c] + g[(2 * (i - 1) + 1) * d + c];
+                if (i < len_raw - 1) v -= g[(2 * i) * d + d_raw + c] + g[(2 * i + 1) * d + c];
+            }
+            o[e] = v;
         }
     }
 }
