@@ -22,6 +22,11 @@ namespace sigamd {
 // which is what the tensor logarithm is built from.
 // The rows of dC may be laid out differently from the others (stride dc_stride, dc_off leading slots) and shared:
 // item b reads row b / dc_share.  families = 1 computes dA only (dB and A are not touched).
+// four consecutive elements with the alignment of one
+template <typename T>
+struct alignas(sizeof(T)) Quad {
+    T v[4];
+};
 constexpr int kCombChunk = 256;
 constexpr int kCombMaxLevels = 64;
 template <typename I>
@@ -105,13 +110,15 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
                 if (!fam_b) {
                     const T* blockp = up + w * (plan.lo[m + 1] - plan.lo[m]) - plan.lo[m];    // words w v
                     I x = seg0;
-                    for (; x + 4 <= seg1; x += 4) {      // all eight loads are issued before the first product needs one
-                        const T g0 = blockp[x], g1 = blockp[x + 1], g2 = blockp[x + 2], g3 = blockp[x + 3];
-                        const T o0 = other[x], o1 = other[x + 1], o2 = other[x + 2], o3 = other[x + 3];
-                        s0 = fmadd(g0, o0, s0);
-                        s1 = fmadd(g1, o1, s1);
-                        s2 = fmadd(g2, o2, s2);
-                        s3 = fmadd(g3, o3, s3);
+                    for (; x + 4 <= seg1; x += 4) {      // all loads are issued before the first product needs one
+                        // a lane walks a block of its own, so every load costs it a cache access of its own: take the
+                        // four consecutive entries in wide loads (element alignment is all that is known)
+                        const Quad<T> gq = *reinterpret_cast<const Quad<T>*>(blockp + x);
+                        const Quad<T> oq = *reinterpret_cast<const Quad<T>*>(other + x);
+                        s0 = fmadd(gq.v[0], oq.v[0], s0);
+                        s1 = fmadd(gq.v[1], oq.v[1], s1);
+                        s2 = fmadd(gq.v[2], oq.v[2], s2);
+                        s3 = fmadd(gq.v[3], oq.v[3], s3);
                     }
                     for (; x < seg1; ++x) s0 = fmadd(blockp[x], other[x], s0);
                 } else {
