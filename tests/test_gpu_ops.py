@@ -50,7 +50,7 @@ def test_combine_kats(P):
 
 
 @pytest.mark.parametrize("d,deg,batch", [(2, 5, 7), (5, 4, 33), (3, 1, 4), (1, 6, 3), (7, 3, 130), (10, 5, 32),
-                                         (37, 2, 5), (2, 14, 2)])
+                                         (37, 2, 5), (2, 14, 2), (4, 4, 9), (6, 3, 5), (11, 3, 3), (13, 3, 5), (9, 4, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
 def test_combine_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
@@ -140,7 +140,7 @@ def test_combine_backprop_golden(P, fixtures, deg, dtype):
 
 
 @pytest.mark.parametrize("d,deg,batch", [(2, 5, 7), (5, 4, 33), (3, 1, 4), (1, 6, 3), (7, 3, 130), (10, 5, 32),
-                                         (37, 2, 5), (2, 14, 2)])
+                                         (37, 2, 5), (2, 14, 2), (4, 4, 9), (6, 3, 5), (11, 3, 3), (13, 3, 5), (9, 4, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
 def test_combine_backprop_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
@@ -265,7 +265,7 @@ def test_linear_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
 
 
 @pytest.mark.parametrize("d,deg,batch", [(2, 5, 5), (3, 4, 70), (5, 2, 4), (1, 5, 3), (4, 1, 2), (10, 5, 32), (40, 2, 3),
-                                         (2, 14, 2)])
+                                         (2, 14, 2), (3, 7, 4), (2, 19, 1), (7, 3, 9), (13, 3, 5)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("prepend", [False, True])
 @pytest.mark.parametrize("scalar_term", [False, True])
@@ -539,7 +539,7 @@ def test_log_sig_backprop_golden(P, fixtures, deg, dtype):
 
 
 @pytest.mark.parametrize("d,deg,batch", [(2, 6, 5), (3, 4, 70), (5, 3, 4), (1, 5, 3), (4, 1, 2), (3, 0, 3), (10, 5, 32),
-                                         (40, 2, 3), (2, 12, 2)])
+                                         (40, 2, 3), (2, 12, 2), (6, 4, 3), (13, 3, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
 def test_sig_to_log_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
