@@ -127,11 +127,11 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
                     for (; x + 4 <= seg1; x += 4) {
                         const T* sp = strided + (x - plan.lo[m]) * sz_t;
                         const T g0 = sp[0], g1 = sp[sz_t], g2 = sp[2 * sz_t], g3 = sp[3 * sz_t];
-                        const T o0 = other[x], o1 = other[x + 1], o2 = other[x + 2], o3 = other[x + 3];
-                        s0 = fmadd(g0, o0, s0);
-                        s1 = fmadd(g1, o1, s1);
-                        s2 = fmadd(g2, o2, s2);
-                        s3 = fmadd(g3, o3, s3);
+                        const Quad<T> oq = *reinterpret_cast<const Quad<T>*>(other + x);      // the same four for the whole wave
+                        s0 = fmadd(g0, oq.v[0], s0);
+                        s1 = fmadd(g1, oq.v[1], s1);
+                        s2 = fmadd(g2, oq.v[2], s2);
+                        s3 = fmadd(g3, oq.v[3], s3);
                     }
                     for (; x < seg1; ++x) s0 = fmadd(strided[(x - plan.lo[m]) * sz_t], other[x], s0);
                 }
