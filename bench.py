@@ -38,7 +38,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all-configs", action="store_true", help="also time configs 2-4 (reported under 'configs')")
+    ap.add_argument("--all-configs", action="store_true", help="(default) also time configs 2-4, reported under 'configs'")
+    ap.add_argument("--headline-only", action="store_true", help="time only the headline workload (configs 1 and 5)")
     ap.add_argument("--ops", action="store_true",
                     help="time the operators either side of the sweep (sig_combine, sig_join, linear_sig, transform_path "
                          "and backward passes) on HBM-bound shapes and print their own JSON line instead")
@@ -287,7 +288,7 @@ def main():
         "C5": {"signatures_per_s": r5.c["batch"] / wall_b, "call_ms": wall_b * 1e3, "kernel": name_b,
                "kernel_ms": kms_b, "tflops": tf_b, "roofline_frac": tf_b / peak},
     }
-    if args.all_configs:
+    if not args.headline_only:      # all five workloads by default (a few seconds more)
         for k in (2, 3, 4):
             r = Runner(k, torch, np, loader, cfgmod)
             n = 3 if k == 3 else max(5, min(args.steps, 50))
