@@ -120,18 +120,22 @@ def cpu_baseline(np, cfgmod):
     rng = np.random.default_rng(2005)
     best = None
     sig = None
-    for _ in range(2):
+    g = None
+    reps = 20       # about 0.3-0.5 s each: 6-10 s of CPU work
+    for _ in range(reps):
         t0 = time.perf_counter()
         sig = sigref.signature(x, c["degree"], n_jobs=threads)
-        g = rng.standard_normal(sig.shape)
         t1 = time.perf_counter()
-        sigref.sig_backprop(x, sig, g, c["degree"], n_jobs=threads)
+        if g is None:
+            g = rng.standard_normal(sig.shape)
         t2 = time.perf_counter()
-        dt = (t1 - t0) + (t2 - t1)
+        sigref.sig_backprop(x, sig, g, c["degree"], n_jobs=threads)
+        t3 = time.perf_counter()
+        dt = (t1 - t0) + (t3 - t2)
         best = dt if best is None else min(best, dt)
     return {"value": c["batch"] / best, "unit": "signatures/s (fwd+bwd)", "cores": threads, "kind": "port",
-            "sample": "full headline workload (32 paths x 999 steps, d=10, degree 5, f64), best of 2, "
-                      "oracle/sigref.c -O3 -march=native, one path per thread"}
+            "sample": "full headline workload (32 paths x 999 steps, d=10, degree 5, f64), best of %d, "
+                      "oracle/sigref.c -O3 -march=native, one path per thread" % reps}
 
 
 def bench_ops(args, torch, loader):
