@@ -121,7 +121,7 @@ def cpu_baseline(np, cfgmod):
     best = None
     sig = None
     g = None
-    reps = 20       # about 0.3-0.5 s each: 6-10 s of CPU work
+    reps = 60       # about 0.13 s each on 16 host threads: ~8 s of CPU work
     for _ in range(reps):
         t0 = time.perf_counter()
         sig = sigref.signature(x, c["degree"], n_jobs=threads)
