@@ -110,6 +110,14 @@ def fwd_cost(D, N, tail, K):
     return cost
 
 
+def lead_lag_mode(D, staged):
+    """Lead-lag twin of a staged forward instance: 1 (time channel last, D odd), 2 (no time channel, D even), 0 none.
+    At least two raw channels, and narrow enough for the skipped half to matter less than the compile time."""
+    if not staged or D < 4 or D > 40:
+        return 0
+    return 1 if D % 2 else 2
+
+
 def choose(D, N, dtype, direction):
     key = (dtype, D, N, direction)
     if key in OVERRIDES:
@@ -193,6 +201,9 @@ def main():
             if direction == "fwd":
                 lines.append("template __global__ void tree_fwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, %s*, int64_t, "
                              "int64_t, int, int64_t, int, int, int64_t, int*, int);" % (T, D, N, tail, K, zs, T, T))
+                if lead_lag_mode(D, zl):
+                    lines.append("template __global__ void tree_fwd_kernel<%s, %d, %d, %d, %d, true, %d>(const %s*, %s*, int64_t, "
+                                 "int64_t, int, int64_t, int, int, int64_t, int*, int);" % (T, D, N, tail, K, lead_lag_mode(D, zl), T, T))
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
                              "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))
@@ -206,8 +217,10 @@ def main():
             name = "%s_%s_d%s_n%d_t%d_k%d%s" % (direction, "f64" if is64 else "f32", "0w" if D < 0 else str(D), N, tail, K,
                                                 "_lds" if zl else "")
             if direction == "fwd":
-                lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
-                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))
+                ll = lead_lag_mode(D, zl)
+                ll_fn = ("&launch_tree_fwd<%s, %d, %d, %d, %d, true, %d>" % (T, D, N, tail, K, ll)) if ll else "nullptr"
+                lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d, %s},'
+                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol, ll_fn))
             else:
                 lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, &bwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))

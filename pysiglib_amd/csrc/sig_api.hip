@@ -306,6 +306,7 @@ static int* nonfinite_flag()
 static int g_force_segments = 0;   // tuning hook (0 = automatic)
 static thread_local int tl_last_segments = 0;   // pieces per path of the last forward sweep on this thread (0: no sweep ran)
 static int g_point_fed = 1;        // tuning hook: 0 always computes the increments in a kernel of their own
+static int g_lead_lag_sparse = 1;  // tuning hook: 0 sweeps lead-lag paths like any other (every letter of every step)
 
 static int simd_count()
 {
@@ -617,6 +618,10 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         FwdParams p;
         p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
         p.lseg = (int64_t(s.L) + nseg - 1) / nseg;
+        // lead-lag sweeps that skip the letters a step cannot move take the step's parity from its position in the
+        // segment: segments start on even steps
+        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
+        if (sparse_ll) p.lseg += p.lseg & 1;
         nseg = int((int64_t(s.L) + p.lseg - 1) / p.lseg);      // drop segments the rounding left empty
         p.nseg = nseg;
         tl_last_segments = nseg;
@@ -647,8 +652,10 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
             p.inc = inc;
         }
-        MainKernelTimer timer(stream, e->name);
-        SIG_HIP(e->fwd(p));
+        const bool use_ll = sparse_ll && e->staged && e->fwd_lead_lag && !p.from_points;
+        const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
+        MainKernelTimer timer(stream, shown.c_str());
+        SIG_HIP(use_ll ? e->fwd_lead_lag(p) : e->fwd(p));
         timer.stop(/*defer=*/true);
         if (nseg > 1) {
             // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches
@@ -935,6 +942,7 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_l
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
 CUSIG_AMD_API int cusig_amd_last_segments(void) noexcept { return tl_last_segments; }
 CUSIG_AMD_API void cusig_amd_set_point_fed(int on) noexcept { g_point_fed = on; }
+CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) noexcept { g_lead_lag_sparse = on; }
 
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force_bwd_segments = segments; }
 

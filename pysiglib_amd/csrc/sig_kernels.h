@@ -230,20 +230,23 @@ __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__
     for (; i + 2 <= count; i += 2) {
         cx.load_inc(zb, row + DIR * d);
         loads_issued();
-        step(za, first + DIR * i, IntC<-1>{});
+        step(za, first + DIR * i, IntC<-1>{}, IntC<0>{});
         if constexpr (WAIT_ALL) wait_all_loads();
         cx.load_inc(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
         loads_issued();
-        step(zb, first + DIR * (i + 1), IntC<-1>{});
+        step(zb, first + DIR * (i + 1), IntC<-1>{}, IntC<1>{});
         if constexpr (WAIT_ALL) wait_all_loads();
         row += 2 * DIR * d;
     }
-    if (i < count) step(za, first + DIR * i, IntC<-1>{});
+    if (i < count) step(za, first + DIR * i, IntC<-1>{}, IntC<0>{});
 }
 
 // staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0
 // points (wave-uniform; forward sweeps of plain paths only): `row` is the path point of the first step instead of an
 // increment row, and the ring takes differences of consecutive points.
+// step(increments, step index, IntC<G0>, IntC<position>): position 0 / 1 alternate from the first step of the range on
+// (chunks hold an even number of steps), so a range that starts on an even step hands the step's parity to `step`
+// as a compile-time constant.
 template <int DIR, int G0, typename Tr, typename Cx, typename T, typename StepFn>
 __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
                                              T* lds_wave, StepFn&& step, bool points = false)
@@ -303,14 +306,14 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
             if constexpr (DIR > 0) wait_lds();
             load_row(zb, lp + DIR * D);
             loads_issued();
-            step(za, first + DIR * (done + i), IntC<G0>{});
+            step(za, first + DIR * (done + i), IntC<G0>{}, IntC<0>{});
             if constexpr (DIR > 0) wait_lds();
             load_row(za, lp + 2 * DIR * D);                      // may be row 0 of the next chunk (contiguous or wrap copy)
             loads_issued();
-            step(zb, first + DIR * (done + i + 1), IntC<G0>{});
+            step(zb, first + DIR * (done + i + 1), IntC<G0>{}, IntC<1>{});
             lp += 2 * DIR * D;
         }
-        if (i < nk) step(za, first + DIR * (done + i), IntC<G0>{});          // odd tail: only in the last chunk
+        if (i < nk) step(za, first + DIR * (done + i), IntC<G0>{}, IntC<0>{});          // odd tail: only in the last chunk
         done += nk;
     }
 }
@@ -318,11 +321,14 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
 // ---------------------------------------------------------------------------
 // Forward sweep.
 // ---------------------------------------------------------------------------
-template <typename T, int D, int N, int TAIL, int K, bool ZL>
+// LL: the increments have lead-lag structure (1: with a time channel as last letter, D odd; 2: without, D even) and every
+// range handed to a wave starts on an even step (lseg even): steps then skip the letters that cannot move (LeadLagLetters).
+template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d_rt,
     int64_t out_stride, int scalar, int nseg, int64_t lseg, int* __restrict__ nonfinite, int from_points)
 {
+    static_assert(LL == 0 || (ZL && D >= 2 && ((LL == 1) == ((D & 1) == 1))), "lead-lag variants: staged, time channel iff D is odd");
     // `nonfinite` (may be null): set to 1 when any stored value is NaN or infinite.
     // `from_points` (staged kernels of narrow paths only): `inc` is the plain path [batch][L + 1][d] itself and the
     // increments are formed while they are staged.
@@ -349,7 +355,10 @@ __global__ __launch_bounds__(kBlock) void tree_fwd_kernel(
     const int64_t ns = (L - t0 < lseg) ? L - t0 : lseg;      // steps of this segment (>= 1)
     // row of the segment's first step (increments: [batch][L + 2][d] with a zero row at either end)
     const T* row = from_points ? inc + ((cx.id.b / nseg) * (L + 1) + t0) * d : inc + ((cx.id.b / nseg) * (L + 2) + 1 + t0) * d;
-    auto step = [&](const typename Tr::Inc& z, int64_t, auto) { S.fwd_step(z); };
+    auto step = [&](const typename Tr::Inc& z, int64_t, auto g0c, auto pos) {
+        if constexpr (LL == 0) S.fwd_step(z);
+        else S.template fwd_step<LeadLagLetters<Tr::DD, decltype(pos)::value, decltype(g0c)::value>>(z);
+    };
     if constexpr (ZL) {
         static_assert(LaneCtx<T, D, N, TAIL, K>::WIDE, "staged increments need the wide layout");
         extern __shared__ double lds_raw_f[];
@@ -643,7 +652,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         wave_lds_sync();
     };
 
-    auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c) {
+    auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c, auto) {
         constexpr int G0 = decltype(g0c)::value;
         constexpr bool FOLD = Ad::template kFoldDepth1<G0>;     // depth-1 pieces already sit in dz.dj
         S.fwd_step(negate<T, D, N, TAIL, K>(z));     // state before the step

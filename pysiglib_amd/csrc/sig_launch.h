@@ -18,9 +18,10 @@ hipError_t allow_lds(Kern kern, size_t bytes)
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
 }
 
-template <typename T, int D, int N, int TAIL, int K, bool ZL>
+template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 hipError_t launch_tree_fwd(const FwdParams& p)
 {
+    if (LL != 0 && ((p.lseg & 1) || p.from_points)) return hipErrorInvalidConfiguration;    // ranges must start on even steps
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);
     if (D < 0 && !g.wide) return hipErrorInvalidConfiguration;     // the kernel was compiled for the wide layout
     const int64_t waves = total_waves(g, p.batch);
@@ -33,10 +34,10 @@ hipError_t launch_tree_fwd(const FwdParams& p)
     if (ZL) {
         if (!g.wide) return hipErrorInvalidConfiguration;
         lds = size_t(kWavesPerBlock) * IncRing<T, (D > 0 ? D : 1), 1>::ELEMS * sizeof(T);
-        hipError_t e = allow_lds(tree_fwd_kernel<T, D, N, TAIL, K, ZL>, lds);
+        hipError_t e = allow_lds(tree_fwd_kernel<T, D, N, TAIL, K, ZL, LL>, lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
+    hipLaunchKernelGGL((tree_fwd_kernel<T, D, N, TAIL, K, ZL, LL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<T*>(p.out), p.batch, p.L, p.d,
                        p.out_stride, p.scalar, p.nseg, p.lseg, p.nonfinite, (ZL && D > 0 && D <= kPointFedMaxDim) ? p.from_points : 0);
     return hipGetLastError();

@@ -47,6 +47,9 @@ struct KernelEntry {
     int preferred;   // default partition of its shape
     int (*waves_per_simd)();   // register-limited residency of the kernel
     int stage_policy;          // which twin to launch: 0 general rules, 1 always the staged one, 2 never, 3 only when under-filled
+    // staged forward instances: the same sweep for lead-lag increments (with a time channel iff D is odd), which
+    // skips the letters a step cannot move; null when not compiled.  Needs an even FwdParams::lseg.
+    FwdFn fwd_lead_lag = nullptr;
 };
 
 // every generated instance file contributes one array

@@ -159,6 +159,27 @@ __device__ __forceinline__ LaneId lane_id(const TreeGeom& G, int64_t batch, bool
 // ---------------------------------------------------------------------------
 // Per-lane signature state and the Horner step on it.
 // ---------------------------------------------------------------------------
+// Which letters of a step's increment can be non-zero, known at compile time.
+// Lead-lag paths move one half of the channels per step (siglib/cpsig/cp_path.h:262-279): with d_raw = D / 2 raw
+// channels, steps of odd index move the letters [0, d_raw), steps of even index the letters [d_raw, 2 d_raw), and a
+// time channel (the last letter when D is odd) moves in every step.  A forward step that knows this skips the
+// multiply-adds by the zero letters - they would add exactly nothing - which is close to half of its work.
+// G0: first depth-1 letter of the lane's group when known at compile time, else -1 (depth 1 is then treated as dense).
+struct AllLetters {
+    static constexpr int G0 = -1;
+    __host__ __device__ static constexpr bool on(int) { return true; }
+};
+template <int D, int PARITY, int G0_>
+struct LeadLagLetters {
+    static constexpr int G0 = G0_;
+    __host__ __device__ static constexpr bool on(int letter)
+    {
+        const int d_raw = D / 2;
+        if ((D & 1) && letter == D - 1) return true;                        // time
+        return PARITY ? letter < d_raw : (letter >= d_raw && letter < 2 * d_raw);
+    }
+};
+
 template <typename T, int D, int N, int TAIL, int K>
 struct Tree {
     static_assert(TAIL >= 1 && TAIL < N, "need a non-empty prefix and a non-empty subtree");
@@ -243,38 +264,47 @@ struct Tree {
 
     // Descend the subtree for target depth I (target level t = M + I).  `upar`
     // is U_t of the parent (depth E-1 node `pidx`; the root is the prefix p).
-    template <int E, int I>
+    // ACT: the letters that can be non-zero in this step; the others' multiply-adds are left out
+    template <int E, typename ACT>
+    __host__ __device__ static constexpr bool letter_on(int ch)
+    {
+        if (E == 1) return ACT::G0 < 0 || ACT::on(ACT::G0 + ch);
+        return ACT::on(ch);
+    }
+    template <int E, int I, typename ACT = AllLetters>
     __device__ __forceinline__ void fwd_desc(const Inc& in, T upar, int pidx)
     {
         constexpr int NCH = (E == 1) ? K : DD;
         if constexpr (E == I) {
 #pragma unroll
             for (int ch = 0; ch < NCH; ++ch)
-                s[off(E) + pidx * NCH + ch] = fmadd(upar, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+                if (letter_on<E, ACT>(ch))
+                    s[off(E) + pidx * NCH + ch] = fmadd(upar, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
         } else {
             // the children's Horner values first, their consumers afterwards: no FMA directly follows its producer
             const T ur = upar * rcp<T>(I - E + 1);
             T uc[NCH];
 #pragma unroll
-            for (int ch = 0; ch < NCH; ++ch) uc[ch] = fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+            for (int ch = 0; ch < NCH; ++ch)
+                uc[ch] = letter_on<E, ACT>(ch) ? fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]) : s[off(E) + pidx * NCH + ch];
             if constexpr (NCH >= 4) pin();      // narrow fans: the regions between pins would be too small to fill
 #pragma unroll
-            for (int ch = 0; ch < NCH; ++ch) fwd_desc<E + 1, I>(in, uc[ch], pidx * NCH + ch);
+            for (int ch = 0; ch < NCH; ++ch) fwd_desc<E + 1, I, ACT>(in, uc[ch], pidx * NCH + ch);
         }
     }
 
     // subtree target levels t, t-1, ..., M+1: descending, so that every read of a shallower depth still sees the
     // value from before the step
-    template <int t>
+    template <int t, typename ACT = AllLetters>
     __device__ __forceinline__ void fwd_subtree(const Inc& in, const Chain& ch)
     {
         if constexpr (t > M) {
-            fwd_desc<1, t - M>(in, ch.u[t][M - 1], 0);
-            fwd_subtree<t - 1>(in, ch);
+            fwd_desc<1, t - M, ACT>(in, ch.u[t][M - 1], 0);
+            fwd_subtree<t - 1, ACT>(in, ch);
         }
     }
 
-    template <int t>
+    template <int t, typename ACT = AllLetters>
     __device__ __forceinline__ void fwd_level(const Inc& in)
     {
         if constexpr (t == 1) {
@@ -286,23 +316,24 @@ struct Tree {
         } else {
             T u[M > 0 ? M : 1];
             chain_u<t, M>(in, u);
-            fwd_desc<1, t - M>(in, u[M - 1], 0);
+            fwd_desc<1, t - M, ACT>(in, u[M - 1], 0);
         }
-        if constexpr (t > 1) fwd_level<t - 1>(in);
+        if constexpr (t > 1) fwd_level<t - 1, ACT>(in);
     }
 
     // S <- S (x) exp(z): target levels in descending order so that every read of
     // a lower level still sees the value from before the step
     // (siglib/cpsig/cp_signature.h:464-499).
+    template <typename ACT = AllLetters>
     __device__ __forceinline__ void fwd_step(const Inc& in)
     {
         if constexpr (!kLockstep) {
-            fwd_level<N>(in);
+            fwd_level<N, ACT>(in);
             return;
         }
         Chain ch;
         chain_all(in, ch);
-        fwd_subtree<N>(in, ch);
+        fwd_subtree<N, ACT>(in, ch);
 #pragma unroll
         for (int t = M; t >= 2; --t) c[t - 1] = fmadd(ch.u[t][t - 2], in.pz[t - 1], c[t - 1]);
         c[0] += in.pz[0];

@@ -253,6 +253,57 @@ def test_point_fed_staging(P):
     assert fed > 100     # the staged kernels did run
 
 
+def test_lead_lag_sparse_steps(P, oracle):
+    """Staged forward sweeps of lead-lag paths leave out the multiply-adds by the channels a step cannot move (their
+    increments are exactly zero): same bits as the dense sweep of the same pieces, for both time-augmentation settings,
+    odd and even lengths, forced time segments (which must start on even steps), and against the oracle."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_lead_lag_sparse.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_lead_lag_sparse.restype = None
+    L.CUSIG.cusig_amd_force_staged.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_staged.restype = None
+    rng = np.random.default_rng(777)
+    ran = 0
+    try:
+        L.CUSIG.cusig_amd_force_staged(1)
+        for (d_raw, n) in ((8, 4), (2, 6), (3, 5), (5, 4), (4, 3), (10, 3), (2, 8)):
+            for time_aug in (False, True):
+                for length in (2, 3, 8, 9, 17, 40):
+                    for segments in (0, 3):
+                        for dtype in (torch.float64, torch.float32):
+                            x = torch.as_tensor(rng.standard_normal((40, length, d_raw)).cumsum(1) * 0.3, dtype=dtype, device=DEV)
+                            kw = dict(time_aug=time_aug, lead_lag=True)
+                            L.CUSIG.cusig_amd_force_segments(segments)
+                            L.CUSIG.cusig_amd_set_lead_lag_sparse(0)
+                            ref = P.sig(x, n, **kw)
+                            pieces = L.CUSIG.cusig_amd_last_segments()
+                            L.CUSIG.cusig_amd_set_lead_lag_sparse(1)
+                            L.CUSIG.cusig_amd_set_profiling(1)
+                            out = P.sig(x, n, **kw)
+                            name = L.CUSIG.cusig_amd_last_kernel_name().decode()
+                            L.CUSIG.cusig_amd_set_profiling(0)
+                            ran += name.endswith("_ll")
+                            if pieces == 1 and L.CUSIG.cusig_amd_last_segments() == 1:
+                                assert torch.equal(out, ref), (d_raw, n, time_aug, length, segments, dtype, name)
+                            else:       # pieces of even length may be cut elsewhere: another order of additions
+                                tol = 1e-12 if dtype == torch.float64 else 2e-5
+                                scale = ref.abs().max().item()
+                                assert (out - ref).abs().max().item() <= tol * max(scale, 1.0), (d_raw, n, time_aug, length, segments, dtype, name)
+        x = rng.standard_normal((256, 21, 4)).cumsum(1) * 0.3
+        for time_aug in (False, True):
+            want = oracle.signature(x, 4, time_aug=time_aug, lead_lag=True)
+            got = P.sig(dev(x), 4, time_aug=time_aug, lead_lag=True).cpu().numpy()
+            assert level_rel_err(got, want, 8 + int(time_aug), 4) <= 1e-10
+    finally:
+        L.CUSIG.cusig_amd_force_segments(0)
+        L.CUSIG.cusig_amd_set_lead_lag_sparse(1)
+        L.CUSIG.cusig_amd_force_staged(-1)
+        L.CUSIG.cusig_amd_set_profiling(0)
+    assert ran > 100     # the lead-lag twins did run
+
+
 def test_overflow_report(P):
     """The kernels that store the signature flag NaN / Inf themselves (the reference scans the result,
     pysiglib/sig.py:299-310): the report must agree with a scan on every forward route."""
