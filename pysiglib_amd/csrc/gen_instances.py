@@ -207,6 +207,10 @@ def main():
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
                              "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))
+                if lead_lag_mode(D, zl):
+                    lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, true, %d>(const %s*, const %s*, "
+                                 "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);"
+                                 % (T, D, N, tail, K, lead_lag_mode(D, zl), T, T, T, T))
         lines.append("")
         lines.append("#if !defined(__HIP_DEVICE_COMPILE__)   // the launcher table is host data")
         lines.append("static const KernelEntry kEntries_%02d[] = {" % fi)
@@ -222,8 +226,10 @@ def main():
                 lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d, %s},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol, ll_fn))
             else:
-                lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, &bwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d},'
-                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol))
+                ll = lead_lag_mode(D, zl)
+                ll_fn = ("&launch_tree_bwd<%s, %d, %d, %d, %d, true, %d>" % (T, D, N, tail, K, ll)) if ll else "nullptr"
+                lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, &bwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d, nullptr, %s},'
+                             % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol, ll_fn))
         lines.append("};")
         lines.append("extern const EntryList kList_%02d = {kEntries_%02d, %d};" % (fi, fi, len(bucket)))
         lines.append("#endif")

@@ -795,14 +795,18 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                                                         return ring ? c : std::max(c, 700e-9);
                                                     },
                                                     sizeof(T) == 8);
+        // lead-lag sweeps that skip the letters a step cannot move read a step's parity off its position in the
+        // segment: segments start on even steps (a lead-lag path has an even number of steps)
+        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
+        int64_t lseg = int64_t(s.L);
         if (nseg > 1) {
-            const int64_t lseg = (int64_t(s.L) + nseg - 1) / nseg;
+            lseg = (int64_t(s.L) + nseg - 1) / nseg;
+            if (sparse_ll) lseg += lseg & 1;
             nseg = int((int64_t(s.L) + lseg - 1) / lseg);
         }
         if (nseg > 1) {
             // (path, segment) rows, scalar-free: segment signatures, their running products from the left (the state
             // at each segment's end), from the right (what follows each segment), and the adjoints of the states
-            const int64_t lseg = (int64_t(s.L) + nseg - 1) / nseg;
             const uint64_t rows = checked_mul(batch, uint64_t(nseg), "segment signatures");
             const uint64_t bytes = checked_mul(checked_mul(rows, n_coef, "segment signatures"), sizeof(T), "segment signatures");
             T* segs = static_cast<T*>(workspace(2, bytes));
@@ -815,7 +819,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             f.lseg = lseg; f.nseg = nseg; f.out = segs; f.out_stride = n; f.scalar = 0;
             const TreeGeom fgeom = make_geom(int(s.d_aug), ef->N - ef->tail, ef->k, ef->D != 0);
             ef = pick_variant(false, ef, total_waves(fgeom, f.batch));
-            SIG_HIP(ef->fwd(f));
+            SIG_HIP((sparse_ll && ef->staged && ef->fwd_lead_lag) ? ef->fwd_lead_lag(f) : ef->fwd(f));
             // both scans by doubling: ceil(log2(nseg)) launches, ping-ponging between two scratch copies
             int steps = 0;
             while ((1 << steps) < nseg) ++steps;
@@ -852,8 +856,10 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
         }
         e = pick_variant(true, e, total_waves(geom, p.batch));
-        MainKernelTimer timer(stream, e->name);
-        SIG_HIP(e->bwd(p));
+        const bool use_ll = sparse_ll && e->staged && e->bwd_lead_lag && (s.L & 1) == 0;
+        const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
+        MainKernelTimer timer(stream, shown.c_str());
+        SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
         timer.stop();
         launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
             using I = decltype(ix);

@@ -486,7 +486,10 @@ __device__ __forceinline__ void dev_add(T* p, T v)
 #endif
 constexpr bool kBwdXcd = SIGAMD_BWD_XCD != 0;
 
-template <typename T, int D, int N, int TAIL, int K, bool ZL>
+// LL: as in tree_fwd_kernel, and every item runs an even number of steps from an even first step (L and lseg even), so
+// that the reverse sweep starts on an odd step; the gradients of the letters a step cannot move are left at zero
+// (the raw path gradient never reads them).
+template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
     T* __restrict__ dzinc, int64_t batch, int64_t L, int d_rt, int64_t sig_stride, int scalar,
@@ -652,10 +655,12 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         wave_lds_sync();
     };
 
-    auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c, auto) {
+    auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c, auto posc) {
         constexpr int G0 = decltype(g0c)::value;
         constexpr bool FOLD = Ad::template kFoldDepth1<G0>;     // depth-1 pieces already sit in dz.dj
-        S.fwd_step(negate<T, D, N, TAIL, K>(z));     // state before the step
+        // position 0 of the reverse sweep is the last step of an even-length range: an odd step
+        using Act = std::conditional_t<LL == 0, AllLetters, LeadLagLetters<Tr::DD, 1 - decltype(posc)::value, G0>>;
+        S.template fwd_step<Act>(negate<T, D, N, TAIL, K>(z));     // state before the step
         typename Ad::DInc dz;
 #pragma unroll
         for (int j = 0; j < Tr::DD; ++j) dz.dj[j] = T(0);
@@ -663,7 +668,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         for (int a = 0; a < K; ++a) dz.da[a] = T(0);
 #pragma unroll
         for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
-        A.template pullback<G0>(S, z, dz);
+        A.template pullback<G0, Act>(S, z, dz);
 
         if (tiled) {
             // Idle lanes need no predicate: their adjoints were loaded as zero, so every piece they produce is zero.

@@ -67,9 +67,12 @@ int bwd_waves_per_simd()
     return blocks < 1 ? 1 : blocks;
 }
 
-template <typename T, int D, int N, int TAIL, int K, bool ZL>
+template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
+    static_assert(LL == 0 || (ZL && D >= 4), "the lead-lag sweep is a staged, fixed-dimension kernel");
+    // the lead-lag sweep reads a step's parity off its position in the range: ranges must be even and start even
+    if (LL != 0 && ((p.L & 1) || (p.nseg > 1 && (p.lseg & 1)))) return hipErrorInvalidConfiguration;
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);
     if (D < 0 && !g.wide) return hipErrorInvalidConfiguration;     // the kernel was compiled for the wide layout
     const int64_t waves = total_waves(g, p.batch);
@@ -89,10 +92,10 @@ hipError_t launch_tree_bwd(const BwdParams& p)
         lds += size_t(kWavesPerBlock) * IncRing<T, (D > 0 ? D : 1), -1>::ELEMS * sizeof(T);
     }
     {
-        hipError_t e = allow_lds(tree_bwd_kernel<T, D, N, TAIL, K, ZL>, lds);
+        hipError_t e = allow_lds(tree_bwd_kernel<T, D, N, TAIL, K, ZL, LL>, lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K, ZL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
+    hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K, ZL, LL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
                        static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,
                        p.sig_stride, p.scalar, use_lds, p.nseg, p.lseg > 0 ? p.lseg : p.L);

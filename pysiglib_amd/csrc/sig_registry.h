@@ -50,6 +50,8 @@ struct KernelEntry {
     // staged forward instances: the same sweep for lead-lag increments (with a time channel iff D is odd), which
     // skips the letters a step cannot move; null when not compiled.  Needs an even FwdParams::lseg.
     FwdFn fwd_lead_lag = nullptr;
+    // staged backward instances: likewise; needs an even number of steps per path and an even BwdParams::lseg.
+    BwdFn bwd_lead_lag = nullptr;
 };
 
 // every generated instance file contributes one array

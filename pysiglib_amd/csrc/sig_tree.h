@@ -370,7 +370,10 @@ struct TreeAdj {
     // gradient at depth I and the recursion's return values above it.
     // G0 >= 0: the lane's depth-1 letters are the compile-time letters G0 .. G0+K-1 and their pieces are added
     // to dj[G0 + a] straight away (da stays untouched); G0 < 0: the letters are only known at run time -> da.
-    template <int E, int I, int G0>
+    // ACT: the letters that can be non-zero in this step.  A letter that cannot move contributes nothing to the
+    // contractions with z, and its increment gradient is never read (the raw path gradient takes, per step, only the
+    // channels that step moves), so both of its multiply-adds are left out; the adjoint itself still flows through it.
+    template <int E, int I, int G0, typename ACT = AllLetters>
     __device__ __forceinline__ T bwd_desc(const Tr& S, const typename Tr::Inc& in, DInc& dz, T upar, int pidx)
     {
         constexpr int NCH = (E == 1) ? K : DD;
@@ -381,7 +384,9 @@ struct TreeAdj {
         if constexpr (E < I) {
             // the children's Horner values first, their consumers afterwards
 #pragma unroll
-            for (int ch = 0; ch < NCH; ++ch) uc[ch] = fmadd(v, Tr::template zc<E>(in, ch), S.s[Tr::off(E) + pidx * NCH + ch]);
+            for (int ch = 0; ch < NCH; ++ch)
+                uc[ch] = Tr::template letter_on<E, ACT>(ch) ? fmadd(v, Tr::template zc<E>(in, ch), S.s[Tr::off(E) + pidx * NCH + ch])
+                                                            : S.s[Tr::off(E) + pidx * NCH + ch];
             if constexpr (NCH >= 4) Tr::pin();
         }
 #pragma unroll
@@ -391,9 +396,10 @@ struct TreeAdj {
             if constexpr (E == I) {
                 adj = gs[ci];
             } else {
-                adj = bwd_desc<E + 1, I, G0>(S, in, dz, uc[ch], pidx * NCH + ch);
+                adj = bwd_desc<E + 1, I, G0, ACT>(S, in, dz, uc[ch], pidx * NCH + ch);
                 gs[ci] += adj;
             }
+            if (!Tr::template letter_on<E, ACT>(ch)) continue;
             if constexpr (E == 1 && kFoldDepth1<G0>) {
                 if (G0 + ch < DD) dz.dj[(G0 + ch < DD) ? G0 + ch : 0] = fmadd(adj, v, dz.dj[(G0 + ch < DD) ? G0 + ch : 0]);
             } else if constexpr (E == 1) {
@@ -422,7 +428,7 @@ struct TreeAdj {
         dz.dc[0] = fmadd(adj, rcp<T>(t), dz.dc[0]);
     }
 
-    template <int t, int G0>
+    template <int t, int G0, typename ACT = AllLetters>
     __device__ __forceinline__ void bwd_level(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
         if constexpr (t == 1) {
@@ -434,22 +440,22 @@ struct TreeAdj {
         } else {
             T u[M > 0 ? M : 1];
             S.template chain_u<t, M>(in, u);
-            const T red = bwd_desc<1, t - M, G0>(S, in, dz, u[M - 1], 0);
+            const T red = bwd_desc<1, t - M, G0, ACT>(S, in, dz, u[M - 1], 0);
             gc[M - 1] += red;
             chain_up<t, M>(in, dz, u, red);
         }
-        if constexpr (t < N) bwd_level<t + 1, G0>(S, in, dz);
+        if constexpr (t < N) bwd_level<t + 1, G0, ACT>(S, in, dz);
     }
 
     // subtree target levels M+1 .. N in ascending order: the upstream adjoint of depth I is consumed before
     // deeper targets add into it.  a[t] receives the adjoint flowing into the prefix node's Horner value.
-    template <int t, int G0>
+    template <int t, int G0, typename ACT = AllLetters>
     __device__ __forceinline__ void bwd_subtree(const Tr& S, const typename Tr::Inc& in, DInc& dz,
                                                 const typename Tr::Chain& ch, T (&a)[N + 1])
     {
         if constexpr (t <= N) {
-            a[t] = bwd_desc<1, t - M, G0>(S, in, dz, ch.u[t][M - 1], 0);
-            bwd_subtree<t + 1, G0>(S, in, dz, ch, a);
+            a[t] = bwd_desc<1, t - M, G0, ACT>(S, in, dz, ch.u[t][M - 1], 0);
+            bwd_subtree<t + 1, G0, ACT>(S, in, dz, ch, a);
         }
     }
 
@@ -457,11 +463,11 @@ struct TreeAdj {
     // the state BEFORE the step.  Target levels ascend so that the adjoint of
     // level t is consumed before higher levels add into it
     // (siglib/cpsig/cp_signature.h:1147-1187).
-    template <int G0 = -1>
+    template <int G0 = -1, typename ACT = AllLetters>
     __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
     {
         if constexpr (!Tr::kLockstep) {
-            bwd_level<1, G0>(S, in, dz);
+            bwd_level<1, G0, ACT>(S, in, dz);
             return;
         }
         typename Tr::Chain ch;
@@ -473,7 +479,7 @@ struct TreeAdj {
         const T g1 = gc[0];
 #pragma unroll
         for (int t = 2; t <= M; ++t) a[t] = gc[t - 1];
-        bwd_subtree<M + 1, G0>(S, in, dz, ch, a);
+        bwd_subtree<M + 1, G0, ACT>(S, in, dz, ch, a);
 #pragma unroll
         for (int t = M + 1; t <= N; ++t) gc[M - 1] += a[t];
 #pragma unroll

@@ -304,6 +304,67 @@ def test_lead_lag_sparse_steps(P, oracle):
     assert ran > 100     # the lead-lag twins did run
 
 
+def test_lead_lag_sparse_backward(P, oracle):
+    """Staged backward sweeps of lead-lag paths leave out, per step, the multiply-adds of the channels that step cannot
+    move (their increments are zero and their increment gradients are never read): same bits as the dense sweep when
+    both run the path in one piece, within tolerance when forced time pieces are cut at different (even) steps, and
+    parity with the oracle."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_bwd_segments.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_bwd_segments.restype = None
+    L.CUSIG.cusig_amd_set_lead_lag_sparse.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_lead_lag_sparse.restype = None
+    L.CUSIG.cusig_amd_force_staged.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_staged.restype = None
+    rng = np.random.default_rng(778)
+    ran = 0
+    try:
+        L.CUSIG.cusig_amd_force_staged(1)
+        for (d_raw, n) in ((8, 4), (2, 6), (3, 5), (5, 4), (4, 3), (10, 3), (2, 8), (15, 3)):
+            for time_aug in (False, True):
+                for length in (2, 3, 8, 9, 17, 40):
+                    for segments in (0, 3):
+                        for dtype in (torch.float64, torch.float32):
+                            x = torch.as_tensor(rng.standard_normal((40, length, d_raw)).cumsum(1) * 0.3, dtype=dtype, device=DEV)
+                            kw = dict(time_aug=time_aug, lead_lag=True)
+                            sg = P.sig(x, n, **kw)
+                            g = torch.as_tensor(rng.standard_normal(tuple(sg.shape)), dtype=dtype, device=DEV)
+                            L.CUSIG.cusig_amd_force_bwd_segments(segments)
+                            L.CUSIG.cusig_amd_set_lead_lag_sparse(0)
+                            ref = P.sig_backprop(x, sg, g, n, **kw)
+                            L.CUSIG.cusig_amd_set_lead_lag_sparse(1)
+                            L.CUSIG.cusig_amd_set_profiling(1)
+                            out = P.sig_backprop(x, sg, g, n, **kw)
+                            name = L.CUSIG.cusig_amd_last_kernel_name().decode()
+                            L.CUSIG.cusig_amd_set_profiling(0)
+                            ran += name.endswith("_ll")
+                            case = (d_raw, n, time_aug, length, segments, dtype, name)
+                            if segments == 0 and length < 32:     # one piece either way; pieces share atomics otherwise
+                                tol = 1e-13 if dtype == torch.float64 else 2e-5     # float atomics land in any order
+                            else:
+                                tol = 1e-11 if dtype == torch.float64 else 1e-4
+                            scale = ref.abs().max().item()
+                            assert (out - ref).abs().max().item() <= tol * max(scale, 1.0), case
+        for (d_raw, n, length) in ((4, 4, 21), (3, 5, 12), (8, 3, 30)):
+            x = rng.standard_normal((64, length, d_raw)).cumsum(1) * 0.3
+            for time_aug in (False, True):
+                aug = dict(time_aug=time_aug, lead_lag=True)
+                ref = oracle.signature(x, n, **aug)
+                g = rng.standard_normal(ref.shape)
+                want = oracle.sig_backprop(x, ref, g, n, n_jobs=-1, **aug)
+                for segments in (0, 4):
+                    L.CUSIG.cusig_amd_force_bwd_segments(segments)
+                    got = P.sig_backprop(dev(x), dev(ref), dev(g), n, **aug).cpu().numpy()
+                    assert bwd_rel_err(got, want) <= 1e-10, (d_raw, n, length, time_aug, segments)
+    finally:
+        L.CUSIG.cusig_amd_force_bwd_segments(0)
+        L.CUSIG.cusig_amd_set_lead_lag_sparse(1)
+        L.CUSIG.cusig_amd_force_staged(-1)
+        L.CUSIG.cusig_amd_set_profiling(0)
+    assert ran > 100     # the lead-lag twins did run
+
+
 def test_overflow_report(P):
     """The kernels that store the signature flag NaN / Inf themselves (the reference scans the result,
     pysiglib/sig.py:299-310): the report must agree with a scan on every forward route."""
