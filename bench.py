@@ -23,11 +23,11 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 # known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
 # reports null instead of a stale figure.
 TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5_lds": 35.6e6,
+    "fwd_f64_d10_n5_t2_k5_lds": 35.5e6,
     "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
-    "fwd_f32_d5_n7_t4_k1_lds": 162.2e6,    # swept in three time pieces: three segment signature sets are written
-    "fwd_f64_d3_n12_t5_k1": 477.9e6,
-    "fwd_f32_d17_n4_t2_k6_lds": 113.7e6,
+    "fwd_f32_d5_n7_t4_k1_lds": 163.0e6,    # swept in three time pieces: three segment signature sets are written
+    "fwd_f64_d3_n12_t5_k1": 478.1e6,
+    "fwd_f32_d17_n4_t2_k6_lds_ll": 114.4e6,
 }
 
 
@@ -303,6 +303,10 @@ def main():
                                   # the whole call (sweep plus, when the paths were cut in time, the Chen folds)
                                   "call_roofline_frac": r.flops_fwd / wall / 1e12 / PEAK_TFLOPS[r.dtype],
                                   "time_segments": int(loader.CUSIG.cusig_amd_last_segments())}
+            if name.endswith("_ll"):
+                configs["C%d" % k]["note"] = ("flops are those of the dense sweep over all augmented channels (the reference's "
+                                              "arithmetic); this kernel leaves out the multiply-adds by the channels a lead-lag "
+                                              "step cannot move, so tflops / roofline_frac are effective rates, not pipe utilisation")
             del r
             torch.cuda.empty_cache()
         # degree 2 on paths of many channels: closed form on the matrix cores (not one of the five benchmark workloads)

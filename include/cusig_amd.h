@@ -227,9 +227,10 @@ CUSIG_AMD_API int cusig_amd_last_segments(void) CUSIG_AMD_NOEXCEPT;
  * the LDS-staged sweeps of plain paths (no time or lead-lag augmentation) of at most 16 channels take the
  * differences of consecutive points while they stage them. */
 CUSIG_AMD_API void cusig_amd_set_point_fed(int on) CUSIG_AMD_NOEXCEPT;
-/* Tuning hook: 1 (default) lets LDS-staged forward sweeps of lead-lag paths (up to 40 augmented channels) skip, in
- * every step, the multiply-adds by the channels that step cannot move (lead and lag halves move in turn; the
- * increments there are exactly zero); 0 sweeps them like any other path. */
+/* Tuning hook: 1 (default) lets LDS-staged forward and backward sweeps of lead-lag paths (up to 40 augmented
+ * channels) skip, in every step, the multiply-adds by the channels that step cannot move (lead and lag halves move in
+ * turn; the increments there are exactly zero and their gradients never reach the path gradient); 0 sweeps them
+ * like any other path. */
 CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT;
