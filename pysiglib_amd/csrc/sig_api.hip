@@ -419,8 +419,18 @@ static int choose_bwd_segments(int64_t waves, int64_t L, int waves_per_simd, uin
 // more channels the ring's LDS reads cost them 3-30 % (f64 at 10-12 channels is mixed).
 static int g_force_staged = -1;   // tuning hook: -1 automatic, 0 never, 1 whenever compiled
 
-static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, int64_t waves)
+// lead_lag_sparse: the path is a lead-lag path and staged twins that skip a step's still letters may be used.  Those
+// twins do about 40 % less arithmetic, which outweighs what the tuned choice for dense paths says: measured on 144
+// lead-lag shapes (2-20 raw channels, both precisions), the forward twin is faster wherever it exists (mean 0.82x), the
+// backward twin in single precision and, in double precision, up to 13 augmented channels (mean 0.85x; beyond, its
+// register pressure costs more than the skipped work saves).
+static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, int64_t waves, bool lead_lag_sparse = false)
 {
+    if (lead_lag_sparse && g_force_staged < 0) {
+        const KernelEntry* twin = base->staged ? base : staged_twin(backward, base);
+        if (twin && (backward ? (twin->bwd_lead_lag && (!twin->is_f64 || twin->D <= 13)) : twin->fwd_lead_lag != nullptr))
+            return twin;
+    }
     const bool small_dim = base->D > 0 && base->D <= (base->is_f64 ? 8 : 13);
     const bool want = g_force_staged >= 0 ? g_force_staged != 0
                       : base->stage_policy == 1 ? true
@@ -604,13 +614,16 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         // Few paths cannot fill the chip with whole-path sweeps: split every path into time segments,
         // sweep all (path, segment) pairs concurrently and fold the pieces with Chen's identity.
         const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
+        // lead-lag sweeps that skip the letters a step cannot move take the step's parity from its position in the
+        // segment: segments start on even steps
+        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
         int nseg = g_force_segments > 0
                              ? int(std::min<uint64_t>(uint64_t(g_force_segments), s.L))
                              : choose_segments(total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
                                                batch * (s.full_len - 1) * sizeof(T),
                                                [&](int g) {
                                                    const double c = lane_step_cost(int(s.d_aug), e->N, e->tail, e->k) * 2.4e-9;
-                                                   const bool ring = pick_variant(false, e, total_waves(geom, int64_t(batch)) * g)->staged;
+                                                   const bool ring = pick_variant(false, e, total_waves(geom, int64_t(batch)) * g, sparse_ll)->staged;
                                                    return ring ? c : std::max(c, 240e-9);
                                                },
                                                sizeof(T) == 8);
@@ -618,9 +631,6 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         FwdParams p;
         p.batch = int64_t(batch) * nseg; p.L = int64_t(s.L); p.d = int(s.d_aug); p.stream = stream;
         p.lseg = (int64_t(s.L) + nseg - 1) / nseg;
-        // lead-lag sweeps that skip the letters a step cannot move take the step's parity from its position in the
-        // segment: segments start on even steps
-        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
         if (sparse_ll) p.lseg += p.lseg & 1;
         nseg = int((int64_t(s.L) + p.lseg - 1) / p.lseg);      // drop segments the rounding left empty
         p.nseg = nseg;
@@ -640,7 +650,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
                                                                  sizeof(T), "segment signatures")));
             p.out = segs; p.out_stride = int64_t(n_coef); p.scalar = 0;
         }
-        e = pick_variant(false, e, total_waves(geom, p.batch));
+        e = pick_variant(false, e, total_waves(geom, p.batch), sparse_ll);
         // staged sweeps of plain narrow paths form the increments themselves while staging the points
         if (e->staged && !time_aug && !lead_lag && e->D > 0 && e->D <= kPointFedMaxDim && g_point_fed) {
             p.inc = path;
@@ -783,6 +793,9 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
         const uint64_t n_coef = s.full_len - 1;
         const KernelEntry* ef = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch, s.L);
+        // lead-lag sweeps that skip the letters a step cannot move read a step's parity off its position in the
+        // segment: segments start on even steps (a lead-lag path has an even number of steps)
+        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
         int nseg = (!ef || degree > uint64_t(kCombMaxLevels)) ? 1
                    : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
                                               : choose_bwd_segments(
@@ -791,13 +804,10 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                                                     [&](int g) {
                                                         // a backward step issues about 3.2 times the forward's instructions
                                                         const double c = lane_step_cost(int(s.d_aug), e->N, e->tail, e->k) * 7.7e-9;
-                                                        const bool ring = pick_variant(true, e, total_waves(geom, int64_t(batch)) * g)->staged;
+                                                        const bool ring = pick_variant(true, e, total_waves(geom, int64_t(batch)) * g, sparse_ll)->staged;
                                                         return ring ? c : std::max(c, 700e-9);
                                                     },
                                                     sizeof(T) == 8);
-        // lead-lag sweeps that skip the letters a step cannot move read a step's parity off its position in the
-        // segment: segments start on even steps (a lead-lag path has an even number of steps)
-        const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
         int64_t lseg = int64_t(s.L);
         if (nseg > 1) {
             lseg = (int64_t(s.L) + nseg - 1) / nseg;
@@ -818,7 +828,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             f.inc = inc; f.batch = int64_t(rows); f.L = int64_t(s.L); f.d = int(s.d_aug); f.stream = stream;
             f.lseg = lseg; f.nseg = nseg; f.out = segs; f.out_stride = n; f.scalar = 0;
             const TreeGeom fgeom = make_geom(int(s.d_aug), ef->N - ef->tail, ef->k, ef->D != 0);
-            ef = pick_variant(false, ef, total_waves(fgeom, f.batch));
+            ef = pick_variant(false, ef, total_waves(fgeom, f.batch), sparse_ll);
             SIG_HIP((sparse_ll && ef->staged && ef->fwd_lead_lag) ? ef->fwd_lead_lag(f) : ef->fwd(f));
             // both scans by doubling: ceil(log2(nseg)) launches, ping-ponging between two scratch copies
             int steps = 0;
@@ -855,7 +865,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             p.sig = left; p.gsig = adj; p.sig_stride = n; p.scalar = 0;
             p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
         }
-        e = pick_variant(true, e, total_waves(geom, p.batch));
+        e = pick_variant(true, e, total_waves(geom, p.batch), sparse_ll);
         const bool use_ll = sparse_ll && e->staged && e->bwd_lead_lag && (s.L & 1) == 0;
         const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str());
