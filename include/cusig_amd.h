@@ -227,8 +227,8 @@ CUSIG_AMD_API int cusig_amd_last_segments(void) CUSIG_AMD_NOEXCEPT;
  * the LDS-staged sweeps of plain paths (no time or lead-lag augmentation) of at most 16 channels take the
  * differences of consecutive points while they stage them. */
 CUSIG_AMD_API void cusig_amd_set_point_fed(int on) CUSIG_AMD_NOEXCEPT;
-/* Tuning hook: 1 (default) lets LDS-staged forward and backward sweeps of lead-lag paths (up to 40 augmented
- * channels) skip, in every step, the multiply-adds by the channels that step cannot move (lead and lag halves move in
+/* Tuning hook: 1 (default) lets the forward and backward sweeps of lead-lag paths that have such a form (up to 40
+ * augmented channels; the LDS-staged kernels and the wider scalar-fed backward kernels) skip, in every step, the multiply-adds by the channels that step cannot move (lead and lag halves move in
  * turn; the increments there are exactly zero and their gradients never reach the path gradient); 0 sweeps them
  * like any other path. */
 CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) CUSIG_AMD_NOEXCEPT;

@@ -118,6 +118,17 @@ def lead_lag_mode(D, staged):
     return 1 if D % 2 else 2
 
 
+def lead_lag_mode_bwd(T, D, tail, staged):
+    """Lead-lag twin of a backward instance.  Staged instances as in the forward; scalar-fed ones where they are the
+    faster choice for lead-lag paths (double precision from 14 channels on, single precision beyond the staged range)
+    and the subtree has a level below the lane's own letters for the mask to act on."""
+    if staged:
+        return lead_lag_mode(D, True)
+    if tail < 2 or D > 40 or D < (14 if T == "double" else 32):
+        return 0
+    return 1 if D % 2 else 2
+
+
 def choose(D, N, dtype, direction):
     key = (dtype, D, N, direction)
     if key in OVERRIDES:
@@ -207,10 +218,10 @@ def main():
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
                              "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))
-                if lead_lag_mode(D, zl):
-                    lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, true, %d>(const %s*, const %s*, "
+                if lead_lag_mode_bwd(T, D, tail, zl):
+                    lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s, %d>(const %s*, const %s*, "
                                  "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);"
-                                 % (T, D, N, tail, K, lead_lag_mode(D, zl), T, T, T, T))
+                                 % (T, D, N, tail, K, zs, lead_lag_mode_bwd(T, D, tail, zl), T, T, T, T))
         lines.append("")
         lines.append("#if !defined(__HIP_DEVICE_COMPILE__)   // the launcher table is host data")
         lines.append("static const KernelEntry kEntries_%02d[] = {" % fi)
@@ -226,8 +237,8 @@ def main():
                 lines.append('    {%d, %d, %d, %d, %d, %d, &launch_tree_fwd<%s, %d, %d, %d, %d, %s>, nullptr, "%s", %d, &fwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d, %s},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol, ll_fn))
             else:
-                ll = lead_lag_mode(D, zl)
-                ll_fn = ("&launch_tree_bwd<%s, %d, %d, %d, %d, true, %d>" % (T, D, N, tail, K, ll)) if ll else "nullptr"
+                ll = lead_lag_mode_bwd(T, D, tail, zl)
+                ll_fn = ("&launch_tree_bwd<%s, %d, %d, %d, %d, %s, %d>" % (T, D, N, tail, K, zs, ll)) if ll else "nullptr"
                 lines.append('    {%d, %d, %d, %d, %d, %d, nullptr, &launch_tree_bwd<%s, %d, %d, %d, %d, %s>, "%s", %d, &bwd_waves_per_simd<%s, %d, %d, %d, %d, %s>, %d, nullptr, %s},'
                              % (is64, D, N, tail, K, zl, T, D, N, tail, K, zs, name, pref, T, D, N, tail, K, zs, pol, ll_fn))
         lines.append("};")

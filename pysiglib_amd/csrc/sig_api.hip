@@ -423,7 +423,8 @@ static int g_force_staged = -1;   // tuning hook: -1 automatic, 0 never, 1 whene
 // twins do about 40 % less arithmetic, which outweighs what the tuned choice for dense paths says: measured on 144
 // lead-lag shapes (2-20 raw channels, both precisions), the forward twin is faster wherever it exists (mean 0.82x), the
 // backward twin in single precision and, in double precision, up to 13 augmented channels (mean 0.85x; beyond, its
-// register pressure costs more than the skipped work saves).
+// register pressure costs more than the skipped work saves, and the general rules below decide; the scalar-fed
+// backward kernels of those dimensions have a lead-lag form of their own).
 static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, int64_t waves, bool lead_lag_sparse = false)
 {
     if (lead_lag_sparse && g_force_staged < 0) {
@@ -866,7 +867,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
         }
         e = pick_variant(true, e, total_waves(geom, p.batch), sparse_ll);
-        const bool use_ll = sparse_ll && e->staged && e->bwd_lead_lag && (s.L & 1) == 0;
+        const bool use_ll = sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
         const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str());
         SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));

@@ -70,7 +70,7 @@ int bwd_waves_per_simd()
 template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 hipError_t launch_tree_bwd(const BwdParams& p)
 {
-    static_assert(LL == 0 || (ZL && D >= 4), "the lead-lag sweep is a staged, fixed-dimension kernel");
+    static_assert(LL == 0 || (D >= 4 && (ZL || TAIL >= 2)), "the lead-lag sweep needs a compile-time dimension");
     // the lead-lag sweep reads a step's parity off its position in the range: ranges must be even and start even
     if (LL != 0 && ((p.L & 1) || (p.nseg > 1 && (p.lseg & 1)))) return hipErrorInvalidConfiguration;
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);

@@ -50,7 +50,8 @@ struct KernelEntry {
     // staged forward instances: the same sweep for lead-lag increments (with a time channel iff D is odd), which
     // skips the letters a step cannot move; null when not compiled.  Needs an even FwdParams::lseg.
     FwdFn fwd_lead_lag = nullptr;
-    // staged backward instances: likewise; needs an even number of steps per path and an even BwdParams::lseg.
+    // backward instances (staged, and scalar-fed ones with a subtree level below the lane's own letters): likewise; needs
+    // an even number of steps per path and an even BwdParams::lseg.
     BwdFn bwd_lead_lag = nullptr;
 };
 

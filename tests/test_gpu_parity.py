@@ -319,14 +319,19 @@ def test_lead_lag_sparse_backward(P, oracle):
     L.CUSIG.cusig_amd_force_staged.restype = None
     rng = np.random.default_rng(778)
     ran = 0
+    ran_direct = 0
     try:
-        L.CUSIG.cusig_amd_force_staged(1)
-        for (d_raw, n) in ((8, 4), (2, 6), (3, 5), (5, 4), (4, 3), (10, 3), (2, 8), (15, 3)):
+        # staged kernels, then the scalar-fed ones (which have a lead-lag form from 14 channels on in double precision
+        # and from 32 on in single precision, where the mask acts on the subtree level below the lane's own letters)
+        cases = [(1, d_raw, n, 40) for (d_raw, n) in ((8, 4), (2, 6), (3, 5), (5, 4), (4, 3), (10, 3), (2, 8), (15, 3))]
+        cases += [(0, d_raw, n, b) for (d_raw, n, b) in ((7, 3, 64), (8, 4, 48), (10, 3, 70), (10, 4, 40), (12, 4, 24))]
+        for (staged, d_raw, n, batch) in cases:
+            L.CUSIG.cusig_amd_force_staged(staged)
             for time_aug in (False, True):
                 for length in (2, 3, 8, 9, 17, 40):
                     for segments in (0, 3):
                         for dtype in (torch.float64, torch.float32):
-                            x = torch.as_tensor(rng.standard_normal((40, length, d_raw)).cumsum(1) * 0.3, dtype=dtype, device=DEV)
+                            x = torch.as_tensor(rng.standard_normal((batch, length, d_raw)).cumsum(1) * 0.3, dtype=dtype, device=DEV)
                             kw = dict(time_aug=time_aug, lead_lag=True)
                             sg = P.sig(x, n, **kw)
                             g = torch.as_tensor(rng.standard_normal(tuple(sg.shape)), dtype=dtype, device=DEV)
@@ -338,7 +343,8 @@ def test_lead_lag_sparse_backward(P, oracle):
                             out = P.sig_backprop(x, sg, g, n, **kw)
                             name = L.CUSIG.cusig_amd_last_kernel_name().decode()
                             L.CUSIG.cusig_amd_set_profiling(0)
-                            ran += name.endswith("_ll")
+                            ran += name.endswith("_lds_ll")
+                            ran_direct += name.endswith("_ll") and not name.endswith("_lds_ll")
                             case = (d_raw, n, time_aug, length, segments, dtype, name)
                             if segments == 0 and length < 32:     # one piece either way; pieces share atomics otherwise
                                 tol = 1e-13 if dtype == torch.float64 else 2e-5     # float atomics land in any order
@@ -346,8 +352,9 @@ def test_lead_lag_sparse_backward(P, oracle):
                                 tol = 1e-11 if dtype == torch.float64 else 1e-4
                             scale = ref.abs().max().item()
                             assert (out - ref).abs().max().item() <= tol * max(scale, 1.0), case
-        for (d_raw, n, length) in ((4, 4, 21), (3, 5, 12), (8, 3, 30)):
-            x = rng.standard_normal((64, length, d_raw)).cumsum(1) * 0.3
+        L.CUSIG.cusig_amd_force_staged(-1)
+        for (d_raw, n, length) in ((4, 4, 21), (3, 5, 12), (8, 3, 30), (8, 4, 14), (10, 3, 11)):
+            x = rng.standard_normal((64 if d_raw < 8 or n < 4 else 6, length, d_raw)).cumsum(1) * 0.3
             for time_aug in (False, True):
                 aug = dict(time_aug=time_aug, lead_lag=True)
                 ref = oracle.signature(x, n, **aug)
@@ -362,7 +369,7 @@ def test_lead_lag_sparse_backward(P, oracle):
         L.CUSIG.cusig_amd_set_lead_lag_sparse(1)
         L.CUSIG.cusig_amd_force_staged(-1)
         L.CUSIG.cusig_amd_set_profiling(0)
-    assert ran > 100     # the lead-lag twins did run
+    assert ran > 100 and ran_direct > 50     # the lead-lag twins of both kinds did run
 
 
 def test_overflow_report(P):
