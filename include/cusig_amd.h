@@ -228,9 +228,9 @@ CUSIG_AMD_API int cusig_amd_last_segments(void) CUSIG_AMD_NOEXCEPT;
  * differences of consecutive points while they stage them. */
 CUSIG_AMD_API void cusig_amd_set_point_fed(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: 1 (default) lets the forward and backward sweeps of lead-lag paths that have such a form (up to 40
- * augmented channels; the LDS-staged kernels and the wider scalar-fed backward kernels) skip, in every step, the multiply-adds by the channels that step cannot move (lead and lag halves move in
- * turn; the increments there are exactly zero and their gradients never reach the path gradient); 0 sweeps them
- * like any other path. */
+ * augmented channels; the LDS-staged kernels and the wider scalar-fed backward kernels) skip, in every step, the
+ * multiply-adds by the channels that step cannot move (lead and lag halves move in turn; the increments there are
+ * exactly zero and their gradients never reach the path gradient); 0 sweeps them like any other path. */
 CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT;
