@@ -669,26 +669,40 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         SIG_HIP(use_ll ? e->fwd_lead_lag(p) : e->fwd(p));
         timer.stop(/*defer=*/true);
         if (nseg > 1) {
-            // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches
+            // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches.  An unpaired last
+            // row stays where it is and joins the next step as its last row (`carry`).
             const T* src = segs;
+            int src_rows = nseg;
+            const T* carry = nullptr;
+            int64_t carry_stride = 0;
             T* next = folds;
-            for (int m = nseg; m > 1; m = (m + 1) / 2) {
+            for (int m = nseg; m > 1;) {
                 const bool last = m == 2;
-                const int half = (m + 1) / 2;
+                const int pairs = m / 2;
                 T* dst = last ? out : next;
                 with_chen_fan(s.d_aug, [&](auto fan) {
                     constexpr int FAN = decltype(fan)::value;
                     const uint64_t items = chen_items(s.d_aug, degree, FAN);
-                    launch_indexed(n_coef, items, batch * uint64_t(half), [&](auto ix, dim3 grid) {
+                    launch_indexed(n_coef, items, batch * uint64_t(pairs), [&](auto ix, dim3 grid) {
                         using I = decltype(ix);
-                        hipLaunchKernelGGL((chen_fold_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, src, dst,
-                                           int64_t(batch), m, last ? int64_t(s.stride) : int64_t(n_coef) * half, last ? sc : 0,
-                                           DivBy<I>(s.d_aug), I(n_coef), I(items), last ? flag : nullptr);
+                        hipLaunchKernelGGL((chen_fold_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, src, src_rows, carry,
+                                           carry_stride, dst, int64_t(batch), m, last ? int64_t(s.stride) : int64_t(n_coef) * pairs,
+                                           last ? sc : 0, DivBy<I>(s.d_aug), I(n_coef), I(items), last ? flag : nullptr);
                     });
                 });
                 SIG_HIP(hipGetLastError());
+                if (m & 1) {
+                    if (!carry) {       // the last row of this step's source becomes the carry
+                        carry = src + uint64_t(m - 1) * n_coef;
+                        carry_stride = int64_t(src_rows) * int64_t(n_coef);
+                    }
+                } else {
+                    carry = nullptr;    // paired in this step, if there was one
+                }
                 src = dst;
-                next += batch * n_coef * uint64_t(half);
+                src_rows = pairs;
+                next += batch * n_coef * uint64_t(pairs);
+                m = pairs + (carry ? 1 : 0);
             }
         }
         exit_sync(stream);

@@ -1173,37 +1173,31 @@ __global__ __launch_bounds__(kBlock) void chen_scan_step_kernel(
     }
 }
 
-// One halving step of the ordered product of m rows per path: dst[path][j] = src[path][2j] (x) src[path][2j+1]
-// (a copy when the right neighbour does not exist).  dst rows have their own stride between paths and may carry a
-// leading scalar slot, so the last step (m = 2) can write the caller's signature directly.
+// One halving step of the ordered product of m rows per path: dst[path][j] = row[2j] (x) row[2j+1] for j < m / 2.
+// The rows of a path are `src_rows` consecutive rows of `src`, followed, when `carry` is set, by one more row that
+// lives elsewhere (carry + path * carry_path_stride).  An unpaired last row is not copied: the caller hands it to the
+// next step as that step's carry.  dst rows have their own stride between paths and may carry a leading scalar slot,
+// so the last step (m = 2) can write the caller's signature directly.
 template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void chen_fold_step_kernel(
-    const T* __restrict__ src, T* __restrict__ dst, int64_t paths, int m, int64_t dst_path_stride, int dst_off,
-    DivBy<I> dv, I sig_len, I items /* chen_items(d, degree, FAN) */, int* __restrict__ nonfinite)
+    const T* __restrict__ src, int src_rows, const T* __restrict__ carry, int64_t carry_path_stride, T* __restrict__ dst,
+    int64_t paths, int m, int64_t dst_path_stride, int dst_off, DivBy<I> dv, I sig_len,
+    I items /* chen_items(d, degree, FAN) */, int* __restrict__ nonfinite)
 {
-    const int half = (m + 1) / 2;
-    for (int64_t y = blockIdx.y; y < paths * half; y += gridDim.y) {
-        const int64_t path = y / half;
-        const int j = int(y % half);
-        const T* a = src + (path * m + 2 * j) * int64_t(sig_len);
-        const T* bb = 2 * j + 1 < m ? a + int64_t(sig_len) : nullptr;
+    const int pairs = m / 2;
+    for (int64_t y = blockIdx.y; y < paths * pairs; y += gridDim.y) {
+        const int64_t path = y / pairs;
+        const int j = int(y % pairs);
+        const T* a = src + (path * src_rows + 2 * j) * int64_t(sig_len);
+        const T* bb = (2 * j + 1 == src_rows) ? carry + path * carry_path_stride : a + int64_t(sig_len);
         T* c = dst + path * dst_path_stride + int64_t(j) * int64_t(sig_len);
-        if (bb) {
-            for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < items; it += I(gridDim.x) * kBlock) {
-                chen_fan<T, I, FAN>(a, bb, it, dv, [&](I r, T sum) {
-                    const T v = a[r] + bb[r] + sum;
-                    c[dst_off + r] = v;
-                    if (nonfinite && not_finite(v)) *nonfinite = 1;
-                });
-                if (dst_off && it == 0) c[0] = T(1);
-            }
-        } else {
-            for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < sig_len; r += I(gridDim.x) * kBlock) {
-                const T v = a[r];
+        for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < items; it += I(gridDim.x) * kBlock) {
+            chen_fan<T, I, FAN>(a, bb, it, dv, [&](I r, T sum) {
+                const T v = a[r] + bb[r] + sum;
                 c[dst_off + r] = v;
                 if (nonfinite && not_finite(v)) *nonfinite = 1;
-                if (dst_off && r == 0) c[0] = T(1);
-            }
+            });
+            if (dst_off && it == 0) c[0] = T(1);
         }
     }
 }
