@@ -718,6 +718,29 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
 // ---------------------------------------------------------------------------
 // backward  (siglib/cpsig/cp_signature.h:909-1019, siglib/cusig/cu_signature.cu:3417-3488)
 // ---------------------------------------------------------------------------
+// increment gradient -> raw path gradient; plain paths with a channel count that allows it take 16 bytes per lane
+template <typename T>
+static void launch_path_grad(const T* dzinc, T* out, uint64_t batch, uint64_t length, uint64_t dimension, bool time_aug,
+                             bool lead_lag, hipStream_t stream)
+{
+    constexpr int V = int(16 / sizeof(T));
+    if (!time_aug && !lead_lag && dimension % V == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(dzinc) % 16 == 0) {
+        const uint64_t per = length * (dimension / V);
+        launch_indexed(per, per, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((path_grad_vec_kernel<T, I, V>), grid, dim3(kBlock), 0, stream, dzinc, out, int64_t(batch),
+                               int64_t(length), DivBy<I>(dimension / V));
+        });
+        return;
+    }
+    launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, dzinc, out, int64_t(batch),
+                           int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
+    });
+}
+
 template <typename T>
 static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const T* sig, uint64_t batch,
                               uint64_t dimension, uint64_t length, uint64_t degree, bool time_aug,
@@ -781,11 +804,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                                int64_t(s.stride), sc, time_tiles, col_groups);
         }
         timer.stop();
-        launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, (const T*)dzinc, out, int64_t(batch),
-                               int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
-        });
+        launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
         SIG_HIP(hipGetLastError());
         exit_sync(stream);      // the workspaces stay locked until the kernels are done
         return;
@@ -886,11 +905,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         MainKernelTimer timer(stream, shown.c_str());
         SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
         timer.stop();
-        launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, (const T*)dzinc, out, int64_t(batch),
-                               int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
-        });
+        launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
         SIG_HIP(hipGetLastError());
         exit_sync(stream);
         return;

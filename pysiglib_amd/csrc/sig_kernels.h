@@ -988,6 +988,43 @@ __global__ __launch_bounds__(kBlock) void path_grad_kernel(
     }
 }
 
+// The same for plain paths (no augmentation) whose channel count is a multiple of V, with V elements per lane in one
+// 16-byte access: there the increment gradient has the layout of the path and the kernel is a pure stream.
+// Grid: x over the len_raw * d_raw / V vector elements of one path, y over the paths; dv divides by d_raw / V.
+template <typename T, int V>
+struct alignas(V * sizeof(T)) VecOf {
+    T v[V];
+};
+template <typename T, typename I, int V>
+__global__ __launch_bounds__(kBlock) void path_grad_vec_kernel(
+    const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, DivBy<I> dv)
+{
+    using Vec = VecOf<T, V>;
+    const I dvec = I(dv.d);
+    const I per = I(len_raw) * dvec;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const Vec* g = reinterpret_cast<const Vec*>(dzinc) + b * (len_raw - 1) * int64_t(dvec);
+        Vec* o = reinterpret_cast<Vec*>(out) + b * int64_t(per);
+        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
+            const int64_t i = int64_t(dv.quot(e));
+            Vec r;
+#pragma unroll
+            for (int k = 0; k < V; ++k) r.v[k] = T(0);
+            if (i > 0) {
+                const Vec a = g[int64_t(e) - dvec];
+#pragma unroll
+                for (int k = 0; k < V; ++k) r.v[k] += a.v[k];
+            }
+            if (i < len_raw - 1) {
+                const Vec a = g[e];
+#pragma unroll
+                for (int k = 0; k < V; ++k) r.v[k] -= a.v[k];
+            }
+            o[e] = r;
+        }
+    }
+}
+
 // level t (1-based) of coefficient r of a scalar-free signature row, its index w inside the level, the start
 // `lo` and the size of the level
 template <typename I>
