@@ -797,6 +797,21 @@ def test_config5_backward_full_size(P, oracle):
     assert bwd_rel_err(got3, ref) <= 1e-10
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_config4_backward_full_size(P, oracle, dtype):
+    """The lead-lag + time workload at its full size through the backward pass (not a benchmark line: the backward
+    of an augmented path takes the lead-lag-aware sweep and the fold-back onto the raw points)."""
+    c = C.CONFIGS[4]
+    x = C.make_path(4).astype(dtype)
+    aug = dict(time_aug=True, lead_lag=True)
+    sig = oracle.signature(x, c["degree"], n_jobs=-1, **aug)
+    g = np.random.default_rng(2004).standard_normal(sig.shape).astype(dtype)
+    ref = oracle.sig_backprop(x, sig, g, c["degree"], n_jobs=-1, **aug)
+    got = P.sig_backprop(dev(x), dev(sig), dev(g), c["degree"], **aug).cpu().numpy()
+    assert got.shape == x.shape
+    assert bwd_rel_err(got, ref) <= TOL[dtype]
+
+
 def test_stream_ordered_mode(P, oracle):
     """Calls that only enqueue on the null stream: results after one synchronisation equal the synchronous ones,
     also when consecutive calls reuse the library's workspaces with different shapes."""
