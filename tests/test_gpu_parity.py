@@ -477,7 +477,7 @@ def test_reused_buffers_and_repeatability(P, oracle):
                            oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)) <= 1e-10
 
 
-@pytest.mark.parametrize("segments", [1, 2, 3, 5, 8, 13, 32])
+@pytest.mark.parametrize("segments", [1, 2, 3, 5, 6, 7, 8, 11, 13, 32])
 def test_time_segmented_forward(P, oracle, segments):
     """The forward sweep may split paths into time segments folded with Chen's identity; every split must agree."""
     import ctypes
