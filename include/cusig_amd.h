@@ -68,6 +68,22 @@ CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const dou
                                       uint64_t correction_len, uint64_t correction_batch_stride,
                                       uint64_t correction_segment_stride) CUSIG_AMD_NOEXCEPT;
 
+/* sig_backprop_cuda_d for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * sig_backprop_cuda_d without the correction (none is applied), plus the stream (a hipStream_t; null = the null
+ * stream) on which the kernels are enqueued.  The call does not wait: inputs must be ready on that stream, and the
+ * result is ready when the stream reaches the end of the enqueued work.  Every buffer the kernels need beyond the
+ * arguments (increments, increment gradient) lives in a fixed array of cusig_amd_noalloc_scratch_bytes() = 32 MiB
+ * inside the library, one copy per GPU, held until the process ends; shapes that need more return status 2 before
+ * anything is launched.  The call makes no hipMalloc / hipFree and uses no allocating library routine; paths are
+ * always swept whole (no time split).  All calls on one GPU share that array: calls whose kernels may overlap on one
+ * GPU (different streams, several threads) race. */
+CUSIG_AMD_API int cusig_amd_sig_backprop_noalloc_d(const double* path, double* out, const double* sig_derivs,
+                                                   const double* sig, uint64_t batch_size, uint64_t dimension,
+                                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                                   double end_time, bool scalar_term, void* stream) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API uint64_t cusig_amd_noalloc_scratch_bytes(void) CUSIG_AMD_NOEXCEPT;
+
 /* Chen product of two signatures per batch item: out = sig1 (x) sig2, all [batch, S(+1)].
  * Replaces: siglib/cusig/cu_sig_combine.cu:157-169 (decl siglib/cusig/cusig.h:364-365),
  * bound by pysiglib/load_siglib.py:450-454, called from pysiglib/sig.py:113-121. */

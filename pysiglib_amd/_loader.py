@@ -67,6 +67,16 @@ CUSIG_SIG_BACKPROP = _table("sig_backprop_cuda", lambda r: (
     c_bool, POINTER(r), c_uint64, c_uint64, c_uint64))
 
 
+# the variant of sig_backprop_cuda_d that allocates nothing (float64 only): same arguments without the correction,
+# plus the stream to enqueue on
+CUSIG_SIG_BACKPROP_NOALLOC = CUSIG.cusig_amd_sig_backprop_noalloc_d
+CUSIG_SIG_BACKPROP_NOALLOC.argtypes = (
+    POINTER(c_double), POINTER(c_double), POINTER(c_double), POINTER(c_double), c_uint64, c_uint64, c_uint64, c_uint64,
+    c_bool, c_bool, c_double, c_bool, ctypes.c_void_p)
+CUSIG_SIG_BACKPROP_NOALLOC.restype = c_int
+CUSIG.cusig_amd_noalloc_scratch_bytes.argtypes = ()
+CUSIG.cusig_amd_noalloc_scratch_bytes.restype = c_uint64
+
 CUSIG_SIG_COMBINE = _table("sig_combine_cuda", lambda r: (
     POINTER(r), POINTER(r), POINTER(r), c_uint64, c_uint64, c_uint64, c_bool))
 

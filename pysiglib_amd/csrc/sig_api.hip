@@ -243,7 +243,7 @@ static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
 struct MainKernelTimer {
     hipStream_t s;
     bool on;
-    MainKernelTimer(hipStream_t stream, const char* name) : s(stream), on(g_profile)
+    MainKernelTimer(hipStream_t stream, const char* name, bool allowed = true) : s(stream), on(g_profile && allowed)
     {
         if (!on) return;
         if (!g_ev0) {
@@ -741,11 +741,29 @@ static void launch_path_grad(const T* dzinc, T* out, uint64_t batch, uint64_t le
     });
 }
 
+// A caller-independent block of device memory that a call carves its buffers out of instead of the workspace pool
+// (the entry point that must not allocate).  With an arena the call only enqueues on `stream`: no waits, no events,
+// whole-path sweeps only (a time split would need buffers of several signature sets).
+struct Arena {
+    char* base = nullptr;
+    size_t bytes = 0, used = 0;
+    hipStream_t stream = nullptr;
+    void* take(size_t n)
+    {
+        const size_t off = (used + 255) & ~size_t(255);
+        if (off > bytes || n > bytes - off)
+            throw std::invalid_argument("this shape needs more than the " + std::to_string(bytes >> 20) +
+                                        " MiB of built-in scratch memory; use sig_backprop_cuda_d");
+        used = off + n;
+        return base + off;
+    }
+};
+
 template <typename T>
 static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const T* sig, uint64_t batch,
                               uint64_t dimension, uint64_t length, uint64_t degree, bool time_aug,
                               bool lead_lag, T end_time, bool scalar_term, const T* correction,
-                              uint64_t correction_len)
+                              uint64_t correction_len, Arena* arena = nullptr)
 {
     if (dimension == 0) throw std::invalid_argument("sig_backprop_cuda received path of dimension 0");
     validate_correction(correction, correction_len, dimension, degree, lead_lag);
@@ -754,9 +772,13 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         throw std::invalid_argument("sig_backprop_cuda: shape out of range");
     const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
     const uint64_t out_elems = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
-    hipStream_t stream = nullptr;
-    entry_sync();
+    hipStream_t stream = arena ? arena->stream : nullptr;
+    if (!arena) entry_sync();
     const int sc = scalar_term ? 1 : 0;
+    // library buffers: the grow-only pool (under its mutex), or the caller-independent arena
+    auto buffer = [&](int slot, uint64_t bytes) -> void* { return arena ? arena->take(bytes) : workspace(slot, bytes); };
+    auto finish = [&] { if (!arena) exit_sync(stream); };
+    std::unique_lock<std::mutex> lk(g_ws_mutex, std::defer_lock);
 
     if (s.len_aug <= 1 || degree == 0) {
         if (out_elems)
@@ -767,24 +789,25 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                            sig_derivs, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), sc);
     } else if (use_degree2(true, s.d_aug, degree, batch)) {
-        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        if (!arena) lk.lock();
         const int d = int(s.d_aug);
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
-        T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
-        T* h = static_cast<T*>(workspace(12, checked_mul(checked_mul(batch, s.d_aug, "increments"), sizeof(T), "increments")));
-        const T time_step = end_time / T(s.len_aug - 1);
-        hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug)), dim3(kBlock), 0, stream, path, sig_derivs, h,
-                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
-                           int64_t(s.stride), sc);
+        T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
+        T* h = static_cast<T*>(buffer(12, checked_mul(checked_mul(batch, s.d_aug, "increments"), sizeof(T), "increments")));
         const int tiles = (d + 15) / 16, col_groups = (tiles + kDeg2Cols - 1) / kDeg2Cols;
         // operands staged through LDS when a block's four waves all have 16 steps to work on and the channels fill the
         // 64-wide slabs (measured: d = 64, 256 1.6-1.75x faster staged, d = 100 equal, d <= 32 up to 2.5x slower)
         const bool staged = g_degree2_staged != 0 && tiles >= kWavesPerBlock && s.L >= 48;
+        T* anti = staged ? static_cast<T*>(buffer(13, checked_mul(checked_mul(batch, s.d_aug * s.d_aug, "level-2 gradient"), sizeof(T),
+                                                                  "level-2 gradient")))
+                         : nullptr;
+        const T time_step = end_time / T(s.len_aug - 1);
+        hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug)), dim3(kBlock), 0, stream, path, sig_derivs, h,
+                           int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
+                           int64_t(s.stride), sc);
         MainKernelTimer timer(stream, sizeof(T) == 8 ? (staged ? "degree2_bwd_f64_lds" : "degree2_bwd_f64")
-                                                     : (staged ? "degree2_bwd_f32_lds" : "degree2_bwd_f32"));
+                                                     : (staged ? "degree2_bwd_f32_lds" : "degree2_bwd_f32"), !arena);
         if (staged) {
-            T* anti = static_cast<T*>(workspace(13, checked_mul(checked_mul(batch, s.d_aug * s.d_aug, "level-2 gradient"), sizeof(T),
-                                                                "level-2 gradient")));
             hipLaunchKernelGGL((degree2_anti_kernel<T>), dim3(grid_for(batch * s.d_aug * s.d_aug)), dim3(kBlock), 0, stream,
                                sig_derivs, anti, int64_t(batch), d, int64_t(s.stride), sc);
             const int64_t time_groups = (int64_t(s.L) + kDeg2Slab - 1) / kDeg2Slab;
@@ -806,19 +829,19 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         timer.stop();
         launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
         SIG_HIP(hipGetLastError());
-        exit_sync(stream);      // the workspaces stay locked until the kernels are done
+        finish();      // the workspaces stay locked until the kernels are done
         return;
     } else {
         const KernelEntry* e = choose_entry(true, sizeof(T) == 8, s.d_aug, degree, batch, s.L);
         if (!e)
             throw std::runtime_error("sig_backprop_cuda: no kernel for dimension " + std::to_string(s.d_aug) +
                                      ", degree " + std::to_string(degree) + " in this build");
-        std::lock_guard<std::mutex> lk(g_ws_mutex);
+        if (!arena) lk.lock();
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
         const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;
-        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
-        T* dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
+        T* inc = static_cast<T*>(buffer(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
+        T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
         // one launch writes the increments and clears the increment-gradient accumulator (dz_elems <= increment elements)
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
         BwdParams p;
@@ -830,7 +853,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         // lead-lag sweeps that skip the letters a step cannot move read a step's parity off its position in the
         // segment: segments start on even steps (a lead-lag path has an even number of steps)
         const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
-        int nseg = (!ef || degree > uint64_t(kCombMaxLevels)) ? 1
+        int nseg = (arena || !ef || degree > uint64_t(kCombMaxLevels)) ? 1
                    : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
                                               : choose_bwd_segments(
                                                     total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
@@ -853,10 +876,10 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             // at each segment's end), from the right (what follows each segment), and the adjoints of the states
             const uint64_t rows = checked_mul(batch, uint64_t(nseg), "segment signatures");
             const uint64_t bytes = checked_mul(checked_mul(rows, n_coef, "segment signatures"), sizeof(T), "segment signatures");
-            T* segs = static_cast<T*>(workspace(2, bytes));
-            T* left = static_cast<T*>(workspace(8, bytes));
-            T* right = static_cast<T*>(workspace(9, bytes));
-            T* adj = static_cast<T*>(workspace(10, bytes));
+            T* segs = static_cast<T*>(buffer(2, bytes));
+            T* left = static_cast<T*>(buffer(8, bytes));
+            T* right = static_cast<T*>(buffer(9, bytes));
+            T* adj = static_cast<T*>(buffer(10, bytes));
             const int64_t n = int64_t(n_coef);
             FwdParams f;
             f.inc = inc; f.batch = int64_t(rows); f.L = int64_t(s.L); f.d = int(s.d_aug); f.stream = stream;
@@ -867,7 +890,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             // both scans by doubling: ceil(log2(nseg)) launches, ping-ponging between two scratch copies
             int steps = 0;
             while ((1 << steps) < nseg) ++steps;
-            T* scratch = steps > 1 ? static_cast<T*>(workspace(11, checked_mul(bytes, steps > 2 ? 4 : 2, "segment signatures")))
+            T* scratch = steps > 1 ? static_cast<T*>(buffer(11, checked_mul(bytes, steps > 2 ? 4 : 2, "segment signatures")))
                                    : nullptr;
             const uint64_t buf = rows * n_coef;
             const T* xsrc = segs;
@@ -902,16 +925,45 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         e = pick_variant(true, e, total_waves(geom, p.batch), sparse_ll);
         const bool use_ll = sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
         const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
-        MainKernelTimer timer(stream, shown.c_str());
+        MainKernelTimer timer(stream, shown.c_str(), !arena);
         SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
         timer.stop();
         launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
         SIG_HIP(hipGetLastError());
-        exit_sync(stream);
+        finish();
         return;
     }
     SIG_HIP(hipGetLastError());
-    exit_sync(stream);
+    finish();
+}
+
+// ---------------------------------------------------------------------------
+// built-in scratch memory of the entry point that allocates nothing
+// ---------------------------------------------------------------------------
+constexpr size_t kScratchBytes = size_t(32) << 20;
+}  // namespace sigamd
+
+// Every GPU the library runs on holds its own copy of this array (at its own address) until the process ends.  In
+// host code the name is only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+static __device__ __align__(256) unsigned char scratch[sigamd::kScratchBytes];
+
+namespace sigamd {
+
+static std::mutex g_scratch_mutex;
+static std::map<int, void*> g_scratch_ptr;      // device -> address of that device's copy of `scratch`
+
+static void* scratch_of_current_device()
+{
+    int dev = 0;
+    SIG_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    auto it = g_scratch_ptr.find(dev);
+    if (it != g_scratch_ptr.end()) return it->second;
+    void* ptr = nullptr;
+    SIG_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) throw std::runtime_error("built-in scratch memory has no device address");
+    g_scratch_ptr[dev] = ptr;
+    return ptr;
 }
 
 }  // namespace sigamd
@@ -965,6 +1017,23 @@ CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const dou
                                   lead_lag, end_time, scalar_term, correction, correction_len);
     });
 }
+
+CUSIG_AMD_API int cusig_amd_sig_backprop_noalloc_d(const double* path, double* out, const double* sig_derivs,
+                                                   const double* sig, uint64_t batch_size, uint64_t dimension,
+                                                   uint64_t length, uint64_t degree, bool time_aug, bool lead_lag,
+                                                   double end_time, bool scalar_term, void* stream) noexcept
+{
+    return guarded([&] {
+        Arena arena;
+        arena.base = static_cast<char*>(scratch_of_current_device());
+        arena.bytes = kScratchBytes;
+        arena.stream = static_cast<hipStream_t>(stream);
+        sig_backprop_impl<double>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug, lead_lag,
+                                  end_time, scalar_term, nullptr, 0, &arena);
+    });
+}
+
+CUSIG_AMD_API uint64_t cusig_amd_noalloc_scratch_bytes(void) noexcept { return kScratchBytes; }
 
 CUSIG_AMD_API const char* cusig_last_error_message(void) noexcept { return g_last_error; }
 
