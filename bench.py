@@ -4,12 +4,17 @@ A "step" is one forward + one backward pass of the headline workload
 (batch 32, length 1000, dimension 10, degree 5, float64; path points iid N(0,1))
 through the library's C ABI with all buffers resident in HBM.  Prints ONE JSON line.
 
+Order of a run: every other leg first (configs 2-4, the degree-2 case, stream-ordered mode, per-kernel timings), then the
+headline: W untimed warm-up steps, K timed steps, each step timed on its own (both calls are synchronous).
+`ms_per_step` is the median step, `ms_per_step_mean` the mean over the same K steps; `value` follows the median.
+
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all-configs]
 """
 import argparse
 import ctypes
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -72,43 +77,73 @@ class Runner:
             rng = np.random.default_rng(2000 + k)
             self.gsig = torch.tensor(rng.standard_normal((c["batch"], n)).astype(self.dtype), device="cuda:0")
             self.grad = torch.empty_like(self.path)
+        # the argument lists are built once: a call is then one ctypes call
+        self._fwd = loader.CUSIG_SIGNATURE[self.dtype]
+        self._fwd_args = (self._p(self.path), self._p(self.sig), c["batch"], c["dim"], c["length"], c["degree"], c["time_aug"],
+                          c["lead_lag"], 1.0, True, False, None, 0, 0, 0)
+        if c["backward"]:
+            self._bwd = loader.CUSIG_SIG_BACKPROP[self.dtype]
+            self._bwd_args = (self._p(self.path), self._p(self.grad), self._p(self.gsig), self._p(self.sig), c["batch"], c["dim"],
+                              c["length"], c["degree"], c["time_aug"], c["lead_lag"], 1.0, False, None, 0, 0, 0)
 
     def _p(self, t):
         return ctypes.cast(t.data_ptr(), ctypes.POINTER(self.real))
 
     def forward(self):
-        c = self.c
-        rc = self.loader.CUSIG_SIGNATURE[self.dtype](
-            self._p(self.path), self._p(self.sig), c["batch"], c["dim"], c["length"], c["degree"], c["time_aug"],
-            c["lead_lag"], 1.0, True, False, None, 0, 0, 0)
+        rc = self._fwd(*self._fwd_args)
         if rc:
             raise RuntimeError("signature_cuda failed: %d %s" % (rc, self.loader.last_error_message()))
 
     def backward(self):
-        c = self.c
-        rc = self.loader.CUSIG_SIG_BACKPROP[self.dtype](
-            self._p(self.path), self._p(self.grad), self._p(self.gsig), self._p(self.sig), c["batch"], c["dim"],
-            c["length"], c["degree"], c["time_aug"], c["lead_lag"], 1.0, False, None, 0, 0, 0)
+        rc = self._bwd(*self._bwd_args)
         if rc:
             raise RuntimeError("sig_backprop_cuda failed: %d %s" % (rc, self.loader.last_error_message()))
 
 
 def time_calls(fn, torch, loader, warmup, steps):
-    """Returns (wall seconds per call, mean sweep-kernel ms, kernel name)."""
+    """Returns (median wall seconds per call, mean sweep-kernel ms, kernel name)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     loader.CUSIG.cusig_amd_set_profiling(1)
-    kms = []
-    t0 = time.perf_counter()
+    kms, walls = [], []
     for _ in range(steps):
+        t0 = time.perf_counter()
         fn()
+        walls.append(time.perf_counter() - t0)
         kms.append(float(loader.CUSIG.cusig_amd_last_kernel_ms()))
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / steps
     name = loader.CUSIG.cusig_amd_last_kernel_name().decode()
     loader.CUSIG.cusig_amd_set_profiling(0)
-    return wall, sum(kms) / len(kms), name
+    return statistics.median(walls), sum(kms) / len(kms), name
+
+
+def time_steps(step, torch, warmup, steps):
+    """W untimed warm-up steps, then K steps timed one by one between two device synchronisations.
+    Returns (median ms, mean ms)."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t_all = time.perf_counter()
+    each = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        step()
+        each.append(time.perf_counter() - t0)
+    torch.cuda.synchronize()
+    mean_ms = (time.perf_counter() - t_all) / steps * 1e3
+    return statistics.median(each) * 1e3, mean_ms
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(np, cfgmod):
@@ -116,7 +151,12 @@ def cpu_baseline(np, cfgmod):
     from oracle import sigref
     x = cfgmod.make_path(1)
     c = cfgmod.CONFIGS[1]
-    threads = min(sigref.max_threads(), 16)
+    # one path per thread (the reference's chunking): at most `batch` threads do work.  A process that is given a
+    # CPU share smaller than the machine (OMP_NUM_THREADS says so) uses that share.
+    threads = min(sigref.max_threads(), c["batch"])
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    if share.isdigit() and int(share) > 0:
+        threads = min(threads, int(share))
     rng = np.random.default_rng(2005)
     best = None
     sig = None
@@ -134,14 +174,15 @@ def cpu_baseline(np, cfgmod):
         dt = (t1 - t0) + (t3 - t2)
         best = dt if best is None else min(best, dt)
     return {"value": c["batch"] / best, "unit": "signatures/s (fwd+bwd)", "cores": threads, "kind": "port",
+            "os_cpu_count": os.cpu_count(), "hardware_threads": sigref.max_threads(), "cpu_model": cpu_model(),
             "sample": "full headline workload (32 paths x 999 steps, d=10, degree 5, f64), best of %d, "
-                      "oracle/sigref.c -O3 -march=native, one path per thread" % reps}
+                      "oracle/sigref.c -O3 -march=native, one path per thread on %d threads (the process's CPU share)"
+                      % (reps, threads)}
 
 
 def bench_ops(args, torch, loader):
     """Operators either side of the sweep: HBM-bound element-wise kernels.  Achieved GB/s = algorithmic bytes (every
     input read once, every output written once) / wall time of the synchronous C-ABI call."""
-    import statistics
     real = loader.DTYPES["float64"]
     d, deg, batch = 10, 5, 1024
     n = int(loader.CUSIG.cusig_amd_sig_length(d, deg)) - 1
@@ -221,7 +262,7 @@ def main():
     import torch
 
     from pysiglib_amd import _loader as loader
-    from tests import _configs as cfgmod
+    from pysiglib_amd import workloads as cfgmod
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -246,53 +287,10 @@ def main():
     r5 = Runner(5, torch, np, loader, cfgmod)
     r5.forward()            # the backward consumes the forward's signature
     torch.cuda.synchronize()
-
-    def step():
-        r1.forward()
-        r5.backward()
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
-    value = r1.c["batch"] / (ms_per_step * 1e-3)
-
-    # the same steps with the library in stream-ordered mode: calls only enqueue, the host syncs once at the end
-    loader.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
-    loader.CUSIG.cusig_amd_set_stream_ordered.restype = None
-    loader.CUSIG.cusig_amd_set_stream_ordered(1)
-    try:
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        ordered_ms = (time.perf_counter() - t0) / args.steps * 1e3
-    finally:
-        loader.CUSIG.cusig_amd_set_stream_ordered(0)
-        torch.cuda.synchronize()
-
-    # per-kernel figures (HIP events inside the library, on the launch stream)
-    wall_f, kms_f, name_f = time_calls(r1.forward, torch, loader, 1, max(5, args.steps))
-    wall_b, kms_b, name_b = time_calls(r5.backward, torch, loader, 1, max(5, args.steps))
-    tf_f = r1.flops_fwd / (kms_f * 1e-3) / 1e12
-    tf_b = r5.flops_bwd / (kms_b * 1e-3) / 1e12
     peak = PEAK_TFLOPS["float64"]
-    dominant = {"kernel": name_b, "ms": kms_b, "tflops": tf_b} if kms_b >= kms_f else {"kernel": name_f, "ms": kms_f, "tflops": tf_f}
+    configs = {}
 
-    configs = {
-        "C1": {"signatures_per_s": r1.c["batch"] / wall_f, "call_ms": wall_f * 1e3, "kernel": name_f,
-               "kernel_ms": kms_f, "tflops": tf_f, "roofline_frac": tf_f / peak},
-        "C5": {"signatures_per_s": r5.c["batch"] / wall_b, "call_ms": wall_b * 1e3, "kernel": name_b,
-               "kernel_ms": kms_b, "tflops": tf_b, "roofline_frac": tf_b / peak},
-    }
-    if not args.headline_only:      # all five workloads by default (a few seconds more)
+    if not args.headline_only:      # all five workloads by default (a few seconds more); the headline comes last
         for k in (2, 3, 4):
             r = Runner(k, torch, np, loader, cfgmod)
             n = 3 if k == 3 else max(5, min(args.steps, 50))
@@ -332,6 +330,47 @@ def main():
             configs[tag] = {"signatures_per_s": db / wall, "call_ms": wall * 1e3, "kernel": name, "kernel_ms": kms,
                             "tflops": mm_flops / (kms * 1e-3) / 1e12, "bound": "mfma",
                             "roofline_frac": mm_flops / (kms * 1e-3) / 1e12 / PEAK_TFLOPS["float32"]}
+        del xp, sg, gg, gx
+        torch.cuda.empty_cache()
+
+    def step():
+        r1.forward()
+        r5.backward()
+
+    # the same steps with the library in stream-ordered mode: calls only enqueue, the host syncs once at the end
+    loader.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
+    loader.CUSIG.cusig_amd_set_stream_ordered.restype = None
+    loader.CUSIG.cusig_amd_set_stream_ordered(1)
+    try:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ordered_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    finally:
+        loader.CUSIG.cusig_amd_set_stream_ordered(0)
+        torch.cuda.synchronize()
+
+    # per-kernel figures (HIP events inside the library, on the launch stream)
+    wall_f, kms_f, name_f = time_calls(r1.forward, torch, loader, 1, max(5, args.steps))
+    wall_b, kms_b, name_b = time_calls(r5.backward, torch, loader, 1, max(5, args.steps))
+    tf_f = r1.flops_fwd / (kms_f * 1e-3) / 1e12
+    tf_b = r5.flops_bwd / (kms_b * 1e-3) / 1e12
+    # the headline comes last, after every other leg of this run, so that it is timed on a device in steady state
+    ms_per_step, ms_mean = time_steps(step, torch, args.warmup, args.steps)
+    value = r1.c["batch"] / (ms_per_step * 1e-3)
+    dominant = {"kernel": name_b, "ms": kms_b, "tflops": tf_b} if kms_b >= kms_f else {"kernel": name_f, "ms": kms_f, "tflops": tf_f}
+    headline = {
+        "C1": {"signatures_per_s": r1.c["batch"] / wall_f, "call_ms": wall_f * 1e3, "kernel": name_f,
+               "kernel_ms": kms_f, "tflops": tf_f, "roofline_frac": tf_f / peak},
+        "C5": {"signatures_per_s": r5.c["batch"] / wall_b, "call_ms": wall_b * 1e3, "kernel": name_b,
+               "kernel_ms": kms_b, "tflops": tf_b, "roofline_frac": tf_b / peak},
+    }
+    headline.update(configs)
+    configs = headline
 
     line = {
         "metric": "signatures/sec, (32,1000,10) deg 5 fwd+bwd, fp64, 1 GPU",
@@ -341,6 +380,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_mean": ms_mean,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -349,11 +389,13 @@ def main():
         "config": {"workload": "sig forward + sig_backprop, batch 32, length 1000, dim 10, degree 5, float64, "
                                "points iid N(0,1) seed 1001; upstream grad iid N(0,1)"},
         "roofline": {
-            "bound": "mfma", "pipe": "vector FP64 FMA (rank-1 updates: no MFMA tile applies; same 78.6 TFLOP/s peak)",
+            "bound": "vector_fp64", "pipe": "vector FP64 FMA (per-path rank-1 updates and GEMVs: no MFMA tile applies)",
             "kernel": dominant["kernel"], "achieved": dominant["tflops"], "peak": peak, "unit": "TFLOP/s",
             "frac": dominant["tflops"] / peak, "kernel_ms": dominant["ms"],
             "traffic": TRAFFIC_BYTES.get(dominant["kernel"]),
             "fwd_bwd_combined_frac": (r1.flops_fwd + r5.flops_bwd) / ((kms_f + kms_b) * 1e-3) / 1e12 / peak,
+            # the whole synchronous step as timed above (launches and host waits included)
+            "step_frac": (r1.flops_fwd + r5.flops_bwd) / (ms_per_step * 1e-3) / 1e12 / peak,
         },
         "configs": configs,
         "stream_ordered": {"value": r1.c["batch"] / (ordered_ms * 1e-3), "ms_per_step": ordered_ms,

@@ -263,6 +263,9 @@ CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: the closed-form degree-2 kernels (matrix cores): -1 automatic, 0 never, 1 whenever the degree is 2. */
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) CUSIG_AMD_NOEXCEPT;
+/* Test hook: 1 routes every sweep of 2, 3 or 4 augmented channels that the run-time-degree kernels can serve
+ * (degree >= 5, 4, 3 respectively) to them; by default they only serve degrees 17 .. 64. */
+CUSIG_AMD_API void cusig_amd_force_deep(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: 0 makes the degree-2 kernels build their operands straight from global memory instead of staging
  * them through LDS (the path taken anyway when a chunk of all channels does not fit). */
 CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) CUSIG_AMD_NOEXCEPT;

@@ -217,10 +217,10 @@ def main():
                                  "int64_t, int, int64_t, int, int, int64_t, int*, int);" % (T, D, N, tail, K, lead_lag_mode(D, zl), T, T))
             else:
                 lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s>(const %s*, const %s*, "
-                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);" % (T, D, N, tail, K, zs, T, T, T, T))
+                             "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t, int);" % (T, D, N, tail, K, zs, T, T, T, T))
                 if lead_lag_mode_bwd(T, D, tail, zl):
                     lines.append("template __global__ void tree_bwd_kernel<%s, %d, %d, %d, %d, %s, %d>(const %s*, const %s*, "
-                                 "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t);"
+                                 "const %s*, %s*, int64_t, int64_t, int, int64_t, int, int, int, int64_t, int);"
                                  % (T, D, N, tail, K, zs, lead_lag_mode_bwd(T, D, tail, zl), T, T, T, T))
         lines.append("")
         lines.append("#if !defined(__HIP_DEVICE_COMPILE__)   // the launcher table is host data")

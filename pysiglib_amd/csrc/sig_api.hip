@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <charconv>
 #include <cstdio>
 #include <cstring>
@@ -22,6 +23,7 @@
 
 #include "../../include/cusig_amd.h"
 #include "sig_chen_adjoint.h"
+#include "sig_deep.h"
 #include "sig_degree2.h"
 #include "sig_host.h"
 #include "sig_kernels.h"
@@ -52,9 +54,12 @@ struct Table {
     }
 };
 
+// Process-wide hooks (tuning, tests, measurement) may be set by one thread while another is inside a call: atomics,
+// read once where a call needs a consistent value.
+using Hook = std::atomic<int>;
 // tuning hook: when set (tail > 0), prefer the compiled partition with this (tail, k)
-static int g_force_tail = 0, g_force_k = 0;
-static int g_force_run_time_wide = 0;   // with a forced partition: take the run-time-dimension kernel in the wide layout
+static Hook g_force_tail{0}, g_force_k{0};
+static Hook g_force_run_time_wide{0};   // with a forced partition: take the run-time-dimension kernel in the wide layout
 
 static const Table& table()
 {
@@ -184,7 +189,7 @@ struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
 };
-int g_force_wide_index = 0;
+std::atomic<int> g_force_wide_index{0};
 std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
@@ -199,7 +204,7 @@ void* workspace(int slot, size_t bytes)
             w.ptr = nullptr;
             w.bytes = 0;
         }
-        const size_t want = bytes + bytes / 8;
+        const size_t want = (bytes + bytes / 8 + 255) & ~size_t(255);
         if (hipMalloc(&w.ptr, want) != hipSuccess) {
             (void)hipGetLastError();
             w.ptr = nullptr;
@@ -208,6 +213,34 @@ void* workspace(int slot, size_t bytes)
         w.bytes = want;
     }
     return w.ptr;
+}
+
+// The increment-gradient accumulators of backward sweeps that form their own increments (no pre-pass launch that could
+// clear one): two buffers per device take turns.  The launch that turns a call's accumulator into the path gradient also
+// clears whatever the other buffer still holds, so the next call finds its accumulator zero.  `dirty` counts the leading
+// bytes that may be non-zero (everything after an allocation; a failed call leaves its buffer dirty and `next`
+// unchanged, and the next call clears it with a launch of its own).  Guarded by the workspace mutex.
+struct DzPair {
+    void* ptr[2] = {nullptr, nullptr};
+    size_t capacity[2] = {0, 0};
+    size_t dirty[2] = {0, 0};
+    int next = 0;
+};
+static std::map<int, DzPair> g_dz;      // per device
+constexpr int kDzSlot[2] = {16, 17};
+
+static void* dz_pair_buffer(DzPair& st, int which, size_t bytes)
+{
+    int dev = 0;
+    SIG_HIP(hipGetDevice(&dev));
+    void* p = workspace(kDzSlot[which], bytes);
+    const size_t capacity = g_ws[{dev, kDzSlot[which]}].bytes;
+    if (p != st.ptr[which] || capacity != st.capacity[which]) {     // fresh memory: all of it may be non-zero
+        st.ptr[which] = p;
+        st.capacity[which] = capacity;
+        st.dirty[which] = capacity;
+    }
+    return p;
 }
 
 static int* g_flag_host = nullptr;     // pinned word the forward kernels report NaN / infinity through
@@ -225,6 +258,7 @@ static void release_workspaces() noexcept
         }
     }
     g_ws.clear();
+    g_dz.clear();
     if (g_flag_host) {
         (void)hipHostFree(g_flag_host);
         g_flag_host = nullptr;
@@ -235,8 +269,9 @@ static void release_workspaces() noexcept
 // ---------------------------------------------------------------------------
 // kernel timing hook for the benchmark
 // ---------------------------------------------------------------------------
-static bool g_profile = false;
-static float g_last_ms = -1.f;
+static std::atomic<bool> g_profile{false};
+static std::atomic<float> g_last_ms{-1.f};
+// name and events are only touched under the workspace mutex (every timer lives inside a locked region)
 static char g_last_name[128] = {0};
 static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
 
@@ -265,7 +300,9 @@ struct MainKernelTimer {
     {
         if (!on) return;
         SIG_HIP(hipEventSynchronize(g_ev1));
-        SIG_HIP(hipEventElapsedTime(&g_last_ms, g_ev0, g_ev1));
+        float ms = -1.f;
+        SIG_HIP(hipEventElapsedTime(&ms, g_ev0, g_ev1));
+        g_last_ms = ms;
     }
 };
 
@@ -273,7 +310,7 @@ struct MainKernelTimer {
 // stream and return; neither the device-wide wait on entry nor the wait for completion is made.  Correct for callers
 // whose producers and consumers are ordered with the null stream (PyTorch's default stream is the null stream, and
 // blocking streams synchronise with it implicitly); it removes the host round trip between consecutive calls.
-static int g_stream_ordered = 0;
+static Hook g_stream_ordered{0};
 static void entry_sync()
 {
     if (!g_stream_ordered) SIG_HIP(hipDeviceSynchronize());
@@ -303,10 +340,10 @@ static int* nonfinite_flag()
 // ---------------------------------------------------------------------------
 // time segmentation of the forward sweep
 // ---------------------------------------------------------------------------
-static int g_force_segments = 0;   // tuning hook (0 = automatic)
+static Hook g_force_segments{0};   // tuning hook (0 = automatic)
 static thread_local int tl_last_segments = 0;   // pieces per path of the last forward sweep on this thread (0: no sweep ran)
-static int g_point_fed = 1;        // tuning hook: 0 always computes the increments in a kernel of their own
-static int g_lead_lag_sparse = 1;  // tuning hook: 0 sweeps lead-lag paths like any other (every letter of every step)
+static Hook g_point_fed{1};        // tuning hook: 0 always computes the increments in a kernel of their own
+static Hook g_lead_lag_sparse{1};  // tuning hook: 0 sweeps lead-lag paths like any other (every letter of every step)
 
 static int simd_count()
 {
@@ -370,7 +407,7 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
 // segment signatures up to g, and the adjoint of that state is the upstream gradient pulled back through the product
 // with the remaining segments.  That costs a segmented forward sweep, two chains of Chen products and one product
 // adjoint, all over (path, segment) rows.
-static int g_force_bwd_segments = 0;   // tuning hook (0 = automatic)
+static Hook g_force_bwd_segments{0};   // tuning hook (0 = automatic)
 
 // g pieces are chosen by the same kind of model as for the forward sweep (fullest SIMD, `pair_rate`, lane_step(g) =
 // seconds per step of a lone wave).  The extra work is larger here: the segmented forward sweep (a third of the
@@ -417,7 +454,7 @@ static int choose_bwd_segments(int64_t waves, int64_t L, int waves_per_simd, uin
 // degrees 4..6, 3-9 waves per SIMD): the f32 forward is always faster staged (1.2-1.8x: SGPR-operand FMAs issue
 // slower than all-VGPR ones), the f32 backward up to 13 channels and both f64 sweeps up to 8 (1.05-1.3x), while with
 // more channels the ring's LDS reads cost them 3-30 % (f64 at 10-12 channels is mixed).
-static int g_force_staged = -1;   // tuning hook: -1 automatic, 0 never, 1 whenever compiled
+static Hook g_force_staged{-1};   // tuning hook: -1 automatic, 0 never, 1 whenever compiled
 
 // lead_lag_sparse: the path is a lead-lag path and staged twins that skip a step's still letters may be used.  Those
 // twins do about 40 % less arithmetic, which outweighs what the tuned choice for dense paths says: measured on 144
@@ -447,8 +484,8 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
 // ---------------------------------------------------------------------------
 // degree 2 in closed form (matrix cores): taken for paths of many channels, where no specialised sweep exists
 // ---------------------------------------------------------------------------
-static int g_force_degree2 = -1;    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
-static int g_degree2_staged = 1;    // tuning hook: 0 keeps the operands of the degree-2 products out of LDS
+static Hook g_force_degree2{-1};    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
+static Hook g_degree2_staged{1};    // tuning hook: 0 keeps the operands of the degree-2 products out of LDS
 
 // Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
 // forward from about 12 channels on and for small dimensions whenever the sweeps cannot fill the chip.
@@ -457,6 +494,24 @@ static bool use_degree2(bool backward, uint64_t d_aug, uint64_t degree, uint64_t
     if (degree != 2 || d_aug < 2 || d_aug > 0x7fff) return false;
     if (g_force_degree2 >= 0) return g_force_degree2 != 0;
     return backward || d_aug >= 12 || batch * 8 <= uint64_t(simd_count());
+}
+
+// ---------------------------------------------------------------------------
+// degrees beyond the instance table: run-time-degree sweeps (sig_deep.hip)
+// ---------------------------------------------------------------------------
+static Hook g_force_deep{0};        // test hook: 1 takes the run-time-degree sweeps wherever they apply
+
+static bool use_deep(uint64_t d_aug, uint64_t degree)
+{
+    if (!deep_supported(d_aug, degree)) return false;
+    return degree > 16 || g_force_deep != 0;
+}
+
+// the reference's run-time-degree kernels stop at degree 64 (siglib/cusig/cu_signature.cu:400,3022-3025)
+static void check_degree_limit(uint64_t d_aug, uint64_t degree, const char* who)
+{
+    if (d_aug >= 2 && degree > uint64_t(kDeepMaxDegree))
+        throw std::invalid_argument(std::string(who) + " requires degree <= 64. Use CPU or reduce the truncation level.");
 }
 
 // ---------------------------------------------------------------------------
@@ -532,6 +587,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
     if (dimension > 0x3fffffff || degree > 0x7fffffff || length > (uint64_t(1) << 40))
         throw std::invalid_argument("signature_cuda: shape out of range");
     const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
+    check_degree_limit(s.d_aug, degree, "signature on this GPU build");
     checked_mul(checked_mul(batch, s.stride, "signature output"), sizeof(T), "signature output");
     hipStream_t stream = nullptr;
     entry_sync();   // inputs may have been produced on any stream
@@ -607,6 +663,18 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         if (slices > 1 && flag)
             hipLaunchKernelGGL((finite_rows_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
                                int64_t(batch * s.stride), flag);
+    } else if (use_deep(s.d_aug, degree)) {
+        if (!deep_fits(s.d_aug, degree, batch)) throw std::runtime_error("signature_cuda: launch too large");
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+        FwdParams p;
+        p.inc = inc; p.out = out; p.batch = int64_t(batch); p.L = int64_t(s.L); p.d = int(s.d_aug); p.out_stride = int64_t(s.stride);
+        p.scalar = sc; p.stream = stream; p.nseg = 1; p.lseg = int64_t(s.L); p.nonfinite = flag;
+        tl_last_segments = 1;
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? "deep_fwd_f64" : "deep_fwd_f32");
+        SIG_HIP(launch_deep_fwd<T>(p, int(degree)));
+        timer.stop();
     } else {
         const KernelEntry* e = choose_entry(false, sizeof(T) == 8, s.d_aug, degree, batch, s.L);
         if (!e)
@@ -721,7 +789,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
 // increment gradient -> raw path gradient; plain paths with a channel count that allows it take 16 bytes per lane
 template <typename T>
 static void launch_path_grad(const T* dzinc, T* out, uint64_t batch, uint64_t length, uint64_t dimension, bool time_aug,
-                             bool lead_lag, hipStream_t stream)
+                             bool lead_lag, hipStream_t stream, T* clear = nullptr, uint64_t clear_count = 0)
 {
     constexpr int V = int(16 / sizeof(T));
     if (!time_aug && !lead_lag && dimension % V == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
@@ -730,14 +798,14 @@ static void launch_path_grad(const T* dzinc, T* out, uint64_t batch, uint64_t le
         launch_indexed(per, per, batch, [&](auto ix, dim3 grid) {
             using I = decltype(ix);
             hipLaunchKernelGGL((path_grad_vec_kernel<T, I, V>), grid, dim3(kBlock), 0, stream, dzinc, out, int64_t(batch),
-                               int64_t(length), DivBy<I>(dimension / V));
+                               int64_t(length), DivBy<I>(dimension / V), clear, int64_t(clear_count));
         });
         return;
     }
     launch_indexed(length * dimension, (length * dimension + 1) / 2, batch, [&](auto ix, dim3 grid) {
         using I = decltype(ix);
         hipLaunchKernelGGL((path_grad_kernel<T, I>), grid, dim3(kBlock), 0, stream, dzinc, out, int64_t(batch),
-                           int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension));
+                           int64_t(length), int(time_aug), int(lead_lag), DivBy<I>(dimension), clear, int64_t(clear_count));
     });
 }
 
@@ -771,6 +839,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
     if (dimension > 0x3fffffff || degree > 0x7fffffff || length > (uint64_t(1) << 40))
         throw std::invalid_argument("sig_backprop_cuda: shape out of range");
     const Shape s = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term);
+    check_degree_limit(s.d_aug, degree, "sig_backprop on this GPU build");
     const uint64_t out_elems = checked_mul(checked_mul(batch, length, "path gradient"), dimension, "path gradient");
     hipStream_t stream = arena ? arena->stream : nullptr;
     if (!arena) entry_sync();
@@ -831,6 +900,24 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         SIG_HIP(hipGetLastError());
         finish();      // the workspaces stay locked until the kernels are done
         return;
+    } else if (use_deep(s.d_aug, degree)) {
+        if (!deep_fits(s.d_aug, degree, batch)) throw std::runtime_error("sig_backprop_cuda: launch too large");
+        if (!arena) lk.lock();
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+        const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        T* inc = static_cast<T*>(buffer(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
+        BwdParams p;
+        p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
+        p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? "deep_bwd_f64" : "deep_bwd_f32", !arena);
+        SIG_HIP(launch_deep_bwd<T>(p, int(degree)));
+        timer.stop();
+        launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
+        SIG_HIP(hipGetLastError());
+        finish();
+        return;
     } else {
         const KernelEntry* e = choose_entry(true, sizeof(T) == 8, s.d_aug, degree, batch, s.L);
         if (!e)
@@ -839,13 +926,10 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         if (!arena) lk.lock();
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+        const uint64_t dz_bytes = checked_mul(dz_elems, sizeof(T), "increments");
         const uint64_t pad = uint64_t(kStageSteps + 2) * s.d_aug;
-        T* inc = static_cast<T*>(buffer(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
-        T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
-        // one launch writes the increments and clears the increment-gradient accumulator (dz_elems <= increment elements)
-        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
         BwdParams p;
-        p.inc = inc; p.sig = sig; p.gsig = sig_derivs; p.dzinc = dzinc; p.batch = int64_t(batch);
+        p.sig = sig; p.gsig = sig_derivs; p.batch = int64_t(batch);
         p.L = int64_t(s.L); p.d = int(s.d_aug); p.sig_stride = int64_t(s.stride); p.scalar = sc; p.stream = stream;
         const TreeGeom geom = make_geom(int(s.d_aug), e->N - e->tail, e->k, e->D != 0);
         const uint64_t n_coef = s.full_len - 1;
@@ -871,6 +955,37 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             if (sparse_ll) lseg += lseg & 1;
             nseg = int((int64_t(s.L) + lseg - 1) / lseg);
         }
+        // Whole-path staged sweeps of plain narrow paths form the increments themselves while staging the points: no
+        // pre-pass launch, so the accumulator comes from the pair that takes turns (cleared by the previous call).
+        const KernelEntry* e_run = pick_variant(true, e, total_waves(geom, int64_t(batch) * nseg), sparse_ll);
+        const bool point_fed = !arena && nseg == 1 && e_run->staged && !time_aug && !lead_lag && e_run->D > 0 &&
+                               e_run->D <= kPointFedMaxDim && g_point_fed != 0;
+        T* inc = nullptr;
+        T* dzinc = nullptr;
+        DzPair* turn = nullptr;
+        int mine = 0;
+        if (point_fed) {
+            int dev = 0;
+            SIG_HIP(hipGetDevice(&dev));
+            turn = &g_dz[dev];
+            mine = turn->next;
+            dzinc = static_cast<T*>(dz_pair_buffer(*turn, mine, dz_bytes));
+            if (turn->dirty[mine]) {        // first use, or a call that failed half-way: clear it here
+                const uint64_t n = (turn->dirty[mine] + sizeof(T) - 1) / sizeof(T);
+                hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(n)), dim3(kBlock), 0, stream, dzinc, int64_t(n));
+                SIG_HIP(hipGetLastError());
+                turn->dirty[mine] = 0;
+            }
+            p.inc = path;
+            p.from_points = 1;
+        } else {
+            inc = static_cast<T*>(buffer(0, checked_mul(inc_elems + 2 * pad, sizeof(T), "increments"))) + pad;
+            dzinc = static_cast<T*>(buffer(1, dz_bytes));
+            // one launch writes the increments and clears the increment-gradient accumulator (dz_elems <= increment elements)
+            compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
+            p.inc = inc;
+        }
+        p.dzinc = dzinc;
         if (nseg > 1) {
             // (path, segment) rows, scalar-free: segment signatures, their running products from the left (the state
             // at each segment's end), from the right (what follows each segment), and the adjoints of the states
@@ -922,14 +1037,26 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             p.sig = left; p.gsig = adj; p.sig_stride = n; p.scalar = 0;
             p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
         }
-        e = pick_variant(true, e, total_waves(geom, p.batch), sparse_ll);
+        e = e_run;
         const bool use_ll = sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
         const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str(), !arena);
+        if (turn) turn->dirty[mine] = dz_bytes;        // from here on the accumulator holds sums
         SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
         timer.stop();
-        launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
-        SIG_HIP(hipGetLastError());
+        if (turn) {
+            // the same launch clears what the other accumulator still holds: it is the next call's
+            const int other = 1 - mine;
+            T* clear = turn->dirty[other] ? static_cast<T*>(turn->ptr[other]) : nullptr;
+            launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream, clear,
+                                (turn->dirty[other] + sizeof(T) - 1) / sizeof(T));
+            SIG_HIP(hipGetLastError());
+            turn->dirty[other] = 0;
+            turn->next = other;
+        } else {
+            launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
+            SIG_HIP(hipGetLastError());
+        }
         finish();
         return;
     }
@@ -1052,7 +1179,13 @@ CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) noexcept { g_profile = e
 
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) noexcept { return g_last_ms; }
 
-CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept { return g_last_name; }
+CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept
+{
+    static thread_local char name[sizeof g_last_name];
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    std::memcpy(name, g_last_name, sizeof name);
+    return name;
+}
 
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
 CUSIG_AMD_API int cusig_amd_last_segments(void) noexcept { return tl_last_segments; }
@@ -1070,6 +1203,8 @@ CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
 
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) noexcept { g_force_degree2 = mode; }
+
+CUSIG_AMD_API void cusig_amd_force_deep(int enabled) noexcept { g_force_deep = enabled; }
 
 CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) noexcept { g_degree2_staged = enabled; }
 

@@ -23,7 +23,7 @@ template <typename T>
 __device__ __forceinline__ T aug_point(const T* __restrict__ x, int64_t t, int c, int d_raw, int time_aug, int lead_lag,
                                        int d, T time_step)
 {
-    if (time_aug && c == d - 1) return T(t) * time_step;
+    if (time_aug && c == d - 1) return mul_rn(T(t), time_step);
     if (!lead_lag) return x[t * d_raw + c];
     return c < d_raw ? x[(t >> 1) * d_raw + c] : x[((t + 1) >> 1) * d_raw + (c - d_raw)];
 }

@@ -1,6 +1,7 @@
 // Kernels of the signature hot path: increment pre-pass, tree forward sweep,
 // tree reverse sweep, increment-gradient fold-back and the closed-form cases.
 #pragma once
+#include <atomic>
 #include <limits>
 
 #include "sig_tree.h"
@@ -82,6 +83,16 @@ struct LaneCtx {
 // NaN or infinity
 __device__ __forceinline__ bool not_finite(double v) { return !(__builtin_fabs(v) <= std::numeric_limits<double>::max()); }
 __device__ __forceinline__ bool not_finite(float v) { return !(__builtin_fabsf(v) <= std::numeric_limits<float>::max()); }
+
+// product rounded on its own: the empty asm hides it from the compiler, which would otherwise contract it into a
+// multiply-add with a neighbouring operation
+template <typename T>
+__device__ __forceinline__ T mul_rn(T a, T b)
+{
+    T p = a * b;
+    asm volatile("" : "+v"(p));
+    return p;
+}
 
 // Nothing may be scheduled across this point: the loads above it are issued
 // before any of the arithmetic below it.
@@ -242,8 +253,8 @@ __device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__
 }
 
 // staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0
-// points (wave-uniform; forward sweeps of plain paths only): `row` is the path point of the first step instead of an
-// increment row, and the ring takes differences of consecutive points.
+// points (wave-uniform; plain paths only): `row` is the path point at which the first step of the sweep starts, instead
+// of that step's increment row, and the ring takes differences of consecutive points.
 // step(increments, step index, IntC<G0>, IntC<position>): position 0 / 1 alternate from the first step of the range on
 // (chunks hold an even number of steps), so a range that starts on an even step hands the step's parity to `step`
 // as a compile-time constant.
@@ -280,9 +291,15 @@ __device__ __forceinline__ void sweep_staged(const Cx& cx, const T* __restrict__
 
     // chunk k holds the elements [k * CHUNK, (k + 1) * CHUNK) of the range; count * D of them exist
     auto issue = [&](int64_t k) {
-        if (DIR > 0 && Ring::kPoints && points) {
-            const int64_t left = count * D - k * Ring::CHUNK;
-            ring.issue_points(chunk_src(k), 0, left < Ring::CHUNK ? int(left) : Ring::CHUNK);
+        if (Ring::kPoints && points) {
+            if (DIR > 0) {
+                const int64_t left = count * D - k * Ring::CHUNK;
+                ring.issue_points(chunk_src(k), 0, left < Ring::CHUNK ? int(left) : Ring::CHUNK);
+            } else {
+                // the chunk ends with the row of local step count - 1 - k * CS; rows of steps before the range are not read
+                const int64_t before = (k + 1) * CS - count;
+                ring.issue_points(chunk_src(k), before > 0 ? int(before) * D : 0, Ring::CHUNK);
+            }
         } else {
             ring.issue(chunk_src(k));
         }
@@ -493,8 +510,10 @@ template <typename T, int D, int N, int TAIL, int K, bool ZL, int LL = 0>
 __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
     T* __restrict__ dzinc, int64_t batch, int64_t L, int d_rt, int64_t sig_stride, int scalar,
-    int use_lds, int nseg, int64_t lseg)
+    int use_lds, int nseg, int64_t lseg, int from_points)
 {
+    // `from_points` (staged kernels of narrow paths only): `inc` is the plain path [paths][L + 1][d] itself and the
+    // increments are formed while they are staged.
     // `batch` counts (path, time segment) items: item vb = path * nseg + segment walks the increments of steps
     // [segment * lseg, min(L, (segment + 1) * lseg)) backwards, starting from the state `sig[vb]` (signature of the
     // path up to the segment's end) and the adjoint `gsig[vb]` (gradient w.r.t. that state).  nseg == 1 is the
@@ -750,18 +769,20 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         }
     };
 
-    const T* row = inc + (it_path * (L + 2) + it_t0 + it_ns) * d;      // row of the item's last step
+    // row of the item's last step; point-fed: the point that step starts from
+    const T* row = from_points ? inc + (it_path * (L + 1) + it_t0 + it_ns - 1) * d : inc + (it_path * (L + 2) + it_t0 + it_ns) * d;
     if constexpr (ZL) {
         static_assert(WIDE, "staged increments need the wide layout");
         T* lds_wave = lds + kWavesPerBlock * Plan::tile_elems(Tr::DD) + wave_in_block * IncRing<T, Tr::DD, -1>::ELEMS;
         constexpr int NG = (Tr::DD + K - 1) / K;
+        const bool points = IncRing<T, Tr::DD, -1>::kPoints && from_points != 0;
         if constexpr (NG <= 3) {
             static_for<0, NG - 1>([&](auto gc) {
                 if (cx.id.g == decltype(gc)::value)
-                    sweep_staged<-1, decltype(gc)::value * K, Tr>(cx, row, count - 1, count, lds_wave, do_step);
+                    sweep_staged<-1, decltype(gc)::value * K, Tr>(cx, row, count - 1, count, lds_wave, do_step, points);
             });
         } else {
-            sweep_staged<-1, -1, Tr>(cx, row, count - 1, count, lds_wave, do_step);
+            sweep_staged<-1, -1, Tr>(cx, row, count - 1, count, lds_wave, do_step, points);
         }
     } else {
         sweep_direct<-1, false, Cx, typename Tr::Inc>(cx, row, count - 1, count, do_step);
@@ -888,7 +909,7 @@ struct DivBy<uint64_t> {
 };
 
 // test hook: nonzero makes launch_indexed pick 64-bit indices whatever the size (defined in sig_api.hip)
-extern int g_force_wide_index;
+extern std::atomic<int> g_force_wide_index;
 
 // calls f(index type tag, 2-D grid): grid.x covers `per_item` work items of one batch entry, grid.y the batch
 template <typename F>
@@ -936,7 +957,8 @@ __global__ __launch_bounds__(kBlock) void increments_kernel(
             } else {
                 const I t = row - 1;
                 if (time_aug && c == d - 1) {
-                    v = T(t + 1) * time_step - T(t) * time_step;
+                    // two separately rounded products, as the reference's GPU code forms it (siglib/cusig/cu_signature.cu:149-152)
+                    v = mul_rn(T(t + 1), time_step) - mul_rn(T(t), time_step);
                 } else if (!lead_lag) {
                     v = x[int64_t(t + 1) * d_raw + c] - x[int64_t(t) * d_raw + c];
                 } else {
@@ -959,12 +981,24 @@ __global__ __launch_bounds__(kBlock) void increments_kernel(
 // raw segment k -> k+1; the time channel has no raw counterpart
 // (siglib/cpsig/cp_signature.h:1189-1201, siglib/cusig/cu_path_transforms.cu:129-147).
 // ---------------------------------------------------------------------------
+// `clear` (optional): clear_count elements of another buffer are set to zero by the same launch: the increment-gradient
+// accumulator the NEXT backward call will add into (the two accumulators of a device take turns, so a call whose
+// sweep forms its own increments needs no launch that clears one).
+template <typename T>
+__device__ __forceinline__ void clear_range(T* __restrict__ clear, int64_t count)
+{
+    if (!clear) return;
+    const int64_t threads = int64_t(gridDim.x) * gridDim.y * kBlock;
+    for (int64_t e = (int64_t(blockIdx.y) * gridDim.x + blockIdx.x) * kBlock + threadIdx.x; e < count; e += threads) clear[e] = T(0);
+}
+
 // Grid: x over the len_raw * d_raw elements of one path's gradient, y over the paths; the only division is by d_raw.
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void path_grad_kernel(
     const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, int time_aug, int lead_lag,
-    DivBy<I> dv)
+    DivBy<I> dv, T* __restrict__ clear, int64_t clear_count)
 {
+    clear_range(clear, clear_count);
     const I d_raw = I(dv.d);
     const I d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
     const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
@@ -997,8 +1031,10 @@ struct alignas(V * sizeof(T)) VecOf {
 };
 template <typename T, typename I, int V>
 __global__ __launch_bounds__(kBlock) void path_grad_vec_kernel(
-    const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, DivBy<I> dv)
+    const T* __restrict__ dzinc, T* __restrict__ out, int64_t batch, int64_t len_raw, DivBy<I> dv,
+    T* __restrict__ clear, int64_t clear_count)
 {
+    clear_range(clear, clear_count);
     using Vec = VecOf<T, V>;
     const I dvec = I(dv.d);
     const I per = I(len_raw) * dvec;

@@ -72,7 +72,8 @@ hipError_t launch_tree_bwd(const BwdParams& p)
 {
     static_assert(LL == 0 || (D >= 4 && (ZL || TAIL >= 2)), "the lead-lag sweep needs a compile-time dimension");
     // the lead-lag sweep reads a step's parity off its position in the range: ranges must be even and start even
-    if (LL != 0 && ((p.L & 1) || (p.nseg > 1 && (p.lseg & 1)))) return hipErrorInvalidConfiguration;
+    if (LL != 0 && ((p.L & 1) || (p.nseg > 1 && (p.lseg & 1)) || p.from_points)) return hipErrorInvalidConfiguration;
+    if (p.from_points && !(ZL && D > 0 && D <= kPointFedMaxDim)) return hipErrorInvalidConfiguration;
     const TreeGeom g = make_geom(p.d, N - TAIL, K, D != 0);
     if (D < 0 && !g.wide) return hipErrorInvalidConfiguration;     // the kernel was compiled for the wide layout
     const int64_t waves = total_waves(g, p.batch);
@@ -98,7 +99,8 @@ hipError_t launch_tree_bwd(const BwdParams& p)
     hipLaunchKernelGGL((tree_bwd_kernel<T, D, N, TAIL, K, ZL, LL>), dim3((unsigned)blocks), dim3(kBlock), lds, p.stream,
                        static_cast<const T*>(p.inc), static_cast<const T*>(p.sig),
                        static_cast<const T*>(p.gsig), static_cast<T*>(p.dzinc), p.batch, p.L, p.d,
-                       p.sig_stride, p.scalar, use_lds, p.nseg, p.lseg > 0 ? p.lseg : p.L);
+                       p.sig_stride, p.scalar, use_lds, p.nseg, p.lseg > 0 ? p.lseg : p.L,
+                       (ZL && D > 0 && D <= kPointFedMaxDim) ? p.from_points : 0);
     return hipGetLastError();
 }
 

@@ -124,6 +124,8 @@ static void prepare_lyndon(uint64_t dimension, uint64_t degree, int method)
     if (method < 0 || method > 3) throw std::invalid_argument("log signature method must be 1, 2, or 3");
     int dev = 0;
     SIG_HIP(hipGetDevice(&dev));
+    // order of the two locks everywhere: workspace mutex first (held by every call that may be using a table)
+    std::lock_guard<std::mutex> ws_lk(g_ws_mutex);
     std::lock_guard<std::mutex> lk(g_lyndon_mutex);
     DeviceLyndon& slot = g_lyndon[std::make_tuple(dev, dimension, degree)];
     if (slot.method >= method) return;                   // preparing for method 2 also serves method 1
@@ -151,6 +153,7 @@ static void prepare_lyndon(uint64_t dimension, uint64_t degree, int method)
 
 void clear_lyndon_tables() noexcept
 {
+    std::lock_guard<std::mutex> ws_lk(g_ws_mutex);      // no call is using a table while they are freed
     std::lock_guard<std::mutex> lk(g_lyndon_mutex);
     int cur = 0;
     const bool have = hipGetDevice(&cur) == hipSuccess;
@@ -244,9 +247,12 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
     check_method(method, "sig_to_log_sig_cuda");
     const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_cuda");
     if (batch == 0) return;
-    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     const uint64_t bytes = checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
     SIG_HIP(hipDeviceSynchronize());
+    // The prepared tables are looked up and used under the workspace mutex, which prepare / clear / shutdown also take
+    // before they free a table: a table found here stays alive until this call's kernels have finished.
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     hipStream_t stream = nullptr;
     if (s.n_coef == 0) {
         // degree 0: the compressed forms are empty, the expanded one holds the scalar slot
@@ -255,7 +261,6 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
         SIG_HIP(hipStreamSynchronize(stream));
         return;
     }
-    std::lock_guard<std::mutex> lk(g_ws_mutex);
     T* ws = degree >= 2 ? static_cast<T*>(workspace(7, checked_mul(bytes, 2, "workspace"))) : nullptr;
     const uint64_t elems = batch * s.stride;
     // Lyndon coordinates are read off the expanded logarithm, which then lives in a scratch copy
@@ -280,9 +285,10 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
     check_method(method, "sig_to_log_sig_backprop_cuda");
     const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_backprop_cuda");
     if (batch == 0) return;
-    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     const uint64_t bytes = checked_mul(checked_mul(batch, s.stride, "signature"), sizeof(T), "signature");
     SIG_HIP(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lk(g_ws_mutex);      // see sig_to_log_sig_impl
+    const DeviceLyndon lyn = method ? find_lyndon(dimension, degree, method) : DeviceLyndon();
     hipStream_t stream = nullptr;
     if (s.n_coef == 0) {
         if (scalar_term) hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch));
@@ -290,7 +296,6 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
         SIG_HIP(hipStreamSynchronize(stream));
         return;
     }
-    std::lock_guard<std::mutex> lk(g_ws_mutex);
     const uint64_t elems = batch * s.stride;
     if (method) {
         // gradient w.r.t. the expanded logarithm: the transposed coordinate map, zero off the Lyndon words

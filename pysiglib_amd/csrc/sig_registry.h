@@ -32,6 +32,7 @@ struct BwdParams {
     hipStream_t stream;
     int nseg = 1;           // time segments per path; batch counts (path, segment) items
     int64_t lseg = 0;       // steps per segment (0: L)
+    int from_points = 0;    // staged kernels of at most kPointFedMaxDim channels: inc is the plain path [paths][L + 1][d]
 };
 
 typedef hipError_t (*FwdFn)(const FwdParams&);

@@ -1,4 +1,4 @@
-"""The five benchmark workloads (synthetic, seeded) shared by the parity tests and bench.py."""
+"""The five benchmark workloads (synthetic, seeded) and their algorithmic flop counts; used by bench.py and the parity tests."""
 import numpy as np
 
 CONFIGS = {

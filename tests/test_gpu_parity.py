@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests import _configs as C
+from pysiglib_amd import workloads as C
 from tests._mathref import level_rel_err
 
 pytestmark = pytest.mark.gpu
@@ -253,6 +253,46 @@ def test_point_fed_staging(P):
     assert fed > 100     # the staged kernels did run
 
 
+def test_point_fed_backward(P, oracle):
+    """Staged backward sweeps of plain paths of at most 16 channels form the increments from the points as well, and
+    their increment-gradient accumulators take turns (each call's last launch clears the other one): against the sweep
+    fed by the increments kernel and against the oracle, for lengths around the 16-step chunk, shapes that change from
+    call to call (growing and shrinking accumulators), both precisions, and the last path of the batch."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_set_point_fed.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_point_fed.restype = None
+    L.CUSIG.cusig_amd_force_staged.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_staged.restype = None
+    rng = np.random.default_rng(4343)
+    fed = 0
+    try:
+        L.CUSIG.cusig_amd_force_staged(1)
+        for (d, n) in ((10, 5), (5, 7), (4, 8), (16, 4), (17, 4), (12, 4), (6, 6)):
+            for length, batch in ((2, 3), (3, 48), (16, 5), (17, 48), (18, 2), (33, 48), (100, 7), (40, 64)):
+                for dtype in (np.float64, np.float32):
+                    x = (rng.standard_normal((batch, length, d)) * 0.4).astype(dtype)
+                    sig = P.sig(dev(x), n)
+                    g = dev(rng.standard_normal(tuple(sig.shape)).astype(dtype))
+                    L.CUSIG.cusig_amd_set_point_fed(0)
+                    ref = P.sig_backprop(dev(x), sig, g, n).cpu().numpy()
+                    L.CUSIG.cusig_amd_set_point_fed(1)
+                    L.CUSIG.cusig_amd_set_profiling(1)
+                    out = P.sig_backprop(dev(x), sig, g, n).cpu().numpy()
+                    name = L.CUSIG.cusig_amd_last_kernel_name().decode()
+                    L.CUSIG.cusig_amd_set_profiling(0)
+                    fed += name.endswith("_lds") and d <= 16
+                    # the same sums in another order of the atomic adds: rounding-level agreement
+                    assert bwd_rel_err(out, ref) <= (1e-13 if dtype == np.float64 else 2e-5), (d, n, length, batch, dtype, name)
+                    if length in (17, 40):
+                        want = oracle.sig_backprop(x, sig.cpu().numpy(), g.cpu().numpy(), n, n_jobs=-1)
+                        assert bwd_rel_err(out, want) <= TOL[dtype], (d, n, length, batch, dtype, name)
+    finally:
+        L.CUSIG.cusig_amd_set_point_fed(1)
+        L.CUSIG.cusig_amd_force_staged(-1)
+    assert fed > 40      # the staged kernels did run
+
+
 def test_lead_lag_sparse_steps(P, oracle):
     """Staged forward sweeps of lead-lag paths leave out the multiply-adds by the channels a step cannot move (their
     increments are exactly zero): same bits as the dense sweep of the same pieces, for both time-augmentation settings,
@@ -426,10 +466,17 @@ def test_error_codes_through_the_abi(P):
     assert f(p, p, 1, 2, 2, 2, False, False, 1.0, True, True, p, 4, 0, 0) == 10            # valid correction: unsupported
     assert f(p, p, 0, 2, 2, 2, False, False, 1.0, True, True, None, 0, 0, 0) == 0          # empty batch
     assert f(p, p, 1, 100, 2, 100, False, False, 1.0, True, True, None, 0, 0, 0) == 10     # size overflow
-    assert f(p, p, 1, 2, 2, 40, False, False, 1.0, True, True, None, 0, 0, 0) == 10        # no kernel for this degree
+    # degrees beyond 64 are refused while the arguments are checked, as in the reference (nothing is launched)
+    assert f(p, p, 1, 2, 2, 62, False, True, 1.0, True, True, None, 0, 0, 0) == 10         # 4 channels: length overflows
+    assert f(p, p, 1, 2, 2, 65, False, False, 1.0, True, True, None, 0, 0, 0) == 10        # 2^66 coefficients: overflows first
+    bp = L.CUSIG_SIG_BACKPROP["float64"]
+    assert f(p, p, 1, 1, 2, 70, True, False, 1.0, True, True, None, 0, 0, 0) == 10         # time-augmented: 2 channels
+    assert f(p, p, 1, 2, 2, 60, False, False, 1.0, True, True, None, 0, 0, 0) == 10        # 2^61 coefficients: no launch possible
+    assert "too large" in L.last_error_message()
+    assert bp(p, p, p, p, 1, 5, 2, 17, False, False, 1.0, True, None, 0, 0, 0) == 10       # 5 channels, degree 17: no kernel
     assert "no kernel" in L.last_error_message()
-    with pytest.raises(Exception, match="Error in pysiglib.sig"):
-        P.sig(torch.zeros(1, 3, 2, dtype=torch.float64, device=DEV), 17)
+    # degree 17 of two channels is served (a path that does not move has the zero signature)
+    assert not P.sig(torch.zeros(1, 3, 2, dtype=torch.float64, device=DEV), 17).any()
     y = torch.zeros(3, 4, 2, dtype=torch.float64, device=DEV)
     with pytest.raises(ValueError):                                   # width matches neither convention
         P.sig_backprop(y, torch.zeros(3, 5, dtype=torch.float64, device=DEV),
@@ -542,6 +589,8 @@ def test_time_segmented_backward(P, oracle, segments):
     ((70000, 3, 2, 2), np.float32), ((66000, 4, 3, 3), np.float64),                                # batch beyond 65535
     ((3, 2000, 2, 4), np.float64), ((1, 20001, 3, 3), np.float64),                                 # long paths
     ((2, 6, 2, 16), np.float64), ((1, 4, 3, 11), np.float64),                                      # highest compiled degrees
+    ((2, 6, 2, 20), np.float64), ((1, 5, 2, 24), np.float64), ((1, 4, 3, 17), np.float64),         # run-time-degree sweeps
+    ((2, 5, 2, 18), np.float32),
 ])
 def test_extreme_shapes(P, oracle, shape, dtype):
     """Shapes the reference's GPU suite probes for its launch and memory limits
@@ -557,6 +606,44 @@ def test_extreme_shapes(P, oracle, shape, dtype):
     ref_b = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
     got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
     assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("shape", [(3, 9, 2, 5), (2, 7, 2, 9), (5, 12, 2, 12), (2, 6, 3, 4), (3, 10, 3, 7), (2, 9, 3, 10),
+                                   (4, 8, 4, 3), (2, 11, 4, 6), (70, 5, 2, 6), (1, 300, 3, 5)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_run_time_degree_sweeps(P, oracle, shape, dtype):
+    """The sweeps that serve degrees 17 .. 64 (2 to 4 augmented channels, chain of run-time length in LDS), forced onto
+    small shapes: against the oracle, forward and backward, plain and augmented paths, with and without scalar term."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_deep.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_deep.restype = None
+    b, length, d, deg = shape
+    rng = np.random.default_rng(b * 1000 + d * 10 + deg)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (0.3 if length < 100 else 0.05)).astype(dtype)
+    L.CUSIG.cusig_amd_force_deep(1)
+    try:
+        ref = oracle.signature(x, deg, n_jobs=-1)
+        g = rng.standard_normal(ref.shape).astype(dtype)
+        got = P.sig(dev(x), deg)
+        assert level_rel_err(got.cpu().numpy(), ref, d, deg) <= TOL[dtype]
+        assert L.CUSIG.cusig_amd_last_kernel_name is not None
+        got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+        assert bwd_rel_err(got_b, oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)) <= TOL[dtype]
+        with_scalar = P.sig(dev(x), deg, scalar_term=True).cpu().numpy()
+        assert np.all(with_scalar[:, 0] == 1) and np.array_equal(with_scalar[:, 1:], got.cpu().numpy())
+        if d == 2 and deg <= 6:
+            # one raw channel with time: 2 augmented channels; with lead-lag and time: 3
+            x1 = x[:, :, :1].copy()
+            for aug in (dict(time_aug=True, end_time=0.7), dict(time_aug=True, lead_lag=True)):
+                ref = oracle.signature(x1, deg, **aug)
+                d_aug = 2 + (1 if aug.get("lead_lag") else 0)
+                assert level_rel_err(P.sig(dev(x1), deg, **aug).cpu().numpy(), ref, d_aug, deg) <= TOL[dtype]
+                g = rng.standard_normal(ref.shape).astype(dtype)
+                want = oracle.sig_backprop(x1, ref, g, deg, **aug)
+                assert bwd_rel_err(P.sig_backprop(dev(x1), dev(ref), dev(g), deg, **aug).cpu().numpy(), want) <= TOL[dtype]
+    finally:
+        L.CUSIG.cusig_amd_force_deep(0)
 
 
 @pytest.mark.parametrize("shape", [
