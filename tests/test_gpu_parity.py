@@ -511,6 +511,93 @@ def test_autograd_wrapper(P, oracle):
     torch.testing.assert_close((grad * direction).sum(), fd, atol=2e-7, rtol=2e-7)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_inputs_from_a_side_stream(P, oracle, dtype, scalar_term):
+    """Inputs produced, and results consumed, on a non-default stream (a non-contiguous batch view, as in
+    tests/test_cuda_horner.py:149-167 of the reference): the entry points wait for the device on entry, so work
+    queued on any stream is seen, and they return with their own work done."""
+    rng = np.random.default_rng(98)
+    data = (0.025 * np.cumsum(rng.standard_normal((2, 2, 131, 6)), axis=-2)).astype(dtype)
+    x = np.ascontiguousarray(data[..., ::2])
+    flat = x.reshape(4, 131, 3)
+    want = oracle.signature(flat, 10, scalar_term=scalar_term, n_jobs=-1)
+    seeds = (0.03 * rng.standard_normal(want.shape)).astype(dtype)
+    want_grad = oracle.sig_backprop(flat, want, seeds, 10, n_jobs=-1)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        # a chain of kernels on the side stream right before the call: the call must not start ahead of them
+        staged = torch.tensor(data, device=DEV)
+        for _ in range(20):
+            staged = staged * 1.0 + 0.0
+        path = staged[..., ::2].requires_grad_()
+        got = P.torch_api.signature(path, 10, scalar_term=scalar_term)
+        (grad,) = torch.autograd.grad(got, path, torch.tensor(seeds.reshape(2, 2, -1), device=DEV))
+        got_host = (got.detach() * 1.0).cpu().numpy()
+        grad_host = (grad * 1.0).cpu().numpy()
+    stream.synchronize()
+    d_tol = TOL[dtype]
+    assert level_rel_err(got_host.reshape(4, -1)[:, (1 if scalar_term else 0):], want[:, (1 if scalar_term else 0):], 3, 10) <= d_tol
+    assert bwd_rel_err(grad_host.reshape(4, 131, 3), want_grad) <= d_tol
+
+
+def test_two_host_threads(P, oracle):
+    """The entry points are re-entrant: two host threads calling sig, sig_backprop and the log signature with different
+    shapes at the same time get the results of serial calls (the library serialises them on its workspaces; error
+    messages and the overflow report are per thread)."""
+    import ctypes
+    import threading
+    from pysiglib_amd import _loader as L
+    rng = np.random.default_rng(606)
+    jobs = []
+    for (b, length, d, deg, dtype) in [(6, 70, 3, 5, np.float64), (3, 33, 10, 4, np.float32), (16, 20, 2, 8, np.float64),
+                                       (2, 150, 6, 3, np.float32), (5, 40, 4, 6, np.float64), (4, 64, 12, 3, np.float64)]:
+        x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * 0.2).astype(dtype)
+        ref = oracle.signature(x, deg, n_jobs=-1)
+        g = rng.standard_normal(ref.shape).astype(dtype)
+        jobs.append((x, deg, g, ref, oracle.sig_backprop(x, ref, g, deg, n_jobs=-1),
+                     oracle.sig_to_log_sig(ref.astype(np.float64), d, deg, 1 if d == 3 else 0)))
+    P.prepare_log_sig(3, 5, method=1)
+    errors = []
+
+    def worker(which):
+        try:
+            torch.cuda.set_device(0)
+            for rep in range(6):
+                for i, (x, deg, g, ref, ref_b, ref_log) in enumerate(jobs):
+                    if (i + rep) % 2 != which:
+                        continue
+                    d = x.shape[2]
+                    out = P.sig(dev(x), deg)
+                    assert level_rel_err(out.cpu().numpy(), ref, d, deg) <= TOL[x.dtype.type], ("fwd", i)
+                    got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+                    assert bwd_rel_err(got_b, ref_b) <= TOL[x.dtype.type], ("bwd", i)
+                    if x.dtype == np.float64:
+                        got_log = P.sig_to_log_sig(dev(ref), d, deg, method=1 if d == 3 else 0).cpu().numpy()
+                        assert np.abs(got_log - ref_log).max() <= 1e-10 * max(1.0, np.abs(ref_log).max()), ("log", i)
+                    if d == 3 and which == 0:
+                        P.prepare_log_sig(3, 5, method=2 if rep % 2 else 1)     # replaces a table while the other thread runs
+                # a failing call leaves its message with the calling thread only
+                bad = torch.zeros(8, dtype=torch.float64, device=DEV)
+                ptr = ctypes.cast(bad.data_ptr(), ctypes.POINTER(ctypes.c_double))
+                if which == 0:
+                    assert L.CUSIG_SIGNATURE["float64"](ptr, ptr, 1, 0, 2, 2, False, False, 1.0, True, True, None, 0, 0, 0) == 2
+                    assert "dimension 0" in L.last_error_message()
+                else:
+                    assert L.CUSIG_SIG_BACKPROP["float64"](ptr, ptr, ptr, ptr, 1, 2, 2, 2, False, True, 1.0, True, ptr, 4, 0, 0) == 2
+                    assert "lead_lag" in L.last_error_message()
+        except BaseException as exc:       # noqa: BLE001 - reported by the main thread
+            errors.append((which, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in (0, 1)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=110)
+    assert not any(t.is_alive() for t in threads)
+    assert not errors, errors
+
+
 def test_reused_buffers_and_repeatability(P, oracle):
     # the library keeps internal workspaces between calls: interleave shapes and repeat
     rng = np.random.default_rng(21)
