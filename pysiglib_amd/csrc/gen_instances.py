@@ -76,9 +76,9 @@ if os.environ.get("SIGAMD_EXTRA_PARTITIONS"):
 def spec_shapes():
     """(D, N) pairs that get specialised kernels."""
     caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 6, 8: 6}
-    caps.update({d: 5 for d in range(9, 17)})
-    caps.update({d: 4 for d in range(17, 33)})
-    caps.update({d: 3 for d in range(33, 65)})
+    caps.update({d: 5 for d in range(9, 21)})
+    caps.update({d: 4 for d in range(21, 41)})
+    caps.update({d: 3 for d in range(41, 129)})
     out = []
     for d, nmax in sorted(caps.items()):
         for n in range(2, nmax + 1):
@@ -133,6 +133,18 @@ def choose(D, N, dtype, direction):
     key = (dtype, D, N, direction)
     if key in OVERRIDES:
         return OVERRIDES[key]
+    # Beyond the dimensions the tuning sweeps covered, measured on MI355X at d = 80, 100, 128 (degree 3) and d = 36, 40
+    # (degree 4) against the model's choice: forward 1.5-5x (35-50 TFLOP/s f32, 23-25 f64 at degree 3; 60 / 23 at degree
+    # 4), backward 1.3-2x (10-12 TFLOP/s f32 at degree 3, 45-52 f32 / 11 f64 at degree 4).
+    if N == 3 and D > 64:
+        if direction == "fwd":
+            return (1, -(-D // 4) if D <= 100 else 13)      # four letter groups without a stub
+        if dtype == "f32":
+            return (2, 2) if D <= 100 else (2, 1)
+    if N == 4 and D > 32:
+        if direction == "fwd":
+            return (1, D) if dtype == "f32" else (1, D // 2)
+        return (2, 3)
     if dtype == "f64" and direction == "fwd" and D >= 24 and N == 3:
         # measured on MI355X (d = 24, 32, 48 at degree 3): the f64 forward runs 1.1-1.8x faster with one subtree level
         # per lane and all (or half of) the letters than with the two-level subtrees the model picks
@@ -229,6 +241,8 @@ def main():
             is64 = 1 if T == "double" else 0
             zs = "true" if zl else "false"
             pol = STAGE_POLICY.get(("f64" if is64 else "f32", D, N, direction), 0)
+            if N == 4 and D > 32 and direction == "fwd":
+                pol = 2         # measured at d = 36, 40: one subtree level with all letters runs 1.7x faster scalar-fed
             name = "%s_%s_d%s_n%d_t%d_k%d%s" % (direction, "f64" if is64 else "f32", "0w" if D < 0 else str(D), N, tail, K,
                                                 "_lds" if zl else "")
             if direction == "fwd":

@@ -584,11 +584,11 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     const int RS = Plan::rows_per_step(d);      // tile rows per step
     const bool tiled = CH > 0;
     const int slots = WIDE ? 1 : cx.G.ppw;
-    T* wbuf = lds + int64_t(wave_in_block) * (tiled ? Plan::tile_elems(d) : int64_t(slots) * d);
+    T* wbuf = lds + int64_t(wave_in_block) * (tiled ? Plan::tile_elems(d) : use_lds == 2 ? int64_t(Plan::kRows) * kRedStride : int64_t(slots) * d);
     T* acc = wbuf + int64_t(cx.id.slot) * d;
     const int nsg = slots > 1 ? slots : 2;                    // column segments per row
     const int seg_cnt = slots > 1 ? int(cx.G.lpp) : kWave / 2; // lanes per segment
-    if (!tiled && use_lds) {
+    if (!tiled && use_lds == 1) {
         for (int e = lane; e < slots * d; e += kWave) wbuf[e] = T(0);
         wave_lds_sync();
     }
@@ -727,6 +727,49 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
                 t_chunk -= cs;
                 cs = 0;
                 limit = CH;
+            }
+        } else if (use_lds == 2) {
+            // Paths too wide for a tile that holds a whole step (wave serves one item): the letters of the step pass
+            // through a tile of kRows rows in groups.  Per group every lane clears its own column, adds the pieces
+            // whose letters fall into the group (own column: no two lanes ever meet), and the rows are summed and
+            // added to the gradient as in reduce_chunk.
+            constexpr int RW = Plan::kRows;
+            T* col = wbuf + lane;
+            const bool live_step = t >= count - it_ns;
+            for (int base = 0; base < d; base += RW) {
+                const int nrow = d - base < RW ? d - base : RW;
+                for (int r = 0; r < nrow; ++r) col[r * kRedStride] = T(0);
+                auto emit = [&](int letter, T v) {
+                    if (letter >= base && letter < base + nrow) lds_add(&col[(letter - base) * kRedStride], v);
+                };
+                if constexpr (TAIL >= 2) {
+#pragma unroll
+                    for (int j = 0; j < Tr::DD; ++j) emit(j, dz.dj[j]);
+                }
+                if constexpr (!FOLD) {
+#pragma unroll
+                    for (int a = 0; a < K; ++a)
+                        if (cx.a0 + a < d) emit(cx.a0 + a, dz.da[a]);
+                }
+#pragma unroll
+                for (int l = 0; l < M; ++l) emit(cx.p[l], dz.dc[l]);
+                wave_lds_sync();
+                for (int it = lane; it < nrow * 2; it += kWave) {
+                    const int sg = it & 1, r = it >> 1;
+                    const T* src = wbuf + r * kRedStride + sg * (kWave / 2);
+                    T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
+#pragma unroll
+                    for (int i = 0; i < kWave / 2; i += 4) {
+                        s0 += src[i];
+                        s1 += src[i + 1];
+                        s2 += src[i + 2];
+                        s3 += src[i + 3];
+                    }
+                    T sum = (s0 + s1) + (s2 + s3);
+                    sum += __shfl_xor(sum, 1);          // the two halves of a row sit in neighbouring lanes
+                    if (sg == 0 && live_step && b_first < batch) dev_add(&dzinc[wave_base + t * d + base + r], sum);
+                }
+                wave_lds_sync();
             }
         } else {
             T* grow_t = dzinc + lane_base + t * d;

@@ -84,6 +84,10 @@ hipError_t launch_tree_bwd(const BwdParams& p)
     using Plan = RedPlan<T, D, TAIL, K, ZL>;
     if (Plan::steps(p.d) > 0) {
         lds = size_t(kWavesPerBlock) * size_t(Plan::tile_elems(p.d)) * sizeof(T);
+    } else if (g.ppw == 1) {
+        // wider than any tile: the letters of a step pass through a tile of kRows rows in groups
+        use_lds = 2;
+        lds = size_t(kWavesPerBlock) * size_t(Plan::kRows) * kRedStride * sizeof(T);
     } else {
         lds = size_t(kWavesPerBlock) * size_t(g.ppw) * size_t(p.d) * sizeof(T);
         if (lds > kMaxDynLds) { use_lds = 0; lds = 0; }

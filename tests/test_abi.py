@@ -116,9 +116,11 @@ def test_kernel_table(lib):
         for f64 in (0, 1):
             for (d, n) in ((10, 5), (5, 7), (3, 12), (17, 4)):
                 assert fn(bwd, f64, d, n, tail, k, spec) == 1 and spec.value == 1 and 1 <= tail.value < n
-            assert fn(bwd, f64, 37, 3, tail, k, spec) == 1 and spec.value == 1      # the table reaches d = 64 at degree 3
-            assert fn(bwd, f64, 70, 3, tail, k, spec) == 1 and spec.value == 0      # run-time-dimension kernel
-            assert fn(bwd, f64, 2, 40, tail, k, spec) == 0                           # beyond the compiled degrees
+            assert fn(bwd, f64, 100, 3, tail, k, spec) == 1 and spec.value == 1     # the table reaches d = 128 at degree 3,
+            assert fn(bwd, f64, 40, 4, tail, k, spec) == 1 and spec.value == 1      # 40 at degree 4, 20 at degree 5
+            assert fn(bwd, f64, 20, 5, tail, k, spec) == 1 and spec.value == 1
+            assert fn(bwd, f64, 150, 3, tail, k, spec) == 1 and spec.value == 0     # run-time-dimension kernel
+            assert fn(bwd, f64, 2, 40, tail, k, spec) == 0                           # served by the run-time-degree sweeps, not by the table
 
 
 def test_wrapper_argument_errors():

@@ -736,7 +736,8 @@ def test_run_time_degree_sweeps(P, oracle, shape, dtype):
 @pytest.mark.parametrize("shape", [
     (3, 9, 13, 4), (2, 12, 20, 3), (5, 7, 30, 2), (2, 6, 32, 3), (3, 8, 50, 2), (4, 9, 40, 2), (2, 5, 18, 5), (2, 6, 100, 2),
     (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2),
-    (2, 6, 70, 3), (1, 5, 34, 4), (2, 5, 17, 5), (3, 40, 65, 3)])        # beyond the specialised table: run-time dimension
+    (2, 6, 70, 3), (1, 5, 34, 4), (2, 5, 17, 5), (3, 40, 65, 3),
+    (2, 6, 130, 3), (2, 7, 97, 3), (1, 5, 41, 4), (2, 5, 21, 5), (1, 4, 200, 3)])        # beyond the specialised table: run-time dimension
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_many_channel_shapes(P, oracle, shape, dtype):
     """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
