@@ -936,7 +936,9 @@ def test_config_forward_full_size(P, oracle, k):
 
 def test_config3_forward(P, oracle):
     """(64, 4096, 3) degree 12: the oracle checks the first 6 paths; all 64 are checked through
-    size-independent properties (level 1 = total increment, level-2 shuffle identity, batch invariance up to rounding)."""
+    size-independent properties: level 1 = total increment, the level-2 shuffle identity, batch invariance up to rounding,
+    and Chen's identity on every coefficient (the signatures of the two halves of each path, multiplied with the
+    oracle-checked Chen product, give the signature of the whole path)."""
     c = C.CONFIGS[3]
     x = C.make_path(3)
     xt = dev(x)
@@ -951,7 +953,17 @@ def test_config3_forward(P, oracle):
     # a smaller batch may be cut into time segments (a different order of additions): equal up to rounding
     again = P.sig(xt[40:47].clone(), 12)
     assert level_rel_err(again.cpu().numpy(), got[40:47].cpu().numpy(), 3, 12) <= 1e-12
-    del got, again
+    del again
+    first, second = P.sig(xt[:, :2049].contiguous(), 12), P.sig(xt[:, 2048:].contiguous(), 12)
+    whole = P.sig_combine(first, second, 3, 12)
+    del first, second
+    lo = 0
+    for level in range(1, 13):
+        a, b = whole[:, lo:lo + 3 ** level], got[:, lo:lo + 3 ** level]
+        err = ((a - b).abs().amax(dim=1) / b.abs().amax(dim=1).clamp_min(1e-300)).max().item()
+        assert err <= 1e-10, (level, err)
+        lo += 3 ** level
+    del got, whole
     torch.cuda.empty_cache()
 
 
