@@ -28,10 +28,10 @@ PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 # known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
 # reports null instead of a stale figure.
 TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5_lds": 35.5e6,
+    "fwd_f64_d10_n5_t2_k5_lds": 35.8e6,
     "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
-    "fwd_f32_d5_n7_t4_k1_lds": 163.0e6,    # swept in three time pieces: three segment signature sets are written
-    "fwd_f64_d3_n12_t5_k1": 478.1e6,
+    "fwd_f32_d5_n7_t4_k1_lds": 163.4e6,    # swept in three time pieces: three segment signature sets are written
+    "fwd_f64_d3_n12_t5_k1": 478.7e6,
     "fwd_f32_d17_n4_t2_k6_lds_ll": 114.4e6,
 }
 
