@@ -255,6 +255,10 @@ CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only
  * taken for rows of 2^31 coefficients or more) whatever the size. */
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
+/* Test hook: kernels of the Chen product's adjoint (sig_combine_backprop, sig_join_backprop, the tensor logarithm's
+ * backward, time-split sig_backprop): 0 = streaming kernels for rows of 4096 coefficients or more, 1 = streaming
+ * kernels wherever they apply, 2 = item-per-word kernels only. */
+CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) CUSIG_AMD_NOEXCEPT;
 /* Stream-ordered mode (no counterpart in the reference, off by default).  When enabled, signature_cuda_{f,d} and
  * sig_backprop_cuda_{f,d} enqueue their kernels on the null stream and return without waiting, and do not wait for
  * other streams on entry: inputs must be ordered before, and consumers after, the null stream (true for PyTorch's

@@ -190,6 +190,7 @@ struct Workspace {
     size_t bytes = 0;
 };
 std::atomic<int> g_force_wide_index{0};
+std::atomic<int> g_chen_adjoint_mode{0};
 std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
@@ -1197,6 +1198,7 @@ CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
 
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
+CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) noexcept { g_chen_adjoint_mode = mode; }
 
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
 

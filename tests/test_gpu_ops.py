@@ -4,6 +4,8 @@ the reference's hand-computed vectors and its golden float32 gradients.
 Tolerances: float64 1e-10, float32 1e-4 (relative to the per-level / per-row max norm); exact for the pure copies
 of transform_path; golden float32 gradients at the reference's 1e-5 (tests/test_sig_combine_backprop.py:24).
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -28,6 +30,17 @@ def P():
 def oracle():
     from oracle import sigref
     return sigref
+
+
+@pytest.fixture(params=[0, 1], ids=["adjoint-auto", "adjoint-streaming"])
+def chen_mode(request):
+    """Kernels of the Chen product's adjoint: automatic choice, then the streaming kernels forced onto every shape."""
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_chen_adjoint.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_chen_adjoint.restype = None
+    L.CUSIG.cusig_amd_force_chen_adjoint(request.param)
+    yield request.param
+    L.CUSIG.cusig_amd_force_chen_adjoint(0)
 
 
 def dev(a, dtype=None):
@@ -143,7 +156,7 @@ def test_combine_backprop_golden(P, fixtures, deg, dtype):
                                          (37, 2, 5), (2, 14, 2), (4, 4, 9), (6, 3, 5), (11, 3, 3), (13, 3, 5), (9, 4, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_combine_backprop_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+def test_combine_backprop_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, scalar_term):
     rng = np.random.default_rng(7 * d + deg)
     n = oracle.sig_length(d, deg) - (0 if scalar_term else 1)
     a, b, g = (rng.standard_normal((batch, n)).astype(dtype) for _ in range(3))
@@ -269,7 +282,7 @@ def test_linear_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("prepend", [False, True])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_sig_join_vs_oracle(P, oracle, d, deg, batch, dtype, prepend, scalar_term):
+def test_sig_join_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, prepend, scalar_term):
     rng = np.random.default_rng(5 * d + deg)
     n = oracle.sig_length(d, deg) - 1
     scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
@@ -542,7 +555,7 @@ def test_log_sig_backprop_golden(P, fixtures, deg, dtype):
                                          (40, 2, 3), (2, 12, 2), (6, 4, 3), (13, 3, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_sig_to_log_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+def test_sig_to_log_sig_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, scalar_term):
     rng = np.random.default_rng(3 * d + deg)
     n = oracle.sig_length(d, deg) - 1
     scale = np.concatenate([np.full(d ** k, 0.5 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)]) if deg else np.zeros(0)
