@@ -190,8 +190,10 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
                            degree <= uint64_t(kStreamMaxLevels) && s.n_coef < (uint64_t(1) << 28) &&
                            !g_force_wide_index;
     LeftPlan lp;
+    RowsPlan wp;
     RightPlan rp;
-    const bool left = streaming && make_left_plan(lp, dimension, degree, kStreamLdsEntries);
+    const bool rows = streaming && make_rows_plan(wp, dimension, degree, kStreamLdsEntries);
+    const bool left = rows || (streaming && make_left_plan(lp, dimension, degree, kStreamLdsEntries));
     const bool right = streaming && families > 1 && make_right_plan(rp, dimension, degree);
     if (!left && !right) {
         launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, degree, s, stream, identity, dc, families, 0);
@@ -200,6 +202,39 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
     // left factor: words shorter than the blocks' own take their low-level terms from the truncated problem first
     if (!left) {
         launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, degree, s, stream, identity, dc, 1, 0);
+    } else if (rows) {
+        if (wp.np >= 2)
+            launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, uint64_t(wp.np), s, stream, identity, dc, 1, 0);
+        const uint64_t groups = (uint64_t(wp.units) + uint64_t(wp.upb) - 1) / uint64_t(wp.upb);
+        const dim3 grid{unsigned(groups), unsigned(std::min<uint64_t>(batch, 65535)), 1};
+        const size_t lds = (size_t(wp.bs) + 2 * size_t(wp.targets) + size_t(wp.img)) * sizeof(T);
+        const int kt = int((wp.top + kBlock - 1) / kBlock), ks = int((wp.targets + kBlock - 1) / kBlock);
+        auto go3 = [&](auto dc_, auto kt_, auto ks_) {
+            hipLaunchKernelGGL((chen_adjoint_left_rows_kernel<T, decltype(dc_)::value, decltype(kt_)::value, decltype(ks_)::value>),
+                               grid, dim3(kBlock), lds, stream, dC, dA, B, int64_t(batch), wp, int64_t(s.stride), s.off, identity,
+                               dc.share, dc.stride, dc.off);
+        };
+        auto go2 = [&](auto dc_, auto ks_) {
+            if (kt <= 2) go3(dc_, std::integral_constant<int, 2>(), ks_);
+            else if (kt <= 4) go3(dc_, std::integral_constant<int, 4>(), ks_);
+            else go3(dc_, std::integral_constant<int, kRowsMaxTop>(), ks_);
+        };
+        // owned entries per thread: more than one only for few channels (targets ~ top / (d - 1))
+        auto go = [&](auto dc_) {
+            constexpr int DC = decltype(dc_)::value;
+            if (ks <= 1) go2(dc_, std::integral_constant<int, 1>());
+            else if constexpr (DC <= 8) {
+                if (ks <= 2) go2(dc_, std::integral_constant<int, 2>());
+                else if constexpr (DC <= 4) go2(dc_, std::integral_constant<int, kRowsMaxLow>());
+                else throw std::logic_error("sig_combine_backprop_cuda: kernel plan");
+            } else throw std::logic_error("sig_combine_backprop_cuda: kernel plan");
+        };
+        const uint64_t d = dimension;
+        if (d <= 4) go(std::integral_constant<int, 4>());
+        else if (d <= 8) go(std::integral_constant<int, 8>());
+        else if (d <= 12) go(std::integral_constant<int, 12>());
+        else if (d <= 16) go(std::integral_constant<int, 16>());
+        else go(std::integral_constant<int, 32>());
     } else {
         if (lp.np >= 2)
             launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, uint64_t(lp.np), s, stream, identity, dc, 1, 0);

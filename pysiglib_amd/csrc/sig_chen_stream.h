@@ -37,6 +37,8 @@ struct StreamLevels {
     uint32_t pw[kStreamMaxLevels + 2];      // d^i while it fits 31 bits
 };
 
+static inline bool fill_stream_levels(StreamLevels& lv, uint64_t d, uint64_t degree);
+
 struct RightPlan {
     int degree, qe, rel;        // rel = degree - qe
     uint32_t d, words;          // words = d^qe
@@ -350,6 +352,283 @@ __global__ __launch_bounds__(kBlock) void chen_adjoint_left_kernel(
             }
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Left factor, d <= 32.  As in chen_adjoint_left_kernel a block owns c words p of length np and copies their pieces of
+// the levels np .. N to LDS with coalesced loads (held in registers while the block works on the unit before); the
+// top level's copy, and the partial sums of the words shorter than np, are formed from those registers.  The top
+// piece (most of the data) is addressed from one wave-uniform base with constant offsets per register; an entry of
+// the lower pieces is loaded by the thread that owns it.  The sums inside the block are taken per owner: a thread
+// owns one entry q of the pieces 0 .. mt - 1, reads its d children q x from LDS into registers and forms
+//   * the whole m = 1 term of dA[q]                                   (B_1: wave-uniform operands),
+//   * one partial sum for every ancestor of q inside the block        (B_m from LDS at (q mod d^(m-1)) d + x).
+// Numbering the entries of the pieces 0 .. mt end to end, the parent of entry e is (e - c) / d and its children are
+// e d + c + x: no per-lane table is needed.  The LDS image gives every run of d children one entry of padding when d
+// is even, so that the owners' reads fall into different banks.  Partial sums meet in LDS accumulators (one per
+// entry of the pieces 0 .. mt - 1, two sets used in turn); runs of 32 or more lanes that share an ancestor are summed
+// in the wave first.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kRowsMaxTop = 8;       // entries of the top piece per thread
+constexpr int kRowsMaxLow = 4;       // owned entries per thread
+
+struct RowsPlan {
+    int degree, mt, np, upb;
+    uint32_t d, c, units, targets, top, bs, pad, img;
+    uint32_t eoff[kLeftMaxTile + 2];        // c (d^j - 1) / (d - 1): piece j in the end-to-end numbering
+    uint32_t boff[kLeftMaxTile + 2];        // level m of B inside its LDS copy
+    uint32_t dmul, dshr;                    // n / d == umulhi(n, dmul) >> dshr for n < 2^31
+    StreamLevels lv;
+};
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+    for (int s = kWave >> 1; s; s >>= 1) v += __shfl_xor(v, s);
+    return v;
+}
+
+template <typename T, int DCEIL, int KT, int KS>
+__global__ __launch_bounds__(kBlock) void chen_adjoint_left_rows_kernel(
+    const T* __restrict__ dC, T* __restrict__ dA, const T* __restrict__ B, int64_t batch, RowsPlan P, int64_t stride,
+    int off, int identity, int64_t dc_share, int64_t dc_stride, int dc_off)
+{
+    extern __shared__ __align__(16) unsigned char chen_lds[];
+    T* Bl = reinterpret_cast<T*>(chen_lds);
+    T* Acc = Bl + P.bs;                     // two sets of P.targets accumulators
+    T* Img = Acc + 2 * P.targets;           // the unit's pieces 0 .. mt, runs of d children padded
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int N = P.degree, mt = P.mt, np = P.np;
+    const uint32_t d = P.d, c = P.c, dp = d + P.pad;
+    const Block2 blk = xcd_block_2d();
+    const uint32_t u0 = blk.x * uint32_t(P.upb);
+    const uint32_t u1 = u0 + uint32_t(P.upb) < P.units ? u0 + uint32_t(P.upb) : P.units;
+    if (u0 >= u1) return;
+    // per-thread constants.  Top piece: entry tid + kBlock i and its place in the image.  Owned entry q = tid +
+    // kBlock s of the lower pieces: its offset in a row of dC is lgo + p0 * lpw, its place in the image limg.
+    uint32_t timg[KT];
+#pragma unroll
+    for (int i = 0; i < KT; ++i) {
+        const uint32_t rel = tid + uint32_t(kBlock) * i;
+        const uint32_t x = P.eoff[mt] + rel;
+        timg[i] = rel < P.top ? x + P.pad * (__umulhi(x - c, P.dmul) >> P.dshr) : 0xffffffffu;
+    }
+    uint32_t lgo[KS], lpw[KS], limg[KS];
+#pragma unroll
+    for (int sl = 0; sl < KS; ++sl) {
+        const uint32_t q = tid + uint32_t(kBlock) * sl;
+        uint32_t gbt = P.lv.lo[np], pwt = 1;
+        for (int jj = 2; jj <= mt; ++jj) {
+            const bool in = q >= P.eoff[jj - 1];
+            gbt = in ? P.lv.lo[np + jj - 1] - P.eoff[jj - 1] : gbt;
+            pwt = in ? P.lv.pw[jj - 1] : pwt;
+        }
+        lgo[sl] = gbt + q;
+        lpw[sl] = q < P.targets ? pwt : 0;      // 0 marks an unused slot
+        limg[sl] = q < c ? q : q + P.pad * (__umulhi(q - c, P.dmul) >> P.dshr);
+    }
+    const uint32_t c1 = np >= 2 ? (P.lv.pw[np] - P.lv.pw[1]) / (d - 1) : 0;      // level shift of the nearest long level
+    for (int64_t b = blk.y; b < batch; b += gridDim.y) {
+        const T* g = dC + (b / dc_share) * dc_stride + dc_off;
+        const T* other = B + b * stride + off;
+        T* out = dA + b * stride + off;
+        if (off && blk.x == 0 && tid == 0) dA[b * stride] = T(0);
+        T rx[KT], rb[KT], rl[KS], rlb[KS];
+        auto fetch = [&](uint32_t unit) {
+            const uint32_t p0 = unit * c;
+            const uint32_t rem1 = np >= 2 ? p0 % P.lv.pw[1] : 0;
+            const T* gt = g + P.lv.lo[N] + p0 * P.lv.pw[mt] + tid;
+            const T* bt = other + P.lv.lo[1 + mt] + rem1 * P.lv.pw[mt] + tid;
+#pragma unroll
+            for (int i = 0; i < KT; ++i) {
+                const bool ok = timg[i] != 0xffffffffu;
+                rx[i] = ok ? gt[kBlock * i] : T(0);
+                rb[i] = (ok && np >= 2) ? bt[kBlock * i] : T(0);
+            }
+#pragma unroll
+            for (int sl = 0; sl < KS; ++sl) {
+                const bool ok = lpw[sl] != 0;
+                rl[sl] = ok ? g[lgo[sl] + p0 * lpw[sl]] : T(0);
+                rlb[sl] = (ok && np >= 2 && lpw[sl] > 1) ? other[lgo[sl] + lpw[sl] * (rem1 - c1)] : T(0);
+            }
+        };
+        auto finish = [&](uint32_t unit, T* Aset) {      // stores the complete entries of a unit, clears their sums
+            const uint32_t p0 = unit * c;
+#pragma unroll
+            for (int sl = 0; sl < KS; ++sl) {
+                const uint32_t q = tid + uint32_t(kBlock) * sl;
+                if (lpw[sl] != 0) {
+                    out[lgo[sl] + p0 * lpw[sl]] = Aset[q];
+                    Aset[q] = T(0);
+                }
+            }
+        };
+        fetch(u0);
+        __syncthreads();                                                        // the row before is done with the LDS
+        for (uint32_t z = tid; z < P.bs; z += kBlock) Bl[z] = other[z];        // levels 1 .. mt open the row
+        for (uint32_t z = tid; z < 2 * P.targets; z += kBlock) Acc[z] = T(0);
+        uint32_t flip = 0;
+        for (uint32_t unit = u0; unit < u1; ++unit, flip ^= 1) {
+            const uint32_t p0 = unit * c;
+            T* A = Acc + flip * P.targets;
+            __syncthreads();                        // the owners of the unit before have read the image and added their sums
+            if (unit > u0) finish(unit - 1, Acc + (flip ^ 1) * P.targets);
+            T s1 = T(0);
+            {
+                T* top = out + P.lv.lo[N] + p0 * P.lv.pw[mt] + tid;            // the top level has no sum
+#pragma unroll
+                for (int i = 0; i < KT; ++i) {
+                    if (timg[i] != 0xffffffffu) {
+                        Img[timg[i]] = rx[i];
+                        top[kBlock * i] = identity ? rx[i] : T(0);
+                        s1 = fmadd(rx[i], rb[i], s1);
+                    }
+                }
+#pragma unroll
+                for (int sl = 0; sl < KS; ++sl) {
+                    if (lpw[sl] != 0) {
+                        Img[limg[sl]] = rl[sl];
+                        s1 = fmadd(rl[sl], rlb[sl], s1);
+                    }
+                }
+            }
+            if (np >= 2) {
+                s1 = wave_sum(s1);
+                if (lane == 0) dev_add(out + P.lv.lo[np - 1] + p0 / P.lv.pw[1], s1);
+            }
+            // words shorter than np - 1: their factors are loaded here (deep signatures of few channels)
+            for (int k = np - 2; k >= 1; --k) {
+                const uint32_t span = P.lv.pw[np - k];
+                const uint32_t row = p0 / span, rem = p0 - row * span;
+                const uint32_t ck = (P.lv.pw[np] - span) / (d - 1);
+                const T* bt = other + P.lv.lo[np - k + mt] + rem * P.lv.pw[mt] + tid;
+                T bk[KT], bl[KS];
+#pragma unroll
+                for (int i = 0; i < KT; ++i) bk[i] = timg[i] != 0xffffffffu ? bt[kBlock * i] : T(0);
+#pragma unroll
+                for (int sl = 0; sl < KS; ++sl) bl[sl] = lpw[sl] > 1 ? other[lgo[sl] + lpw[sl] * (rem - ck)] : T(0);
+                T sk = T(0);
+#pragma unroll
+                for (int i = 0; i < KT; ++i) sk = fmadd(rx[i], bk[i], sk);
+#pragma unroll
+                for (int sl = 0; sl < KS; ++sl) sk = fmadd(rl[sl], bl[sl], sk);
+                sk = wave_sum(sk);
+                if (lane == 0) dev_add(out + P.lv.lo[k] + row, sk);
+            }
+            __syncthreads();                        // the image is complete
+            if (unit + 1 < u1) fetch(unit + 1);
+#pragma unroll
+            for (int sl = 0; sl < KS; ++sl) {
+                const uint32_t q = tid + uint32_t(kBlock) * sl;
+                const bool live = lpw[sl] != 0;
+                T ch[DCEIL];
+                const T* row = Img + c + (live ? q : 0) * dp;
+#pragma unroll
+                for (int v = 0; v < DCEIL; ++v) ch[v] = (uint32_t(v) < d && live) ? row[v] : T(0);
+                T s = (identity && live) ? Img[limg[sl]] : T(0);
+#pragma unroll
+                for (int v = 0; v < DCEIL; ++v)
+                    if (uint32_t(v) < d) s = fmadd(ch[v], other[v], s);       // m = 1: the whole term of q itself
+                if (live) lds_add_shared(A + q, s);
+                // ancestors inside the block
+                uint32_t a = q, rem = 0;
+                bool on = live;
+                for (int m = 2; m <= mt; ++m) {
+                    on = on && a >= c;
+                    const uint32_t num = on ? a - c : 0;
+                    const uint32_t quo = __umulhi(num, P.dmul) >> P.dshr;
+                    rem += (num - quo * d) * P.lv.pw[m - 2];
+                    a = quo;
+                    T t = T(0);
+                    if (on) {
+                        const T* br = Bl + P.boff[m] + rem * d;
+#pragma unroll
+                        for (int v = 0; v < DCEIL; ++v)
+                            if (uint32_t(v) < d) t = fmadd(ch[v], br[v], t);
+                    }
+                    if (P.lv.pw[m - 1] >= 32) {          // long runs of lanes share an ancestor: sum them in the wave
+                        uint64_t todo = __ballot(on);
+                        while (todo) {
+                            const int first = __ffsll((unsigned long long)todo) - 1;
+                            const uint32_t key = __shfl(a, first);
+                            const bool sel = on && a == key;
+                            const T sum = wave_sum(sel ? t : T(0));
+                            if (int(lane) == first) lds_add_shared(A + key, sum);
+                            todo &= ~__ballot(sel);
+                        }
+                    } else if (on) {
+                        lds_add_shared(A + a, t);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        finish(u1 - 1, Acc + (flip ^ 1) * P.targets);
+    }
+}
+
+static inline bool make_rows_plan(RowsPlan& P, uint64_t d, uint64_t degree, uint64_t lds_entries)
+{
+    if (d < 2 || d > 32 || degree < 2 || !fill_stream_levels(P.lv, d, degree)) return false;
+    auto levels = [&](int mt) {      // d + .. + d^mt
+        uint64_t s = 0, p = 1;
+        for (int j = 1; j <= mt; ++j) { p *= d; s += p; if (s > (uint64_t(1) << 30)) return uint64_t(1) << 30; }
+        return s;
+    };
+    const uint64_t pad = d % 2 == 0 ? 1 : 0;
+    // LDS entries: B's levels 1 .. mt, two sets of sums, and the image of c words' pieces with its padding
+    auto need = [&](int mt, uint64_t c) {
+        const uint64_t targets = c * (levels(mt) + 1 - uint64_t(P.lv.pw[mt]));
+        return levels(mt) + 2 * targets + c * (levels(mt) + 1) + pad * targets;
+    };
+    int mt = 1;
+    while (mt + 1 <= int(degree) - 1 && mt + 1 <= kLeftMaxTile && P.lv.pw[mt + 1] != 0 && need(mt + 1, 1) <= lds_entries) ++mt;
+    const uint64_t ks_max = d <= 4 ? uint64_t(kRowsMaxLow) : d <= 8 ? 2 : 1;      // owned entries per thread the kernels are built for
+    uint64_t c = 0, per = 0;
+    for (; mt >= 1 && c == 0; --mt) {
+        per = levels(mt) + 1 - uint64_t(P.lv.pw[mt]);      // entries of the pieces 0 .. mt - 1 for c = 1
+        double best = 0;
+        for (uint64_t cand = 1; cand <= d; ++cand) {
+            if (d % cand) continue;
+            const uint64_t targets = cand * per, top = cand * uint64_t(P.lv.pw[mt]);
+            const uint64_t ks = (targets + kBlock - 1) / kBlock, kt = (top + kBlock - 1) / kBlock;
+            if (ks > ks_max || kt > uint64_t(kRowsMaxTop) || need(mt, cand) > lds_entries) continue;
+            const double use = 0.3 * double(targets) / double(ks * kBlock) + 0.7 * double(top) / double(kt * kBlock);
+            if (use > best + 1e-9) { best = use; c = cand; }
+        }
+        if (c != 0) break;
+    }
+    if (c == 0) return false;
+    P.degree = int(degree);
+    P.mt = mt;
+    P.np = int(degree) - mt;
+    P.d = uint32_t(d);
+    P.c = uint32_t(c);
+    P.pad = uint32_t(pad);
+    P.units = uint32_t(uint64_t(P.lv.pw[P.np]) / c);
+    P.targets = uint32_t(c * per);
+    P.top = uint32_t(c * uint64_t(P.lv.pw[mt]));
+    P.bs = uint32_t(levels(mt));
+    P.img = uint32_t(c * (levels(mt) + 1) + pad * P.targets);
+    uint64_t x = 0, p = 1, bo = 0;
+    for (int j = 0; j <= mt + 1; ++j) {
+        P.eoff[j] = uint32_t(c * x);
+        x += p;
+        p *= d;
+    }
+    p = d;
+    P.boff[0] = 0;
+    for (int m = 1; m <= mt + 1; ++m) {
+        P.boff[m] = uint32_t(bo);
+        bo += p;
+        p *= d;
+    }
+    const DivBy<uint32_t> dv(d);
+    P.dmul = dv.mul;
+    P.dshr = dv.shr;
+    const uint64_t moved = uint64_t(P.targets) * d;
+    P.upb = int(std::max<uint64_t>(1, std::min<uint64_t>((4 * uint64_t(P.bs) + moved - 1) / moved, P.units)));
+    return true;
 }
 
 static inline bool fill_stream_levels(StreamLevels& lv, uint64_t d, uint64_t degree)
