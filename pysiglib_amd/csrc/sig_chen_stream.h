@@ -80,7 +80,10 @@ struct RightLane {
     T acc[kRightMaxRel + 1];
 };
 
-constexpr int kLeafBatch = 4;        // loads of the deepest level that are in flight together
+#ifndef SIGAMD_LEAF_BATCH
+#define SIGAMD_LEAF_BATCH 5
+#endif
+constexpr int kLeafBatch = SIGAMD_LEAF_BATCH;       // loads of the deepest level that are in flight together
 
 // visits the words (x w), x = 0 .. d-1, in front of the lane's word; `widx` is the index of w (length DEPTH - 1) and
 // pfx[i] the index of its first i letters.  The deepest level issues its loads kLeafBatch at a time, and an inner
@@ -99,11 +102,16 @@ __device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPl
             T w[QL > 0 ? QL : 1][kLeafBatch];
 #pragma unroll
             for (int i = 0; i < kLeafBatch; ++i) {
-                const uint32_t x = x0 + i < P.d ? x0 + i : P.d - 1;
+                const uint32_t x = x0 + i;
                 const uint32_t idx = x * P.lv.pw[DEPTH - 1] + widx;
-                e[i] = L.live ? load_at(grow + idx * P.words, L.fo) : T(0);
+                e[i] = T(0);
 #pragma unroll
-                for (int t = 1; t <= QL; ++t) w[t - 1][i] = load_at(L.a + P.lv.lo[lvl - t] + idx * P.lv.pw[P.qe - t], L.cqo[t - 1]);
+                for (int t = 1; t <= QL; ++t) w[t - 1][i] = T(0);
+                if (x < P.d) {      // wave-uniform
+                    if (L.live) e[i] = load_at(grow + idx * P.words, L.fo);
+#pragma unroll
+                    for (int t = 1; t <= QL; ++t) w[t - 1][i] = load_at(L.a + P.lv.lo[lvl - t] + idx * P.lv.pw[P.qe - t], L.cqo[t - 1]);
+                }
             }
 #pragma unroll
             for (int i = 0; i < kLeafBatch; ++i) {
