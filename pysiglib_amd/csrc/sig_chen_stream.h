@@ -389,13 +389,6 @@ struct RowsPlan {
     StreamLevels lv;
 };
 
-template <typename T>
-__device__ __forceinline__ T wave_sum(T v)
-{
-    for (int s = kWave >> 1; s; s >>= 1) v += __shfl_xor(v, s);
-    return v;
-}
-
 template <typename T, int DCEIL, int KT, int KS>
 __global__ __launch_bounds__(kBlock) void chen_adjoint_left_rows_kernel(
     const T* __restrict__ dC, T* __restrict__ dA, const T* __restrict__ B, int64_t batch, RowsPlan P, int64_t stride,

@@ -488,6 +488,14 @@ __device__ __forceinline__ void lds_add_shared(T* p, T v)
 }
 __device__ __forceinline__ void lds_add(double* p, double v) { lds_add_shared(p, v); }
 __device__ __forceinline__ void lds_add(float* p, float v) { *p += v; }
+// sum over the 64 lanes of a wave, in every lane
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+    for (int s = kWave >> 1; s; s >>= 1) v += __shfl_xor(v, s);
+    return v;
+}
+
 template <typename T>
 __device__ __forceinline__ void dev_add(T* p, T v)
 {

@@ -773,6 +773,36 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
 
 
 @pytest.mark.parametrize("shape,aug", [
+    ((3, 9, 2), {}), ((2, 30, 5), {}), ((4, 17, 16), dict(time_aug=True)), ((2, 21, 17), dict(lead_lag=True)),
+    ((3, 12, 33), dict(time_aug=True, lead_lag=True)), ((2, 2, 70), {}), ((2, 40, 64), {}), ((3, 25, 80), {}),
+    ((1, 9, 130), dict(time_aug=True)), ((1, 6, 256), {}), ((70, 5, 65), {})])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("scalar_term", [False, True])
+def test_degree_three_matrix_backward(P, oracle, shape, aug, dtype, scalar_term):
+    """The degree-3 backward as two library matrix products and a scan, forced onto narrow paths too, against the
+    oracle (its automatic range, 64 channels and more, is also covered by test_many_channel_shapes)."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_force_degree3.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_force_degree3.restype = None
+    b, length, d = shape
+    rng = np.random.default_rng(b * 1000 + d * 10 + length)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * 0.3).astype(dtype)
+    ref = oracle.signature(x, 3, n_jobs=-1, scalar_term=scalar_term, **aug)
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    want = oracle.sig_backprop(x, ref, g, 3, n_jobs=-1, **aug)
+    try:
+        L.CUSIG.cusig_amd_force_degree3(1)
+        got = P.sig_backprop(dev(x), dev(ref), dev(g), 3, **aug).cpu().numpy()
+        L.CUSIG.cusig_amd_force_degree3(0)
+        sweep = P.sig_backprop(dev(x), dev(ref), dev(g), 3, **aug).cpu().numpy()
+    finally:
+        L.CUSIG.cusig_amd_force_degree3(-1)
+    assert bwd_rel_err(got, want) <= TOL[dtype], shape
+    assert bwd_rel_err(sweep, want) <= TOL[dtype], shape
+
+
+@pytest.mark.parametrize("shape,aug", [
     ((3, 9, 2, 2), {}), ((2, 30, 5, 2), {}), ((4, 17, 16, 2), {}), ((2, 21, 17, 2), dict(time_aug=True)),
     ((2, 13, 31, 2), dict(lead_lag=True)), ((3, 12, 33, 2), dict(time_aug=True, lead_lag=True)), ((1, 2, 70, 2), {}),
     ((2, 700, 20, 2), {}),                      # few long paths: time slices adding into the output
