@@ -267,9 +267,9 @@ CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: the closed-form degree-2 kernels (matrix cores): -1 automatic, 0 never, 1 whenever the degree is 2. */
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) CUSIG_AMD_NOEXCEPT;
-/* Tuning hook: the degree-3 backward as two rocBLAS matrix products and a scan (any width):
- * -1 automatic (from 48 channels in float32, 36 in float64, enough paths to fill the chip, and librocblas can be
- * opened), 0 never, 1 whenever the degree is 3. */
+/* Tuning hook: degree 3 as rocBLAS matrix products around a scan kernel (backward: two products, forward: one):
+ * -1 automatic (backward from 48 channels in float32 and 36 in float64, forward from 112, given enough paths to fill
+ * the chip and a librocblas that can be opened), 0 never, 1 whenever the degree is 3. */
 CUSIG_AMD_API void cusig_amd_force_degree3(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: 1 routes every sweep of 2, 3 or 4 augmented channels that the run-time-degree kernels can serve
  * (degree >= 5, 4, 3 respectively) to them; by default they only serve degrees 17 .. 64. */

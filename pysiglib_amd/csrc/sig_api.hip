@@ -494,15 +494,16 @@ static Hook g_degree2_staged{1};    // tuning hook: 0 keeps the operands of the 
 static Hook g_force_degree3{-1};    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 3
 constexpr uint64_t kDeg3BufBytes = uint64_t(4) << 30;
 
-// degree-3 backward as two library matrix products and a scan (sig_degree3.h).  Measured against the sweep kernels at
+// degree 3 as library matrix products around a scan (sig_degree3.h): two products backward, one forward.  Measured against the sweep kernels at
 // batch 512, length 256: float32 1.3x faster from 48 channels (4.6x at 80, 11x at 128), float64 from 36 (10x at 80);
 // the scan needs a wave per SIMD to be worth it (a wave: 8 rows x 64 columns of one path's level 2).
-static bool want_degree3_gemm(uint64_t d_aug, uint64_t degree, uint64_t L, uint64_t batch, bool f64)
+static bool want_degree3_gemm(uint64_t d_aug, uint64_t degree, uint64_t L, uint64_t batch, bool f64, bool backward)
 {
     if (degree != 3 || d_aug < 2 || d_aug > uint64_t(kDeg3MaxDim) || L > 0x7fffffff) return false;
     if (g_force_degree3 >= 0) return g_force_degree3 != 0;
     const uint64_t waves = ((d_aug + kWave - 1) / kWave) * ((d_aug + kDeg3RowsPerThread - 1) / kDeg3RowsPerThread) * batch;
-    return d_aug >= (f64 ? 36u : 48u) && waves >= 1024;
+    const uint64_t from = backward ? (f64 ? 36u : 48u) : 112u;      // forward: 1.3x at 128 channels, slower at 80
+    return d_aug >= from && waves >= 1024;
 }
 
 static bool use_degree2(bool backward, uint64_t d_aug, uint64_t degree, uint64_t batch)
@@ -634,6 +635,33 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         hipLaunchKernelGGL((degree_one_fwd_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
                            path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), time_step, sc, flag);
+    } else if (want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, false) && rocblas_ready()) {
+        const int d = int(s.d_aug);
+        const int64_t L = int64_t(s.L);
+        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+        const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
+        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(batch, kDeg3BufBytes / per_path));
+        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+        T* rows = static_cast<T*>(workspace(19, checked_mul(chunk, per_path, "level-2 rows")));
+        compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
+        RocBlas::Handle h = rocblas_handle_for(stream);
+        tl_last_segments = 1;
+        MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree3_fwd_gemm_f64" : "degree3_fwd_gemm_f32");
+        const int64_t dd = int64_t(d) * d;
+        const int groups = (d + kDeg3RowsPerThread - 1) / kDeg3RowsPerThread;
+        for (uint64_t first = 0; first < batch; first += chunk) {
+            const int nb = int(std::min<uint64_t>(chunk, batch - first));
+            const dim3 sgrid(unsigned((d + kWave - 1) / kWave), unsigned(nb), unsigned((groups + kWavesPerBlock - 1) / kWavesPerBlock));
+            hipLaunchKernelGGL((degree3_fwd_scan_kernel<T>), sgrid, dim3(kBlock), 0, stream, (const T*)inc, rows, out, L, d,
+                               int64_t(s.stride), sc, int64_t(first));
+            // level 3 (row-major d^2 x d) = V^T Z; column-major: [d x d^2] = Z^T (stored: d x L) * (V^T stored: d^2 x L)^T
+            gemm_col_major<T>(h, false, true, d, int(dd), int(L), inc + (first * (s.L + 2) + 1) * s.d_aug, d, (L + 2) * d,
+                              (const T*)rows, int(dd), L * dd, T(0), out + first * s.stride + sc + d + dd, d, int64_t(s.stride), nb);
+        }
+        timer.stop();
+        if (flag)
+            hipLaunchKernelGGL((finite_rows_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
+                               int64_t(batch * s.stride), flag);
     } else if (use_degree2(false, s.d_aug, degree, batch)) {
         const int d = int(s.d_aug);
         const int tiles = (d + 15) / 16, col_groups = (tiles + kDeg2Cols - 1) / kDeg2Cols;
@@ -865,7 +893,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
     auto finish = [&] { if (!arena) exit_sync(stream); };
     std::unique_lock<std::mutex> lk(g_ws_mutex, std::defer_lock);
     auto lock_pool = [&] { if (!arena && !lk.owns_lock()) lk.lock(); };
-    bool degree3 = !arena && s.len_aug > 1 && want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8);
+    bool degree3 = !arena && s.len_aug > 1 && want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, true);
     if (degree3) {
         lock_pool();
         degree3 = rocblas_ready();

@@ -76,20 +76,30 @@ static RocBlas::Handle rocblas_handle_for(hipStream_t stream)
     return h;
 }
 
-// row-major C[m x n] (ldc) = alpha * A[m x k] * op(B) + beta * C, batched; op(B) = B[k x n] or B^T with B[n x k]
+// rocBLAS strided-batched gemm as the library defines it (column-major): C[m x n] = op(A) op(B) + beta C
 template <typename T>
-static void gemm_row_major(RocBlas::Handle h, bool b_transposed, int m, int n, int k, const T* A, int lda, int64_t sa,
-                           const T* B, int ldb, int64_t sb, T beta, T* C, int ldc, int64_t sc, int batches)
+static void gemm_col_major(RocBlas::Handle h, bool a_transposed, bool b_transposed, int m, int n, int k, const T* A, int lda,
+                           int64_t sa, const T* B, int ldb, int64_t sb, T beta, T* C, int ldc, int64_t sc, int batches)
 {
     const T alpha = T(1);
     constexpr int kNone = 111, kTrans = 112;
     int rc;
-    // column-major view: C^T[n x m] = op(B)^T A^T
     if constexpr (sizeof(T) == 8)
-        rc = g_rocblas.dgemm(h, b_transposed ? kTrans : kNone, kNone, n, m, k, &alpha, B, ldb, sb, A, lda, sa, &beta, C, ldc, sc, batches);
+        rc = g_rocblas.dgemm(h, a_transposed ? kTrans : kNone, b_transposed ? kTrans : kNone, m, n, k, &alpha, A, lda, sa, B, ldb, sb,
+                             &beta, C, ldc, sc, batches);
     else
-        rc = g_rocblas.sgemm(h, b_transposed ? kTrans : kNone, kNone, n, m, k, &alpha, B, ldb, sb, A, lda, sa, &beta, C, ldc, sc, batches);
-    if (rc != 0) throw std::runtime_error("sig_backprop_cuda: rocBLAS gemm failed (status " + std::to_string(rc) + ")");
+        rc = g_rocblas.sgemm(h, a_transposed ? kTrans : kNone, b_transposed ? kTrans : kNone, m, n, k, &alpha, A, lda, sa, B, ldb, sb,
+                             &beta, C, ldc, sc, batches);
+    if (rc != 0) throw std::runtime_error("rocBLAS gemm failed (status " + std::to_string(rc) + ")");
+}
+
+// row-major C[m x n] (ldc) = A[m x k] * op(B) + beta * C, batched; op(B) = B[k x n] or B^T with B[n x k].
+// Column-major view: C^T[n x m] = op(B)^T A^T
+template <typename T>
+static void gemm_row_major(RocBlas::Handle h, bool b_transposed, int m, int n, int k, const T* A, int lda, int64_t sa,
+                           const T* B, int ldb, int64_t sb, T beta, T* C, int ldc, int64_t sc, int batches)
+{
+    gemm_col_major<T>(h, b_transposed, false, n, m, k, B, ldb, sb, A, lda, sa, beta, C, ldc, sc, batches);
 }
 
 // ---- the scan ------------------------------------------------------------------------------------------------------
@@ -193,6 +203,58 @@ __global__ __launch_bounds__(kBlock) void degree3_scan_kernel(
         wave_sum_many(sums, lane);
         if (row_writer) dev_add(row_dst + t * d, sums[0]);
     }
+}
+
+// Forward: S3 = sum_t V_t (x) z_t = V^T Z with the same V_t = S2 + S1 (x) z_t / 2 + z_t (x) z_t / 6 (state before step
+// t).  This scan walks the steps forwards, writes V ([path][L][d * d]) and leaves levels 1 and 2 (and the scalar term)
+// in the output row; the product fills level 3.  Same grid as degree3_scan_kernel; no sums across lanes.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void degree3_fwd_scan_kernel(const T* __restrict__ inc, T* __restrict__ buf,
+                                                                  T* __restrict__ out, int64_t L, int d, int64_t out_stride,
+                                                                  int scalar, int64_t first_path)
+{
+    constexpr int R = kDeg3RowsPerThread;
+    const int lane = threadIdx.x & (kWave - 1), w = int(blockIdx.z) * kWavesPerBlock + int(threadIdx.x >> 6);
+    const int j = blockIdx.x * kWave + lane;
+    const bool jon = j < d;
+    const int64_t pl = blockIdx.y, pg = first_path + pl;
+    const T* z_rows = inc + (pg * (L + 2) + 1) * d;
+    T* V = buf + pl * L * int64_t(d) * d;
+    T* O = out + pg * out_stride + scalar;
+    const int i0 = w * R;
+    if (i0 >= d) return;
+    T s2[R], s1[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        s2[r] = T(0);
+        s1[r] = T(0);
+    }
+    T s1j = T(0);
+    T zj = jon ? z_rows[j] : T(0);
+    for (int64_t t = 0; t < L; ++t) {
+        const T* z = z_rows + t * d;
+        T* Vt = V + t * int64_t(d) * d;
+        const T zn = (jon && t + 1 < L) ? z[d + j] : T(0);      // next step's increment, in flight during this one
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = i0 + r;
+            if (i < d) {                                        // wave-uniform
+                const T zi = z[i];
+                if (jon) Vt[i * d + j] = fmadd(s1[r] * T(0.5) + zi * T(1.0 / 6.0), zj, s2[r]);
+                s2[r] = fmadd(s1[r] + zi * T(0.5), zj, s2[r]);
+                s1[r] += zi;
+            }
+        }
+        s1j += zj;
+        zj = zn;
+    }
+    if (jon) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (i0 + r < d) O[d + (i0 + r) * d + j] = s2[r];
+        if (i0 == 0) O[j] = s1j;
+    }
+    if (scalar && i0 == 0 && j == 0) out[pg * out_stride] = T(1);
 }
 
 // dz[t][m] += a1 after step t;  a1 runs backwards: a1 <- a1 + r1[t].  One thread per (path, m).

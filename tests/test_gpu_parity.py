@@ -778,9 +778,9 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
     ((1, 9, 130), dict(time_aug=True)), ((1, 6, 256), {}), ((70, 5, 65), {})])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_degree_three_matrix_backward(P, oracle, shape, aug, dtype, scalar_term):
-    """The degree-3 backward as two library matrix products and a scan, forced onto narrow paths too, against the
-    oracle (its automatic range, 64 channels and more, is also covered by test_many_channel_shapes)."""
+def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
+    """Degree 3 as library matrix products around a scan (forward: one product, backward: two), forced onto narrow
+    paths too, against the oracle; the sweep kernels' backward on the same inputs beside it."""
     import ctypes
     from pysiglib_amd import _loader as L
     L.CUSIG.cusig_amd_force_degree3.argtypes = (ctypes.c_int,)
@@ -793,11 +793,18 @@ def test_degree_three_matrix_backward(P, oracle, shape, aug, dtype, scalar_term)
     want = oracle.sig_backprop(x, ref, g, 3, n_jobs=-1, **aug)
     try:
         L.CUSIG.cusig_amd_force_degree3(1)
+        fwd = P.sig(dev(x), 3, scalar_term=scalar_term, **aug).cpu().numpy()
+        assert L.CUSIG.cusig_amd_last_sig_nonfinite() == 0
         got = P.sig_backprop(dev(x), dev(ref), dev(g), 3, **aug).cpu().numpy()
         L.CUSIG.cusig_amd_force_degree3(0)
         sweep = P.sig_backprop(dev(x), dev(ref), dev(g), 3, **aug).cpu().numpy()
     finally:
         L.CUSIG.cusig_amd_force_degree3(-1)
+    d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+    off = 1 if scalar_term else 0
+    assert level_rel_err(fwd[:, off:], ref[:, off:], d_aug, 3) <= TOL[dtype], shape
+    if scalar_term:
+        assert np.all(fwd[:, 0] == 1)
     assert bwd_rel_err(got, want) <= TOL[dtype], shape
     assert bwd_rel_err(sweep, want) <= TOL[dtype], shape
 
