@@ -628,7 +628,7 @@ static inline bool make_rows_plan(RowsPlan& P, uint64_t d, uint64_t degree, uint
     P.dmul = dv.mul;
     P.dshr = dv.shr;
     const uint64_t moved = uint64_t(P.targets) * d;
-    P.upb = int(std::max<uint64_t>(1, std::min<uint64_t>((4 * uint64_t(P.bs) + moved - 1) / moved, P.units)));
+    P.upb = int(std::max<uint64_t>(1, std::min<uint64_t>((16 * uint64_t(P.bs) + moved - 1) / moved, P.units)));
     return true;
 }
 

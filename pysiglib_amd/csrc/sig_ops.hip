@@ -446,15 +446,17 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     T* E = static_cast<T*>(workspace(4, bytes));
     T* dE = static_cast<T*>(workspace(5, bytes));
-    with_chen_fan(dimension, [&](auto fan) {
-        constexpr int FAN = decltype(fan)::value;
-        const uint64_t items = chen_items(dimension, degree, FAN);
-        launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
-            using I = decltype(ix);
-            hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
-                               DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+    // exp(z) up to level degree - 1: the adjoint never multiplies with a factor's top level
+    if (degree >= 2)
+        with_chen_fan(dimension, [&](auto fan) {
+            constexpr int FAN = decltype(fan)::value;
+            const uint64_t items = chen_items(dimension, degree - 1, FAN);
+            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+                using I = decltype(ix);
+                hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, E, int64_t(batch),
+                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+            });
         });
-    });
     // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
     if (prepend) launch_combine_bwd<T>(d_out, dE, d_sig, (const T*)E, sig, batch, dimension, degree, s, stream);
     else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream);
