@@ -640,7 +640,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         const int64_t L = int64_t(s.L);
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
-        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(batch, kDeg3BufBytes / per_path));
+        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(batch, 65535), kDeg3BufBytes / per_path));
         T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
         T* rows = static_cast<T*>(workspace(19, checked_mul(chunk, per_path, "level-2 rows")));
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
@@ -913,7 +913,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
         const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
-        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(batch, kDeg3BufBytes / per_path));
+        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(batch, 65535), kDeg3BufBytes / per_path));
         T* inc = static_cast<T*>(buffer(0, checked_mul(inc_elems, sizeof(T), "increments")));
         T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
         T* r1 = static_cast<T*>(buffer(18, checked_mul(dz_elems, sizeof(T), "increments")));

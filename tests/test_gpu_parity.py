@@ -775,7 +775,7 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
 @pytest.mark.parametrize("shape,aug", [
     ((3, 9, 2), {}), ((2, 30, 5), {}), ((4, 17, 16), dict(time_aug=True)), ((2, 21, 17), dict(lead_lag=True)),
     ((3, 12, 33), dict(time_aug=True, lead_lag=True)), ((2, 2, 70), {}), ((2, 40, 64), {}), ((3, 25, 80), {}),
-    ((1, 9, 130), dict(time_aug=True)), ((1, 6, 256), {}), ((70, 5, 65), {})])
+    ((1, 9, 130), dict(time_aug=True)), ((1, 6, 256), {}), ((70, 5, 65), {}), ((70000, 3, 2), {})])      # the last: more paths than a grid dimension holds
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
 def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
@@ -786,6 +786,9 @@ def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
     L.CUSIG.cusig_amd_force_degree3.argtypes = (ctypes.c_int,)
     L.CUSIG.cusig_amd_force_degree3.restype = None
     b, length, d = shape
+    if b > 60000 and dtype == np.float32:
+        pytest.skip("among 70000 two-step paths some nearly close: level 3 cancels to 1e-6 and every float32 "
+                    "implementation (the oracle's and the sweep kernels' included) is 2-3e-4 off the float64 value")
     rng = np.random.default_rng(b * 1000 + d * 10 + length)
     x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * 0.3).astype(dtype)
     ref = oracle.signature(x, 3, n_jobs=-1, scalar_term=scalar_term, **aug)
