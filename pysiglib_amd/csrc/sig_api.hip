@@ -261,6 +261,7 @@ static void release_workspaces() noexcept
     }
     g_ws.clear();
     g_dz.clear();
+    rocblas_release();
     if (g_flag_host) {
         (void)hipHostFree(g_flag_host);
         g_flag_host = nullptr;

@@ -35,6 +35,7 @@ constexpr int kDeg3MaxDim = 1024;
 struct RocBlas {
     using Handle = void*;
     int (*create)(Handle*) = nullptr;
+    int (*destroy)(Handle) = nullptr;
     int (*set_stream)(Handle, hipStream_t) = nullptr;
     int (*sgemm)(Handle, int, int, int, int, int, const float*, const float*, int, int64_t, const float*, int, int64_t,
                  const float*, float*, int, int64_t, int) = nullptr;
@@ -54,6 +55,7 @@ static bool rocblas_ready()
         if (!lib) lib = dlopen("librocblas.so", RTLD_NOW | RTLD_LOCAL);
         if (lib) {
             r.create = reinterpret_cast<decltype(r.create)>(dlsym(lib, "rocblas_create_handle"));
+            r.destroy = reinterpret_cast<decltype(r.destroy)>(dlsym(lib, "rocblas_destroy_handle"));
             r.set_stream = reinterpret_cast<decltype(r.set_stream)>(dlsym(lib, "rocblas_set_stream"));
             r.sgemm = reinterpret_cast<decltype(r.sgemm)>(dlsym(lib, "rocblas_sgemm_strided_batched"));
             r.dgemm = reinterpret_cast<decltype(r.dgemm)>(dlsym(lib, "rocblas_dgemm_strided_batched"));
@@ -91,6 +93,20 @@ static void gemm_col_major(RocBlas::Handle h, bool a_transposed, bool b_transpos
         rc = g_rocblas.sgemm(h, a_transposed ? kTrans : kNone, b_transposed ? kTrans : kNone, m, n, k, &alpha, A, lda, sa, B, ldb, sb,
                              &beta, C, ldc, sc, batches);
     if (rc != 0) throw std::runtime_error("rocBLAS gemm failed (status " + std::to_string(rc) + ")");
+}
+
+// gives the handles (and the device memory they hold) back; the library stays loaded.  Caller holds the workspace mutex.
+static void rocblas_release() noexcept
+{
+    for (auto& kv : g_rocblas.handles) {
+        if (!kv.second || !g_rocblas.destroy) continue;
+        int cur = 0;
+        if (hipGetDevice(&cur) == hipSuccess && hipSetDevice(kv.first) == hipSuccess) {
+            (void)g_rocblas.destroy(kv.second);
+            (void)hipSetDevice(cur);
+        }
+    }
+    g_rocblas.handles.clear();
 }
 
 // row-major C[m x n] (ldc) = A[m x k] * op(B) + beta * C, batched; op(B) = B[k x n] or B^T with B[n x k].

@@ -46,15 +46,17 @@ __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
 
 // after the adjoint of x (x) P_{k+1} (tmpA w.r.t. x, tmpB w.r.t. P_{k+1}):
 //   g_next = -tmpB,   dx += -tmpA + g_next / (k + 1)      over the `count` coefficients of levels <= N - k + 1
+// `first` (the k = 1 update, which covers every coefficient): dx starts from g, so that no separate pass copies it
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void tensor_log_bwd_update_kernel(
-    T* __restrict__ dx, T* __restrict__ g_next, const T* __restrict__ tmpA, const T* __restrict__ tmpB, int64_t batch,
+    T* dx, const T* first, T* __restrict__ g_next, const T* __restrict__ tmpA, const T* __restrict__ tmpB, int64_t batch,
     I count, I count_next, T inv_next, int64_t stride, int off)
 {
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const int64_t base = b * stride + off;
         for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < count; r += I(gridDim.x) * kBlock) {
-            T v = dx[base + r] - tmpA[base + r];
+            if (first && off && r == 0) dx[b * stride] = T(0);
+            T v = (first ? first[base + r] : dx[base + r]) - tmpA[base + r];
             if (r < count_next) {
                 const T gn = -tmpB[base + r];
                 g_next[base + r] = gn;
@@ -311,11 +313,12 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
     }
     // P_1 (discarded), P_2 .. P_N, two adjoint buffers, two product-adjoint buffers
     T* ws = degree >= 2 ? static_cast<T*>(workspace(7, checked_mul(bytes, degree + 4, "workspace"))) : nullptr;
-    launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
-        using I = decltype(ix);
-        hipLaunchKernelGGL((tensor_log_bwd_init_kernel<T, I>), grid, dim3(kBlock), 0, stream, out, derivs, int64_t(batch),
-                           I(s.n_coef), int64_t(s.stride), s.off);
-    });
+    if (degree < 2)
+        launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((tensor_log_bwd_init_kernel<T, I>), grid, dim3(kBlock), 0, stream, out, derivs, int64_t(batch),
+                               I(s.n_coef), int64_t(s.stride), s.off);
+        });
     if (degree >= 2) {
         T* p_base = ws;                                   // P_k at p_base + (k - 1) * elems
         T* g_buf[2] = {ws + degree * elems, ws + (degree + 1) * elems};
@@ -331,7 +334,8 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
             const uint64_t count = sk.n_coef, count_next = coef_count(dimension, top - 1);
             launch_indexed(s.n_coef, count, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
-                hipLaunchKernelGGL((tensor_log_bwd_update_kernel<T, I>), grid, dim3(kBlock), 0, stream, out, g_next,
+                hipLaunchKernelGGL((tensor_log_bwd_update_kernel<T, I>), grid, dim3(kBlock), 0, stream, out,
+                                   k == 1 ? derivs : static_cast<const T*>(nullptr), g_next,
                                    (const T*)tmpA, (const T*)tmpB, int64_t(batch), I(count), I(count_next), T(1) / T(k + 1),
                                    int64_t(s.stride), s.off);
             });
