@@ -170,6 +170,20 @@ def test_combine_backprop_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, 
     assert row_rel_err(d2.cpu().numpy(), w2) < TOL[dtype]
 
 
+@pytest.mark.parametrize("d,deg,batch", [(2, 20, 1), (3, 12, 2), (4, 10, 1), (6, 8, 1), (12, 6, 1), (33, 4, 1), (100, 3, 2)])
+def test_combine_backprop_long_rows(P, oracle, d, deg, batch):
+    """Rows of 0.8-3.3 million coefficients: the streaming adjoint kernels with several levels of words above a
+    block's own (deep signatures of few channels) and the wide-path kernel (more than 32 channels)."""
+    rng = np.random.default_rng(11 * d + deg)
+    n = oracle.sig_length(d, deg) - 1
+    scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
+    a, b, g = (rng.standard_normal((batch, n)) * scale for _ in range(3))
+    w1, w2 = oracle.sig_combine_backprop(g, a, b, d, deg)
+    d1, d2 = P.sig_combine_backprop(dev(g), dev(a), dev(b), d, deg)
+    assert row_rel_err(d1.cpu().numpy(), w1) < TOL[np.float64]
+    assert row_rel_err(d2.cpu().numpy(), w2) < TOL[np.float64]
+
+
 def test_combine_autograd(P):
     d, deg = 3, 4
     n = P.sig_length(d, deg)
