@@ -37,15 +37,26 @@ struct SharedRows {
     int off = 0;
 };
 
+// B = exp(z) and the caller wants dz (zeroed beforehand) rather than dB: the right factor's kernel may add the terms
+// of the levels above `level` straight into dz.  On return dB holds, at `level`, the row on which the adjoint of exp
+// truncated at `level` gives the remaining terms (levels above it are not written); level = degree: nothing folded.
+template <typename T>
+struct ExpFold {
+    const T* z = nullptr;   // (batch, dimension)
+    T* dz = nullptr;
+    int level = 0;
+};
+
 // launches the adjoint of the Chen product on `stream` (defined in sig_chen_adjoint.hip for float and double).
 // identity = 0 drops the dC_t[w] terms; families = 1 computes dA only (dB and A are not touched)
 template <typename T>
 void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint64_t batch, uint64_t dimension,
                         uint64_t degree, const SigShape& s, hipStream_t stream, int identity = 1,
-                        SharedRows dc = SharedRows(), int families = 2);
+                        SharedRows dc = SharedRows(), int families = 2, ExpFold<T>* fold = nullptr);
 extern template void launch_combine_bwd<float>(const float*, float*, float*, const float*, const float*, uint64_t, uint64_t,
-                                               uint64_t, const SigShape&, hipStream_t, int, SharedRows, int);
+                                               uint64_t, const SigShape&, hipStream_t, int, SharedRows, int, ExpFold<float>*);
 extern template void launch_combine_bwd<double>(const double*, double*, double*, const double*, const double*, uint64_t,
-                                                uint64_t, uint64_t, const SigShape&, hipStream_t, int, SharedRows, int);
+                                                uint64_t, uint64_t, const SigShape&, hipStream_t, int, SharedRows, int,
+                                                ExpFold<double>*);
 
 }  // namespace sigamd

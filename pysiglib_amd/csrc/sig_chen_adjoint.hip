@@ -164,26 +164,50 @@ static void launch_combine_bwd_items(const T* dC, T* dA, T* dB, const T* A, cons
     });
 }
 
+// LDS of the right factor's kernel when it folds exp(z): one slot per lane and letter
+template <typename T>
+static bool right_fold_fits(uint64_t dimension)
+{
+    return dimension * uint64_t(kBlock) * sizeof(T) <= uint64_t(64) << 10;
+}
+
 template <typename T, int QL = 0, int REL = 1>
 static void launch_right_stream(const RightPlan& rp, const T* dC, T* dB, const T* A, uint64_t batch, const SigShape& s,
-                                hipStream_t stream, int identity, const SharedRows& dc)
+                                hipStream_t stream, int identity, const SharedRows& dc, const ExpFold<T>* fold)
 {
     if constexpr (QL <= kRightMaxLow && REL <= kRightMaxRel) {
-        if (rp.qe - 1 != QL) return launch_right_stream<T, QL + 1, REL>(rp, dC, dB, A, batch, s, stream, identity, dc);
-        if (rp.rel != REL) return launch_right_stream<T, QL, REL + 1>(rp, dC, dB, A, batch, s, stream, identity, dc);
+        if (rp.qe - 1 != QL) return launch_right_stream<T, QL + 1, REL>(rp, dC, dB, A, batch, s, stream, identity, dc, fold);
+        if (rp.rel != REL) return launch_right_stream<T, QL, REL + 1>(rp, dC, dB, A, batch, s, stream, identity, dc, fold);
         const uint64_t waves = (uint64_t(rp.words) + kWave - 1) / kWave;
         const dim3 grid{unsigned((waves + kWavesPerBlock - 1) / kWavesPerBlock), unsigned(std::min<uint64_t>(batch, 65535)), 1};
-        hipLaunchKernelGGL((chen_adjoint_right_kernel<T, QL, REL>), grid, dim3(kBlock), 0, stream, dC, dB, A, int64_t(batch),
-                           rp, int64_t(s.stride), s.off, identity, dc.share, dc.stride, dc.off);
+        FoldScale<T> fs{};
+        if (fold) {
+            double fact = 1.0;
+            for (int t = 1; t <= rp.qe; ++t) fact *= double(t);
+            for (int D = 0; D <= REL; ++D) {
+                if (D) fact *= double(rp.qe + D);
+                fs.inv_level[D] = T(1.0 / double(rp.qe + D));
+                fs.inv_fact[D] = T(1.0 / fact);
+            }
+            hipLaunchKernelGGL((chen_adjoint_right_kernel<T, QL, REL, true>), grid, dim3(kBlock),
+                               size_t(rp.d) * kBlock * sizeof(T), stream, dC, dB, A, int64_t(batch), rp, int64_t(s.stride), s.off,
+                               identity, dc.share, dc.stride, dc.off, fold->z, fold->dz, fs);
+        } else {
+            hipLaunchKernelGGL((chen_adjoint_right_kernel<T, QL, REL, false>), grid, dim3(kBlock), 0, stream, dC, dB, A,
+                               int64_t(batch), rp, int64_t(s.stride), s.off, identity, dc.share, dc.stride, dc.off,
+                               (const T*)nullptr, (T*)nullptr, fs);
+        }
     }
 }
 
 // launches the adjoint of the Chen product on `stream`
 template <typename T>
 void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint64_t batch, uint64_t dimension,
-                        uint64_t degree, const SigShape& s, hipStream_t stream, int identity, SharedRows dc, int families)
+                        uint64_t degree, const SigShape& s, hipStream_t stream, int identity, SharedRows dc, int families,
+                        ExpFold<T>* fold)
 {
     if (dc.stride < 0) { dc.stride = int64_t(s.stride); dc.off = s.off; }
+    if (fold) fold->level = int(degree);
     if (degree > uint64_t(kCombMaxLevels)) throw std::runtime_error("sig_combine_backprop_cuda: degree too high");
     const int mode = g_chen_adjoint_mode;
     const bool streaming = mode != 2 && (mode == 1 || s.n_coef >= kStreamMinCoef) && dimension >= 2 && degree >= 2 &&
@@ -258,13 +282,16 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
     } else {
         if (rp.qe >= 2)
             launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, uint64_t(rp.qe - 1), s, stream, identity, dc, 1, 1);
-        launch_right_stream<T>(rp, dC, dB, A, batch, s, stream, identity, dc);
+        const bool folding = fold && identity == 1 && rp.rel >= 1 && right_fold_fits<T>(dimension);
+        if (folding) fold->level = rp.qe;
+        launch_right_stream<T>(rp, dC, dB, A, batch, s, stream, identity, dc, folding ? fold : nullptr);
     }
 }
 
 template void launch_combine_bwd<float>(const float*, float*, float*, const float*, const float*, uint64_t, uint64_t,
-                                        uint64_t, const SigShape&, hipStream_t, int, SharedRows, int);
+                                        uint64_t, const SigShape&, hipStream_t, int, SharedRows, int, ExpFold<float>*);
 template void launch_combine_bwd<double>(const double*, double*, double*, const double*, const double*, uint64_t,
-                                         uint64_t, uint64_t, const SigShape&, hipStream_t, int, SharedRows, int);
+                                         uint64_t, uint64_t, const SigShape&, hipStream_t, int, SharedRows, int,
+                                         ExpFold<double>*);
 
 }  // namespace sigamd

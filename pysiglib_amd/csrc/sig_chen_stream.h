@@ -78,6 +78,18 @@ struct RightLane {
     uint32_t cqo[QL > 0 ? QL : 1];      // the same as byte offsets
     T low[QL > 0 ? QL : 1];
     T acc[kRightMaxRel + 1];
+    // folding with exp(z) as the right factor (FOLD): see chen_adjoint_right_kernel
+    const T* z;                         // displacement of the row
+    T* slot;                            // the lane's own d partial sums in LDS, kBlock entries apart
+    T kacc[kRightMaxRel + 2];           // kacc[D]: sum over the visited children x of the node at depth D - 1
+    T zp[kRightMaxRel + 1];             // product of z over the letters of the word at depth D
+};
+
+// 1 / level and 1 / level! of the words at depth D of the walk (level = qe + D)
+template <typename T>
+struct FoldScale {
+    T inv_level[kRightMaxRel + 1];
+    T inv_fact[kRightMaxRel + 1];
 };
 
 #ifndef SIGAMD_LEAF_BATCH
@@ -89,14 +101,16 @@ constexpr int kLeafBatch = SIGAMD_LEAF_BATCH;       // loads of the deepest leve
 // pfx[i] the index of its first i letters.  The deepest level issues its loads kLeafBatch at a time, and an inner
 // level loads the entry of its next word before it walks below the current one: a lane's loads would otherwise
 // pay their latency one after the other.
-template <typename T, int QL, int REL, int DEPTH>
-__device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPlan& P, uint32_t widx,
+template <typename T, int QL, int REL, bool FOLD, int DEPTH>
+__device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPlan& P, const FoldScale<T>& F, uint32_t widx,
                                               const uint32_t (&pfx)[kRightMaxRel + 1])
 {
     const int lvl = P.qe + DEPTH;
     const T* grow = L.g + P.lv.lo[lvl];
     T* orow = L.out + P.lv.lo[lvl];
     if constexpr (DEPTH == REL) {
+        [[maybe_unused]] T zq = T(0);
+        if constexpr (FOLD) zq = L.zp[DEPTH - 1] * F.inv_fact[DEPTH];
         for (uint32_t x0 = 0; x0 < P.d; x0 += kLeafBatch) {
             T e[kLeafBatch];
             T w[QL > 0 ? QL : 1][kLeafBatch];
@@ -126,7 +140,12 @@ __device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPl
                     }
 #pragma unroll
                     for (int t = 1; t <= QL; ++t) L.low[t - 1] = fmadd(w[t - 1][i], e[i], L.low[t - 1]);
-                    if (L.live) store_at(orow + idx * P.words, L.fo, L.identity ? e[i] : T(0));
+                    if constexpr (FOLD) {
+                        L.kacc[DEPTH] = fmadd(L.z[x] * F.inv_level[DEPTH], e[i], L.kacc[DEPTH]);
+                        lds_add(L.slot + x * kBlock, e[i] * zq);
+                    } else {
+                        if (L.live) store_at(orow + idx * P.words, L.fo, L.identity ? e[i] : T(0));
+                    }
                 }
             }
         }
@@ -141,27 +160,52 @@ __device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPl
 #pragma unroll
             for (int i = 1; i <= DEPTH; ++i) np[i] = x * P.lv.pw[i - 1] + pfx[i - 1];
             L.acc[DEPTH] = L.identity ? e : T(0);
+            [[maybe_unused]] T zx = T(0);
+            if constexpr (FOLD) {
+                zx = L.z[x];
+                L.zp[DEPTH] = L.zp[DEPTH - 1] * zx;
+                L.kacc[DEPTH + 1] = T(0);
+            }
 #pragma unroll
             for (int j = 0; j < DEPTH; ++j) L.acc[j] = fmadd(L.a[P.lv.lo[DEPTH - j] + np[DEPTH - j]], e, L.acc[j]);
 #pragma unroll
             for (int t = 1; t <= QL; ++t)
                 L.low[t - 1] = fmadd(load_at(L.a + P.lv.lo[lvl - t] + idx * P.lv.pw[P.qe - t], L.cqo[t - 1]), e, L.low[t - 1]);
-            right_descend<T, QL, REL, DEPTH + 1>(L, P, idx, np);
-            if (L.live) store_at(orow + idx * P.words, L.fo, L.acc[DEPTH]);
+            right_descend<T, QL, REL, FOLD, DEPTH + 1>(L, P, F, idx, np);
+            if constexpr (FOLD) {
+                const T k = L.acc[DEPTH] + L.kacc[DEPTH + 1];
+                L.kacc[DEPTH] = fmadd(zx * F.inv_level[DEPTH], k, L.kacc[DEPTH]);
+                lds_add(L.slot + x * kBlock, k * (L.zp[DEPTH - 1] * F.inv_fact[DEPTH]));
+            } else {
+                if (L.live) store_at(orow + idx * P.words, L.fo, L.acc[DEPTH]);
+            }
             e = en;
         }
     }
 }
 
 // grid: x over the waves of a row (4 per block), y over the rows
-template <typename T, int QL, int REL>
+//
+// FOLD: B = exp(z) and the caller wants dz, not dB (sig_join_backprop, siglib/cpsig/cp_sig_join.h:36-238).  With
+//   K_t[v] = dB_t[v] + 1/(t+1) sum_a z[a] K_{t+1}[a v]      (K_N = dB_N)
+// the adjoint of z -> exp(z) is dz[a] = sum_t 1/t! <K_t[a .], z^(t-1)>: a word's K sums over the letters in front of
+// it, which is the order of the walk, so K_t for t > qe never leaves the lane.  Its terms go into dz here (a private
+// LDS slot per lane and letter, summed over the wave at the end of a row, then one atomic per wave and letter);
+// level qe of dB receives K_qe, levels below it dB itself as without FOLD, and the caller finishes with the adjoint of
+// exp truncated at level qe on that row.  Needs identity = 1 and d * kBlock entries of dynamic LDS.
+template <typename T, int QL, int REL, bool FOLD>
 __global__ __launch_bounds__(kBlock) void chen_adjoint_right_kernel(
     const T* __restrict__ dC, T* __restrict__ dB, const T* __restrict__ A, int64_t batch, RightPlan P, int64_t stride,
-    int off, int identity, int64_t dc_share, int64_t dc_stride, int dc_off)
+    int off, int identity, int64_t dc_share, int64_t dc_stride, int dc_off, const T* __restrict__ Z, T* __restrict__ dz,
+    FoldScale<T> F)
 {
+    extern __shared__ double right_lds_raw[];
     const Block2 blk = xcd_block_2d();
     const uint32_t wave = blk.x * kWavesPerBlock + (threadIdx.x >> 6);
     if (wave * kWave >= P.words) return;
+    [[maybe_unused]] T* slot = reinterpret_cast<T*>(right_lds_raw) + threadIdx.x;
+    if constexpr (FOLD)
+        for (uint32_t x = 0; x < P.d; ++x) slot[x * kBlock] = T(0);
     for (int64_t b = blk.y; b < batch; b += gridDim.y) {
         RightLane<T, QL> L;
         L.g = dC + (b / dc_share) * dc_stride + dc_off;
@@ -184,8 +228,29 @@ __global__ __launch_bounds__(kBlock) void chen_adjoint_right_kernel(
         L.acc[0] = identity ? e : T(0);
 #pragma unroll
         for (int t = 1; t <= QL; ++t) L.low[t - 1] = fmadd(L.a[P.lv.lo[P.qe - t] + L.cq[t - 1]], e, L.low[t - 1]);
+        if constexpr (FOLD) {
+            L.z = Z + b * int64_t(P.d);
+            L.slot = slot;
+            T prod = T(1);
+            uint32_t rest = L.f;
+            for (int i = 0; i < P.qe; ++i) {
+                const uint32_t q = rest / P.d;
+                prod *= L.z[rest - q * P.d];
+                rest = q;
+            }
+            L.zp[0] = prod;
+            L.kacc[1] = T(0);
+        }
         const uint32_t root[kRightMaxRel + 1] = {0, 0, 0, 0, 0};
-        right_descend<T, QL, REL, 1>(L, P, 0u, root);
+        right_descend<T, QL, REL, FOLD, 1>(L, P, F, 0u, root);
+        if constexpr (FOLD) {
+            L.acc[0] += L.kacc[1];
+            for (uint32_t x = 0; x < P.d; ++x) {
+                const T v = wave_sum(slot[x * kBlock]);
+                slot[x * kBlock] = T(0);
+                if ((threadIdx.x & (kWave - 1)) == 0) dev_add(dz + b * int64_t(P.d) + x, v);
+            }
+        }
         if (L.live) {
             L.out[pos] = L.acc[0];
 #pragma unroll

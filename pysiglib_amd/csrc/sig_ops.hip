@@ -457,9 +457,15 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
                                    DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
             });
         });
-    // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor
+    // the Chen product's adjoint with exp(z) as the right (append) or left (prepend) factor; as the right factor its
+    // kernel may fold the levels above `top` into d_disp, and the adjoint of exp below then stops at `top`
+    ExpFold<T> fold;
+    fold.z = disp;
+    fold.dz = d_disp;
+    fold.level = int(degree);
     if (prepend) launch_combine_bwd<T>(d_out, dE, d_sig, (const T*)E, sig, batch, dimension, degree, s, stream);
-    else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream);
+    else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream, 1, SharedRows(), 2, &fold);
+    const uint64_t top = uint64_t(fold.level);
     if (dimension == 1) {
         hipLaunchKernelGGL((exp_pullback_dim_one_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, (const T*)dE, disp,
                            d_disp, int64_t(batch), int64_t(degree), int64_t(s.stride), s.off);
@@ -468,7 +474,7 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
         const int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(32, uint64_t(kExpAccMax) / dimension))) : 1;
         with_chen_fan(dimension, [&](auto fan) {
             constexpr int FAN = decltype(fan)::value;
-            const uint64_t items = chen_items(dimension, degree, FAN);
+            const uint64_t items = chen_items(dimension, top, FAN);
             // a few items per thread, so that a block's LDS partial sums amortise their flush
             launch_indexed(s.n_coef, (items + 3) / 4, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
@@ -479,9 +485,9 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
                                        d_disp, int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, use_lds,
                                        copies);
                 };
-                if (degree <= 5) go(IntC<4>{});
-                else if (degree <= 9) go(IntC<8>{});
-                else if (degree <= 17) go(IntC<16>{});
+                if (top <= 5) go(IntC<4>{});
+                else if (top <= 9) go(IntC<8>{});
+                else if (top <= 17) go(IntC<16>{});
                 else go(IntC<64>{});
             });
         });
