@@ -48,10 +48,12 @@ struct ExpFold {
 };
 
 // launches the adjoint of the Chen product on `stream` (defined in sig_chen_adjoint.hip for float and double).
-// identity = 0 drops the dC_t[w] terms; families = 1 computes dA only (dB and A are not touched)
+// identity: bit 0 keeps the dC_k[u] term of dA, bit 1 the dC_t[w] term of dB; a gradient without that term is zero at
+// the top level, which the streaming kernels then leave unwritten.  families = 1 computes dA only (dB and A are not
+// touched)
 template <typename T>
 void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint64_t batch, uint64_t dimension,
-                        uint64_t degree, const SigShape& s, hipStream_t stream, int identity = 1,
+                        uint64_t degree, const SigShape& s, hipStream_t stream, int identity = 3,
                         SharedRows dc = SharedRows(), int families = 2, ExpFold<T>* fold = nullptr);
 extern template void launch_combine_bwd<float>(const float*, float*, float*, const float*, const float*, uint64_t, uint64_t,
                                                uint64_t, const SigShape&, hipStream_t, int, SharedRows, int, ExpFold<float>*);

@@ -60,8 +60,8 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_init_kernel(
     for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         for (I r = I(xcd_block_2d().x) * kBlock + threadIdx.x; r < init_len; r += I(gridDim.x) * kBlock) {
             const T v = identity ? dC[(b / dc_share) * dc_stride + dc_off + r] : T(0);
-            if (!only_b) dA[b * stride + off + r] = v;
-            if (families > 1 || only_b) dB[b * stride + off + r] = v;
+            if (!only_b) dA[b * stride + off + r] = (identity & 1) ? v : T(0);
+            if (families > 1 || only_b) dB[b * stride + off + r] = (identity & 2) ? v : T(0);
         }
     }
 }
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(kBlock) void sig_combine_bwd_kernel(
             const I r = plan.lo[t] + w;
             T* dst = (fam_b ? dB : dA) + b * stride + off + r;
             const T sum = (s0 + s1) + (s2 + s3);
-            if (plan.parts[t] == 1) *dst = (identity ? g[r] : T(0)) + sum;
+            if (plan.parts[t] == 1) *dst = ((identity >> int(fam_b)) & 1 ? g[r] : T(0)) + sum;
             else dev_add(dst, sum);
             if (off && it == 0) {
                 if (!only_b) dA[b * stride] = T(0);
@@ -208,6 +208,7 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
 {
     if (dc.stride < 0) { dc.stride = int64_t(s.stride); dc.off = s.off; }
     if (fold) fold->level = int(degree);
+    const int ida = identity & 1, idb = (identity >> 1) & 1;
     if (degree > uint64_t(kCombMaxLevels)) throw std::runtime_error("sig_combine_backprop_cuda: degree too high");
     const int mode = g_chen_adjoint_mode;
     const bool streaming = mode != 2 && (mode == 1 || s.n_coef >= kStreamMinCoef) && dimension >= 2 && degree >= 2 &&
@@ -235,7 +236,7 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
         const int kt = int((wp.top + kBlock - 1) / kBlock), ks = int((wp.targets + kBlock - 1) / kBlock);
         auto go3 = [&](auto dc_, auto kt_, auto ks_) {
             hipLaunchKernelGGL((chen_adjoint_left_rows_kernel<T, decltype(dc_)::value, decltype(kt_)::value, decltype(ks_)::value>),
-                               grid, dim3(kBlock), lds, stream, dC, dA, B, int64_t(batch), wp, int64_t(s.stride), s.off, identity,
+                               grid, dim3(kBlock), lds, stream, dC, dA, B, int64_t(batch), wp, int64_t(s.stride), s.off, ida,
                                dc.share, dc.stride, dc.off);
         };
         auto go2 = [&](auto dc_, auto ks_) {
@@ -267,7 +268,7 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
         const size_t lds = (size_t(lp.xs) + size_t(lp.bs)) * sizeof(T);
         auto go = [&](auto kx) {
             hipLaunchKernelGGL((chen_adjoint_left_kernel<T, decltype(kx)::value>), grid, dim3(kBlock), lds, stream, dC, dA, B,
-                               int64_t(batch), lp, int64_t(s.stride), s.off, identity, dc.share, dc.stride, dc.off);
+                               int64_t(batch), lp, int64_t(s.stride), s.off, ida, dc.share, dc.stride, dc.off);
         };
         const uint32_t per = (lp.xs + kBlock - 1) / kBlock;      // entries of a unit per thread
         if (per <= 4) go(std::integral_constant<int, 4>());
@@ -282,9 +283,9 @@ void launch_combine_bwd(const T* dC, T* dA, T* dB, const T* A, const T* B, uint6
     } else {
         if (rp.qe >= 2)
             launch_combine_bwd_items<T>(dC, dA, dB, A, B, batch, dimension, uint64_t(rp.qe - 1), s, stream, identity, dc, 1, 1);
-        const bool folding = fold && identity == 1 && rp.rel >= 1 && right_fold_fits<T>(dimension);
+        const bool folding = fold && idb == 1 && rp.rel >= 1 && right_fold_fits<T>(dimension);
         if (folding) fold->level = rp.qe;
-        launch_right_stream<T>(rp, dC, dB, A, batch, s, stream, identity, dc, folding ? fold : nullptr);
+        launch_right_stream<T>(rp, dC, dB, A, batch, s, stream, idb, dc, folding ? fold : nullptr);
     }
 }
 

@@ -144,7 +144,7 @@ __device__ __forceinline__ void right_descend(RightLane<T, QL>& L, const RightPl
                         L.kacc[DEPTH] = fmadd(L.z[x] * F.inv_level[DEPTH], e[i], L.kacc[DEPTH]);
                         lds_add(L.slot + x * kBlock, e[i] * zq);
                     } else {
-                        if (L.live) store_at(orow + idx * P.words, L.fo, L.identity ? e[i] : T(0));
+                        if (L.live && L.identity) store_at(orow + idx * P.words, L.fo, e[i]);
                     }
                 }
             }
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kBlock) void chen_adjoint_left_kernel(
                     if (zw < P.xs) {
                         X[zw + (tid & (kWave - 1))] = rx[i];                    // padding receives zeros
                         if (zw >= P.xoff[mt] && zw - P.xoff[mt] + (tid & (kWave - 1)) < P.c * P.lv.pw[mt])
-                            store_at(top + (zw - P.xoff[mt]), lane_off, identity ? rx[i] : T(0));
+                            if (identity) store_at(top + (zw - P.xoff[mt]), lane_off, rx[i]);
                         s1 = fmadd(rx[i], rb1[i], s1);
                     }
                 }
@@ -546,7 +546,7 @@ __global__ __launch_bounds__(kBlock) void chen_adjoint_left_rows_kernel(
                 for (int i = 0; i < KT; ++i) {
                     if (timg[i] != 0xffffffffu) {
                         Img[timg[i]] = rx[i];
-                        top[kBlock * i] = identity ? rx[i] : T(0);
+                        if (identity) top[kBlock * i] = rx[i];
                         s1 = fmadd(rx[i], rb[i], s1);
                     }
                 }

@@ -44,25 +44,23 @@ __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
     }
 }
 
-// after the adjoint of x (x) P_{k+1} (tmpA w.r.t. x, tmpB w.r.t. P_{k+1}):
-//   g_next = -tmpB,   dx += -tmpA + g_next / (k + 1)      over the `count` coefficients of levels <= N - k + 1
-// `first` (the k = 1 update, which covers every coefficient): dx starts from g, so that no separate pass copies it
+// after the adjoint of x (x) P_{k+1} with -P_{k+1} as the left factor's partner (tmpB w.r.t. P_{k+1}; w.r.t. x:
+// -tmpA, which the k = 1 call has already added to g inside dx and the later calls leave in `neg_a`):
+//   g_next = -tmpB,   dx += neg_a + g_next / (k + 1)      over the `count_next` coefficients of levels <= N - k
+// (neither gradient has a term at level N - k + 1: the Chen product's adjoint without its dC term stops one level short)
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void tensor_log_bwd_update_kernel(
-    T* dx, const T* first, T* __restrict__ g_next, const T* __restrict__ tmpA, const T* __restrict__ tmpB, int64_t batch,
-    I count, I count_next, T inv_next, int64_t stride, int off)
+    T* __restrict__ dx, T* __restrict__ g_next, const T* __restrict__ neg_a, const T* __restrict__ tmpB, int64_t batch,
+    I count_next, T inv_next, int64_t stride, int off)
 {
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const int64_t base = b * stride + off;
-        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < count; r += I(gridDim.x) * kBlock) {
-            if (first && off && r == 0) dx[b * stride] = T(0);
-            T v = (first ? first[base + r] : dx[base + r]) - tmpA[base + r];
-            if (r < count_next) {
-                const T gn = -tmpB[base + r];
-                g_next[base + r] = gn;
-                v = fmadd(gn, inv_next, v);
-            }
-            dx[base + r] = v;
+        for (I r = I(blockIdx.x) * kBlock + threadIdx.x; r < count_next; r += I(gridDim.x) * kBlock) {
+            const T gn = -tmpB[base + r];
+            g_next[base + r] = gn;
+            T v = dx[base + r];
+            if (neg_a) v += neg_a[base + r];
+            dx[base + r] = fmadd(gn, inv_next, v);
         }
     }
 }
@@ -217,15 +215,16 @@ __global__ __launch_bounds__(kBlock) void lyndon_expand_kernel(
 // number of coefficients of levels 1 .. t
 static uint64_t coef_count(uint64_t d, uint64_t t) { return sig_length_u64(d, t) - 1; }
 
-// runs the recursion; P_k (k >= 2) lands in p_of(k), P_1 in `out`
+// runs the recursion down to k = k_min; P_k (k >= 2) lands in p_of(k), P_1 in `out`.  sign = -1 computes -P_k instead
+// (the recursion is linear in x / k, the only place the sign enters)
 template <typename T, typename PofK>
 static void run_tensor_log(const T* sig, T* out, uint64_t batch, uint64_t dimension, uint64_t degree, const SigShape& s,
-                           hipStream_t stream, PofK&& p_of)
+                           hipStream_t stream, PofK&& p_of, uint64_t k_min = 1, int sign = 1)
 {
     launch_indexed(s.n_coef, 1, batch, [&](auto ix, dim3) {
         using I = decltype(ix);
         const DivBy<I> dv(dimension);
-        for (uint64_t k = degree; k >= 1; --k) {
+        for (uint64_t k = degree; k >= k_min; --k) {
             const uint64_t count = coef_count(dimension, degree - k + 1);
             const T* pin = k == degree ? sig : p_of(k + 1);       // unused when k == degree: only level 1 is computed
             T* pout = k == 1 ? out : p_of(k);
@@ -234,7 +233,7 @@ static void run_tensor_log(const T* sig, T* out, uint64_t batch, uint64_t dimens
                 const uint64_t items = chen_items(dimension, degree - k + 1, FAN);
                 launch_indexed(0, items, batch, [&](auto, dim3 grid) {
                     hipLaunchKernelGGL((tensor_log_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig, pin, pout,
-                                       int64_t(batch), dv, I(items), T(1) / T(k), int64_t(s.stride), s.off, int64_t(s.stride),
+                                       int64_t(batch), dv, I(items), T(sign) / T(k), int64_t(s.stride), s.off, int64_t(s.stride),
                                        int(k == 1));
                 });
             });
@@ -311,7 +310,7 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
         });
         derivs = dexp;
     }
-    // P_1 (discarded), P_2 .. P_N, two adjoint buffers, two product-adjoint buffers
+    // -P_2 .. -P_N (the slot of P_1 stays unused), two adjoint buffers, two product-adjoint buffers
     T* ws = degree >= 2 ? static_cast<T*>(workspace(7, checked_mul(bytes, degree + 4, "workspace"))) : nullptr;
     if (degree < 2)
         launch_indexed(s.n_coef, s.n_coef, batch, [&](auto ix, dim3 grid) {
@@ -324,20 +323,24 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
         T* g_buf[2] = {ws + degree * elems, ws + (degree + 1) * elems};
         T* tmpA = ws + (degree + 2) * elems;
         T* tmpB = ws + (degree + 3) * elems;
-        run_tensor_log<T>(sig, p_base, batch, dimension, degree, s, stream, [&](uint64_t k) { return p_base + (k - 1) * elems; });
+        // the backward pass never reads P_1, and takes the others negated: the left factor's gradient of
+        // x (x) (-P_{k+1}) is the term dx needs, sign included
+        run_tensor_log<T>(sig, p_base, batch, dimension, degree, s, stream, [&](uint64_t k) { return p_base + (k - 1) * elems; },
+                          2, -1);
         const T* g = derivs;
         for (uint64_t k = 1; k < degree; ++k) {
             const uint64_t top = degree - k + 1;          // levels of g_k
             const SigShape sk{coef_count(dimension, top), s.stride, s.off};
-            launch_combine_bwd<T>(g, tmpA, tmpB, sig, p_base + k * elems, batch, dimension, top, sk, stream, /*identity=*/0);
+            // k = 1: the left factor's gradient keeps its dC term and lands in `out`, which is then g - tmpA already
+            launch_combine_bwd<T>(g, k == 1 ? out : tmpA, tmpB, sig, p_base + k * elems, batch, dimension, top, sk, stream,
+                                  /*identity=*/k == 1 ? 1 : 0);
             T* g_next = g_buf[k & 1];
-            const uint64_t count = sk.n_coef, count_next = coef_count(dimension, top - 1);
-            launch_indexed(s.n_coef, count, batch, [&](auto ix, dim3 grid) {
+            const uint64_t count_next = coef_count(dimension, top - 1);
+            launch_indexed(s.n_coef, count_next, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
-                hipLaunchKernelGGL((tensor_log_bwd_update_kernel<T, I>), grid, dim3(kBlock), 0, stream, out,
-                                   k == 1 ? derivs : static_cast<const T*>(nullptr), g_next,
-                                   (const T*)tmpA, (const T*)tmpB, int64_t(batch), I(count), I(count_next), T(1) / T(k + 1),
-                                   int64_t(s.stride), s.off);
+                hipLaunchKernelGGL((tensor_log_bwd_update_kernel<T, I>), grid, dim3(kBlock), 0, stream, out, g_next,
+                                   k == 1 ? static_cast<const T*>(nullptr) : (const T*)tmpA, (const T*)tmpB, int64_t(batch),
+                                   I(count_next), T(1) / T(k + 1), int64_t(s.stride), s.off);
             });
             g = g_next;
         }

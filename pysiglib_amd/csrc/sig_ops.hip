@@ -464,7 +464,7 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     fold.dz = d_disp;
     fold.level = int(degree);
     if (prepend) launch_combine_bwd<T>(d_out, dE, d_sig, (const T*)E, sig, batch, dimension, degree, s, stream);
-    else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream, 1, SharedRows(), 2, &fold);
+    else launch_combine_bwd<T>(d_out, d_sig, dE, sig, (const T*)E, batch, dimension, degree, s, stream, 3, SharedRows(), 2, &fold);
     const uint64_t top = uint64_t(fold.level);
     if (dimension == 1) {
         hipLaunchKernelGGL((exp_pullback_dim_one_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, (const T*)dE, disp,
