@@ -679,10 +679,16 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream, out,
                                int64_t(batch * s.stride));
         const T time_step = end_time / T(s.len_aug - 1);
-        // operands staged through LDS: two slabs of `chunk` steps by 64 channels
-        const size_t row_bytes = size_t(kDeg2SlabStride) * sizeof(T) * 2;
-        int chunk = sizeof(T) == 8 ? 32 : 64;
-        while (chunk > 8 && chunk / 2 >= slice_len) chunk /= 2;
+        // points staged through LDS: slabs of 4 * rq + 1 points by 64 channels, rq odd, at most 43 KB a slab; chunks of
+        // equal length
+        const size_t row_bytes = size_t(kDeg2SlabStride) * sizeof(T);
+        const bool two_slabs = tiles > kWavesPerBlock;      // row and column channels of a block can differ
+        const int rq_max = (sizeof(T) == 8 ? 15 : 33) / (two_slabs ? 2 : 1) | 1;
+        const int64_t n_chunks = (slice_len + 4 * rq_max - 1) / (4 * rq_max);
+        int rq = int((slice_len + 4 * n_chunks - 1) / (4 * n_chunks));
+        rq = std::min(rq | 1, rq_max);
+        const bool vec = !time_aug && !lead_lag && dimension % (16 / sizeof(T)) == 0 && reinterpret_cast<uintptr_t>(path) % 16 == 0 &&
+                         4 * rq + 1 <= deg2_prefetch_rows<T>();
         // with fewer than four row tiles some of a block's waves would idle and its slabs be mostly padding (measured:
         // d = 64..256 1.4-1.5x faster staged, d <= 32 up to 3x slower)
         const bool staged = g_degree2_staged != 0 && tiles >= kWavesPerBlock;
@@ -692,10 +698,16 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             const int64_t row_groups = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
             const int64_t blocks = int64_t(batch) * row_groups * col_groups * slices;
             if (blocks > 2147483647LL) throw std::runtime_error("signature_cuda: launch too large");
-            hipLaunchKernelGGL((degree2_fwd_staged_kernel<T>), dim3(unsigned(blocks)), dim3(kBlock), chunk * row_bytes, stream, path,
-                               out, int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
-                               int64_t(s.stride), sc, tiles, col_groups, int(slices), slice_len, chunk,
-                               slices > 1 ? nullptr : flag);
+            auto go = [&](auto mode) {
+                hipLaunchKernelGGL((degree2_fwd_staged_kernel<T, decltype(mode)::value>), dim3(unsigned(blocks)), dim3(kBlock),
+                                   size_t(4 * rq + 1) * row_bytes * (two_slabs ? 2 : 1), stream, path, out,
+                                   int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
+                                   int64_t(s.stride), sc, tiles, col_groups, int(slices), slice_len, rq,
+                                   slices > 1 ? nullptr : flag);
+            };
+            if (vec) go(std::integral_constant<int, 2>());
+            else if (!time_aug && !lead_lag) go(std::integral_constant<int, 1>());
+            else go(std::integral_constant<int, 0>());
         } else {
             const int64_t total = waves * slices;
             const int64_t blocks = (total + kWavesPerBlock - 1) / kWavesPerBlock;

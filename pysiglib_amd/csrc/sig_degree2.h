@@ -139,27 +139,51 @@ __global__ __launch_bounds__(kBlock) void degree2_fwd_kernel(
     if (nonfinite && !(chk == T(0))) *nonfinite = 1;
 }
 
-// Forward, operands staged through LDS.  A block serves one (path, time slice, group of four 16-row tiles, group of
-// kDeg2Cols column tiles): its four waves own one row tile each and share the column group.  Per chunk of `chunk`
-// steps the block writes the U values of its 64 row channels and the Z values of its 64 column channels to LDS
-// (coalesced reads of the path, every element computed once per block), then every wave feeds its products from
-// LDS.  Slab rows are 80 words long so that the four step rows a fragment read touches fall into different banks.
+// Forward, points staged through LDS.  A block serves one (path, time slice, group of four 16-row tiles, group of
+// kDeg2Cols column tiles): its four waves own one row tile each and share the column group.  Per chunk of 4 * rq
+// steps the block copies the points Y_t = X_t - X_0 of its 64 row channels and of its 64 column channels to LDS
+// (coalesced reads of the path, every point read once per block; one slab when the two channel groups coincide).
+// The four step indices k of a product stand for four contiguous runs of rq steps, so that a lane walks the rows of
+// its run and forms U_t = (Y_t + Y_{t+1}) / 2 and z_t = Y_{t+1} - Y_t from the row it already holds and the next:
+// one LDS read per operand and product.  Rows past the end of the slice repeat its last point (z = 0: no term).
+// Slab rows are 80 words long and rq is odd, so that the four runs' rows fall into different banks.
 constexpr int kDeg2Slab = 16 * kDeg2Cols;       // channels per slab (64)
 constexpr int kDeg2SlabStride = kDeg2Slab + 16;
 static_assert(kBlock % kDeg2Slab == 0 && kWavesPerBlock == kDeg2Cols, "staging assumes 4 waves and 64-channel slabs");
 
+// MODE 0: any augmentation, a point's channels evaluated one by one.  MODE 1: neither lead-lag nor time augmentation
+// (a point's channels are one contiguous row of the input).  MODE 2: such rows in 16-byte pieces (dimension a
+// multiple of 16 bytes, aligned input), and the next chunk's pieces are loaded into registers before the products of
+// the current one start, so that a block's loads and products overlap.
+constexpr int kDeg2StageBatch = 8;      // staged rows whose loads a thread has in flight together
+constexpr int kDeg2Prefetch = 9;        // 16-byte pieces a thread holds for the next chunk (MODE 2)
 template <typename T>
+struct Vec16;
+template <>
+struct Vec16<float> {
+    typedef float type __attribute__((ext_vector_type(4)));
+    static constexpr int n = 4;
+};
+template <>
+struct Vec16<double> {
+    typedef double type __attribute__((ext_vector_type(2)));
+    static constexpr int n = 2;
+};
+// rows of a chunk that MODE 2 can hold in its registers
+template <typename T>
+constexpr int deg2_prefetch_rows() { return kDeg2Prefetch * (kBlock / (kDeg2Slab / Vec16<T>::n)); }
+
+template <typename T, int MODE>
 __global__ __launch_bounds__(kBlock) void degree2_fwd_staged_kernel(
     const T* __restrict__ path, T* __restrict__ out, int64_t batch, int64_t len_raw, int d_raw, int time_aug, int lead_lag,
-    T time_step, int64_t out_stride, int scalar, int tiles, int col_groups, int slices, int64_t slice_len, int chunk,
+    T time_step, int64_t out_stride, int scalar, int tiles, int col_groups, int slices, int64_t slice_len, int rq,
     int* __restrict__ nonfinite)
 {
     using M = Mfma16<T>;
-    extern __shared__ double lds_raw_d2[];
+    extern __shared__ __align__(16) double lds_raw_d2[];
+    constexpr bool PLAIN = MODE != 0;
     const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
     const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
-    T* lds_u = reinterpret_cast<T*>(lds_raw_d2);
-    T* lds_z = lds_u + int64_t(chunk) * kDeg2SlabStride;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int row_groups = (tiles + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -174,6 +198,9 @@ __global__ __launch_bounds__(kBlock) void degree2_fwd_staged_kernel(
     const bool has_task = ta < tiles;
     const T* x = path + b * len_raw * d_raw;
     T* o = out + b * out_stride + scalar;
+    const int rows = 4 * rq + 1;                                // points of a chunk
+    T* lds_u = reinterpret_cast<T*>(lds_raw_d2);
+    T* lds_z = rg == cg ? lds_u : lds_u + int64_t(rows) * kDeg2SlabStride;
 
     const int li = lane & 15, lk = lane >> 4;
     typename M::Acc acc[kDeg2Cols];
@@ -185,37 +212,96 @@ __global__ __launch_bounds__(kBlock) void degree2_fwd_staged_kernel(
     const int sc_col = threadIdx.x % kDeg2Slab, sc_row0 = threadIdx.x / kDeg2Slab;
     const int cu = rg * kDeg2Slab + sc_col, cz = cg * kDeg2Slab + sc_col;
     const T x0u = cu < d ? aug_point(x, 0, cu, d_raw, time_aug, lead_lag, d, time_step) : T(0);
+    const T x0z = cz < d ? aug_point(x, 0, cz, d_raw, time_aug, lead_lag, d, time_step) : T(0);
 
     const int64_t t_begin = int64_t(slice) * slice_len;
     const int64_t t_end = t_begin + slice_len < L ? t_begin + slice_len : L;
-    for (int64_t t0 = t_begin; t0 < t_end; t0 += chunk) {
+    auto point = [&](int64_t t, int c) {
+        if constexpr (PLAIN) return x[t * d_raw + c];
+        else return aug_point(x, t, c, d_raw, time_aug, lead_lag, d, time_step);
+    };
+    constexpr int kRowStep = kBlock / kDeg2Slab;
+    // MODE 2: thread -> 16-byte piece `vcol` of the rows vrow0, vrow0 + kVecRows, ..
+    using V = typename Vec16<T>::type;
+    constexpr int kVecCols = kDeg2Slab / Vec16<T>::n, kVecRows = kBlock / kVecCols;
+    const int vcol = int(threadIdx.x % kVecCols) * Vec16<T>::n, vrow0 = int(threadIdx.x / kVecCols);
+    [[maybe_unused]] V pfu[kDeg2Prefetch], pfz[kDeg2Prefetch], x0uv = V(T(0)), x0zv = V(T(0));
+    [[maybe_unused]] const bool vu_ok = rg * kDeg2Slab + vcol < d, vz_ok = rg != cg && cg * kDeg2Slab + vcol < d;
+    [[maybe_unused]] auto fetch = [&](int64_t t0) {
+#pragma unroll
+        for (int k = 0; k < kDeg2Prefetch; ++k) {
+            const int r = vrow0 + kVecRows * k;
+            const int64_t t = t0 + r < t_end ? t0 + r : t_end;
+            pfu[k] = vu_ok ? *reinterpret_cast<const V*>(x + t * d_raw + rg * kDeg2Slab + vcol) : V(T(0));
+            pfz[k] = vz_ok ? *reinterpret_cast<const V*>(x + t * d_raw + cg * kDeg2Slab + vcol) : V(T(0));
+        }
+    };
+    if constexpr (MODE == 2) {
+        if (vu_ok) x0uv = *reinterpret_cast<const V*>(x + rg * kDeg2Slab + vcol);
+        if (vz_ok) x0zv = *reinterpret_cast<const V*>(x + cg * kDeg2Slab + vcol);
+        fetch(t_begin);
+    }
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += 4 * rq) {
         __syncthreads();        // the previous chunk has been consumed
-        for (int r = sc_row0; r < chunk; r += kBlock / kDeg2Slab) {
-            const int64_t t = t0 + r;
-            T u = T(0), z = T(0);
-            if (t < t_end) {
-                if (cu < d)
-                    u = T(0.5) * (aug_point(x, t, cu, d_raw, time_aug, lead_lag, d, time_step) +
-                                  aug_point(x, t + 1, cu, d_raw, time_aug, lead_lag, d, time_step)) - x0u;
-                if (cz < d)
-                    z = aug_point(x, t + 1, cz, d_raw, time_aug, lead_lag, d, time_step) -
-                        aug_point(x, t, cz, d_raw, time_aug, lead_lag, d, time_step);
+        if constexpr (MODE == 2) {
+#pragma unroll
+            for (int k = 0; k < kDeg2Prefetch; ++k) {
+                const int r = vrow0 + kVecRows * k;
+                if (r < rows) {
+                    *reinterpret_cast<V*>(lds_u + r * kDeg2SlabStride + vcol) = pfu[k] - x0uv;
+                    if (rg != cg) *reinterpret_cast<V*>(lds_z + r * kDeg2SlabStride + vcol) = pfz[k] - x0zv;
+                }
             }
-            lds_u[r * kDeg2SlabStride + sc_col] = u;
-            lds_z[r * kDeg2SlabStride + sc_col] = z;
+        } else {
+            for (int r0 = sc_row0; r0 < rows; r0 += kRowStep * kDeg2StageBatch) {
+                T vu[kDeg2StageBatch], vz[kDeg2StageBatch];
+#pragma unroll
+                for (int k = 0; k < kDeg2StageBatch; ++k) {
+                    const int r = r0 + kRowStep * k;
+                    const int64_t t = t0 + r < t_end ? t0 + r : t_end;
+                    vu[k] = cu < d ? point(t, cu) : T(0);
+                    vz[k] = (rg != cg && cz < d) ? point(t, cz) : T(0);
+                }
+#pragma unroll
+                for (int k = 0; k < kDeg2StageBatch; ++k) {
+                    const int r = r0 + kRowStep * k;
+                    if (r < rows) {
+                        lds_u[r * kDeg2SlabStride + sc_col] = vu[k] - x0u;
+                        if (rg != cg) lds_z[r * kDeg2SlabStride + sc_col] = vz[k] - x0z;
+                    }
+                }
+            }
         }
         __syncthreads();
+        if constexpr (MODE == 2)
+            if (t0 + 4 * rq < t_end) fetch(t0 + 4 * rq);
         if (has_task) {
-            const T* pu = lds_u + lk * kDeg2SlabStride + wave * 16 + li;
-            const T* pz = lds_z + lk * kDeg2SlabStride + li;
-            for (int r0 = 0; r0 < chunk; r0 += 4) {
-                const T ua = pu[r0 * kDeg2SlabStride];
-                T zb[kDeg2Cols];
+            const T* pu = lds_u + lk * rq * kDeg2SlabStride + wave * 16 + li;
+            const T* pz = lds_z + lk * rq * kDeg2SlabStride + li;
+            // all kDeg2Cols column tiles, in use or not (channels past the last hold zeros): no branch in the loop
+            // the rows r and r + 1 are in registers while row r + 2 is on its way from LDS
+            T u0 = pu[0], u1 = pu[kDeg2SlabStride], z0[kDeg2Cols], z1[kDeg2Cols];
 #pragma unroll
-                for (int j = 0; j < kDeg2Cols; ++j) zb[j] = j < nb ? pz[r0 * kDeg2SlabStride + j * 16] : T(0);
+            for (int j = 0; j < kDeg2Cols; ++j) {
+                z0[j] = pz[j * 16];
+                z1[j] = pz[kDeg2SlabStride + j * 16];
+            }
+            for (int r = 1; r <= rq; ++r) {
+                const int rn = r < rq ? r + 1 : r;
+                const T u2 = pu[rn * kDeg2SlabStride];
+                T z2[kDeg2Cols];
 #pragma unroll
-                for (int j = 0; j < kDeg2Cols; ++j)
-                    if (j < nb) acc[j] = M::mma(ua, zb[j], acc[j]);
+                for (int j = 0; j < kDeg2Cols; ++j) z2[j] = pz[rn * kDeg2SlabStride + j * 16];
+                const T ua = T(0.5) * (u0 + u1);
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) acc[j] = M::mma(ua, z1[j] - z0[j], acc[j]);
+                u0 = u1;
+                u1 = u2;
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) {
+                    z0[j] = z1[j];
+                    z1[j] = z2[j];
+                }
             }
         }
     }

@@ -817,7 +817,8 @@ def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
     ((2, 13, 31, 2), dict(lead_lag=True)), ((3, 12, 33, 2), dict(time_aug=True, lead_lag=True)), ((1, 2, 70, 2), {}),
     ((2, 700, 20, 2), {}),                      # few long paths: time slices adding into the output
     ((2, 600, 50, 2), {}), ((1, 300, 36, 2), dict(lead_lag=True)),      # the same with operands staged through LDS
-    ((1, 1500, 7, 2), dict(lead_lag=True)), ((70, 6, 65, 2), {}), ((2, 5, 130, 2), dict(time_aug=True))])
+    ((1, 1500, 7, 2), dict(lead_lag=True)), ((70, 6, 65, 2), {}), ((2, 5, 130, 2), dict(time_aug=True)),
+    ((3, 300, 64, 2), {}), ((2, 41, 128, 2), {}), ((2, 150, 100, 2), {}), ((5, 3, 64, 2), {})])     # rows in 16-byte pieces
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
     """Degree 2 has a closed form in the path (S2 = U^T Z, pullback through the antisymmetric part of the level-2
