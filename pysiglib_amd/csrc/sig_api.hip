@@ -971,6 +971,34 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
                                                                   "level-2 gradient")))
                          : nullptr;
         const T time_step = end_time / T(s.len_aug - 1);
+        if (g_degree2_staged != 0 && tiles >= 3 && tiles <= kDeg2Cols && s.L >= 1) {
+            // at most 64 channels: one launch, the level-2 gradient's fragments in registers; plain paths receive
+            // their gradient directly
+            const bool plain = !time_aug && !lead_lag;
+            const bool vec = plain && dimension % (16 / sizeof(T)) == 0 && reinterpret_cast<uintptr_t>(path) % 16 == 0;
+            const int64_t out_rows = plain ? int64_t(s.L) + 1 : int64_t(s.L);
+            const int64_t chunks = (out_rows + kDeg2BwdRows - 1) / kDeg2BwdRows;
+            int64_t parts = std::min<int64_t>(chunks, std::max<int64_t>(1, (2 * int64_t(simd_count()) / 4 + int64_t(batch) - 1) / int64_t(batch)));
+            const int64_t part_rows = (chunks + parts - 1) / parts * kDeg2BwdRows;
+            parts = (out_rows + part_rows - 1) / part_rows;
+            const int64_t blocks = int64_t(batch) * parts;
+            if (blocks > 2147483647LL) throw std::runtime_error("sig_backprop_cuda: launch too large");
+            MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_bwd_f64_rows" : "degree2_bwd_f32_rows", !arena);
+            auto go = [&](auto mode) {
+                constexpr int MODE = decltype(mode)::value;
+                hipLaunchKernelGGL((degree2_bwd_rows_kernel<T, MODE>), dim3(unsigned(blocks)), dim3(kBlock), deg2_bwd_lds_bytes<T>(),
+                                   stream, path, sig_derivs, MODE ? out : dzinc, int64_t(batch), int64_t(length), int(dimension),
+                                   int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, int(parts), part_rows);
+            };
+            if (vec) go(std::integral_constant<int, 2>());
+            else if (plain) go(std::integral_constant<int, 1>());
+            else go(std::integral_constant<int, 0>());
+            timer.stop();
+            if (!plain) launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
+            SIG_HIP(hipGetLastError());
+            finish();
+            return;
+        }
         hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug)), dim3(kBlock), 0, stream, path, sig_derivs, h,
                            int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
                            int64_t(s.stride), sc);

@@ -534,4 +534,198 @@ __global__ __launch_bounds__(kBlock) void degree2_bwd_staged_kernel(
     }
 }
 
+// Backward for at most 64 (augmented) channels, one launch.  A block serves a run of output rows of one path, 64 rows
+// at a time: four waves of 16 rows each, all kDeg2Cols column tiles.  The antisymmetric part of the level-2 gradient
+// is built once per block (G2 copied to LDS with coalesced loads, then every lane keeps its 16 x kDeg2Cols fragment
+// values in registers for the whole run), and h = G1 + G2 S1 is formed in the block as well.  The product's k index
+// stands for the channel lk * 16 + kk, so that a lane reads its 16 operands of a row as four 16-byte pieces.
+// MODE 0: any augmentation; output rows are the increments' gradients dz_t = h + U_t A, t < L.
+// MODE 1 / 2 (plain paths; 2: input rows in 16-byte pieces, next 64 rows prefetched into registers): the rows are the
+// path's gradient itself, out_t = dz_{t-1} - dz_t = (Y_{t-1} - Y_{t+1}) / 2 A for 0 < t < L, out_0 = -dz_0,
+// out_L = dz_{L-1}: with Y_{-1} = Y_0 = 0 and Y_{L+1} = -Y_L the same operand form serves every row, and only the
+// two end rows see h.
+constexpr int kDeg2BwdRows = 64;                    // output rows per chunk
+constexpr int kDeg2BwdStride = kDeg2Slab + 4;       // LDS row of points: 16-byte pieces of neighbouring rows in different banks
+constexpr int kDeg2GStride = kDeg2Slab + 1;         // LDS row of G2: a column walk changes bank
+template <typename T>
+constexpr size_t deg2_bwd_lds_bytes()
+{
+    return (size_t(kDeg2BwdRows + 2) * kDeg2BwdStride + size_t(kDeg2Slab) * kDeg2GStride + 2 * kDeg2Slab) * sizeof(T);
+}
+
+// registers for three (f32) resp. two (f64) blocks per CU: a block's phases (copy to LDS, products, stores) do not
+// overlap with each other, only with those of its neighbours
+template <typename T, int MODE>
+__global__ __launch_bounds__(kBlock, sizeof(T) == 8 ? 2 : 3) void degree2_bwd_rows_kernel(
+    const T* __restrict__ path, const T* __restrict__ gsig, T* __restrict__ outp, int64_t batch, int64_t len_raw, int d_raw,
+    int time_aug, int lead_lag, T time_step, int64_t sig_stride, int scalar, int parts, int64_t part_rows)
+{
+    using M = Mfma16<T>;
+    using V = typename Vec16<T>::type;
+    constexpr int VN = Vec16<T>::n;
+    constexpr bool DIRECT = MODE != 0;
+    constexpr int HI = DIRECT ? 2 : 1;              // the operand of row i combines the staged rows i and i + HI
+    extern __shared__ __align__(16) double lds_raw_d2r[];
+    T* Ys = reinterpret_cast<T*>(lds_raw_d2r);
+    T* Gs = Ys + (kDeg2BwdRows + 2) * kDeg2BwdStride;
+    T* hb = Gs + kDeg2Slab * kDeg2GStride;
+    T* s1 = hb + kDeg2Slab;
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    const int64_t out_rows = DIRECT ? L + 1 : L;
+    const int64_t b = int64_t(blockIdx.x) / parts;
+    const int part = int(int64_t(blockIdx.x) - b * parts);
+    const int64_t row_begin = int64_t(part) * part_rows;
+    const int64_t row_end = row_begin + part_rows < out_rows ? row_begin + part_rows : out_rows;
+    if (row_begin >= row_end) return;
+    const T* x = path + b * len_raw * d_raw;
+    const T* g1 = gsig + b * sig_stride + scalar;
+    const T* g2 = g1 + d;
+    T* o = outp + b * out_rows * d;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int li = lane & 15, lk = lane >> 4;
+    auto point = [&](int64_t t, int c) {
+        if constexpr (DIRECT) return x[t * d_raw + c];
+        else return aug_point(x, t, c, d_raw, time_aug, lead_lag, d, time_step);
+    };
+    // staged row r of the chunk at `base`: the point base + r - (DIRECT ? 1 : 0), as Y = X - X_0
+    //   before the path: 0;  past it: -Y_L once (DIRECT), then 0
+    constexpr int kVecCols = kDeg2Slab / VN, kVecRows = kBlock / kVecCols;
+    constexpr int kPf = (kDeg2BwdRows + 2 + kVecRows - 1) / kVecRows;
+    const int vcol = (tid % kVecCols) * VN, vrow0 = tid / kVecCols;
+    [[maybe_unused]] V pf[kPf], x0v = V(T(0));
+    [[maybe_unused]] const bool v_ok = vcol < d;
+    [[maybe_unused]] auto fetch = [&](int64_t base) {
+#pragma unroll
+        for (int k = 0; k < kPf; ++k) {
+            const int64_t t = base + vrow0 + kVecRows * k - 1;
+            const int64_t tc = t < 0 ? 0 : (t > L ? L : t);
+            pf[k] = v_ok ? *reinterpret_cast<const V*>(x + tc * d_raw + vcol) : V(T(0));
+        }
+    };
+    if constexpr (MODE == 2) {
+        if (v_ok) x0v = *reinterpret_cast<const V*>(x + vcol);
+        fetch(row_begin);
+    }
+    // G2 and S1 to LDS
+    for (int e = tid; e < kDeg2Slab * kDeg2Slab; e += kBlock) {
+        const int a = e / kDeg2Slab, c = e % kDeg2Slab;
+        Gs[a * kDeg2GStride + c] = (a < d && c < d) ? g2[int64_t(a) * d + c] : T(0);
+    }
+    if (tid < kDeg2Slab) s1[tid] = tid < d ? point(L, tid) - point(0, tid) : T(0);
+    __syncthreads();
+    // fragments of A = G2 - G2^T: lane (li, lk) supplies A[lk * 16 + kk][16 j + li].  They are the same for the four
+    // waves: the first one builds them and, once h is done, puts them in place of G2, in the order the products read
+    T bf[16][kDeg2Cols];
+    if (wave == 0) {
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) {
+                const int a = lk * 16 + kk, c = 16 * j + li;
+                bf[kk][j] = T(0.5) * (Gs[a * kDeg2GStride + c] - Gs[c * kDeg2GStride + a]);     // the operands' 1/2 sits here
+            }
+        }
+    } else if (wave == 1) {
+        T sum[4] = {lane < d ? g1[lane] : T(0), T(0), T(0), T(0)};
+#pragma unroll
+        for (int e = 0; e < kDeg2Slab; e += 4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) sum[q] = fmadd(Gs[lane * kDeg2GStride + e + q], s1[e + q], sum[q]);
+        }
+        hb[lane] = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+    }
+    __syncthreads();
+    T* Bf = Gs;                                     // [kk][lane][j]
+    if (wave == 0) {
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) Bf[(kk * kWave + lane) * kDeg2Cols + j] = bf[kk][j];
+        }
+    }
+    const int sc_col = tid % kDeg2Slab, sc_row0 = tid / kDeg2Slab;
+    const T x0s = (MODE != 2 && sc_col < d) ? point(0, sc_col) : T(0);
+
+    for (int64_t base = row_begin; base < row_end; base += kDeg2BwdRows) {
+        __syncthreads();        // the chunk before has been consumed (first pass: hb is complete)
+        if constexpr (MODE == 2) {
+#pragma unroll
+            for (int k = 0; k < kPf; ++k) {
+                const int r = vrow0 + kVecRows * k;
+                const int64_t t = base + r - 1;
+                if (r < kDeg2BwdRows + 2) {
+                    V v = pf[k] - x0v;
+                    if (t < 0 || t > L + 1) v = V(T(0));
+                    else if (t == L + 1) v = -v;
+                    *reinterpret_cast<V*>(Ys + r * kDeg2BwdStride + vcol) = v;
+                }
+            }
+        } else {
+            constexpr int kRowStep = kBlock / kDeg2Slab;
+            for (int r0 = sc_row0; r0 < kDeg2BwdRows + 2; r0 += kRowStep * kDeg2StageBatch) {
+                T v[kDeg2StageBatch];
+#pragma unroll
+                for (int k = 0; k < kDeg2StageBatch; ++k) {
+                    const int64_t t = base + r0 + kRowStep * k - (DIRECT ? 1 : 0);
+                    const int64_t tc = t < 0 ? 0 : (t > L ? L : t);
+                    v[k] = sc_col < d ? point(tc, sc_col) - x0s : T(0);
+                    if (t < 0 || t > L + 1 || (!DIRECT && t > L)) v[k] = T(0);
+                    else if (t == L + 1) v[k] = -v[k];
+                }
+#pragma unroll
+                for (int k = 0; k < kDeg2StageBatch; ++k) {
+                    const int r = r0 + kRowStep * k;
+                    if (r < kDeg2BwdRows + 2) Ys[r * kDeg2BwdStride + sc_col] = v[k];
+                }
+            }
+        }
+        __syncthreads();
+        if constexpr (MODE == 2)
+            if (base + kDeg2BwdRows < row_end) fetch(base + kDeg2BwdRows);
+        if (base + 16 * wave < row_end) {
+            const T* lo = Ys + (16 * wave + li) * kDeg2BwdStride + lk * 16;
+            const T* hi = lo + HI * kDeg2BwdStride;
+            T u[16];
+#pragma unroll
+            for (int q = 0; q < 16 / VN; ++q) {
+                const V a = *reinterpret_cast<const V*>(lo + q * VN), c = *reinterpret_cast<const V*>(hi + q * VN);
+#pragma unroll
+                for (int e = 0; e < VN; ++e) u[q * VN + e] = DIRECT ? a[e] - c[e] : a[e] + c[e];
+            }
+            typename M::Acc acc[kDeg2Cols];
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) acc[j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+#pragma unroll
+            for (int kk = 0; kk < 16; ++kk) {
+                T bq[kDeg2Cols];
+#pragma unroll
+                for (int q = 0; q < kDeg2Cols / VN; ++q) {
+                    const V v = *reinterpret_cast<const V*>(Bf + (kk * kWave + lane) * kDeg2Cols + q * VN);
+#pragma unroll
+                    for (int e = 0; e < VN; ++e) bq[q * VN + e] = v[e];
+                }
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) acc[j] = M::mma(u[kk], bq[j], acc[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < kDeg2Cols; ++j) {
+                const int c = 16 * j + li;
+                if (c >= d) continue;
+                const T hc = hb[c];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t row = base + 16 * wave + M::row(lk, r);
+                    if (row < row_end) {
+                        T v = acc[j][r];
+                        if constexpr (DIRECT) v += row == 0 ? -hc : (row == L ? hc : T(0));
+                        else v += hc;
+                        o[row * d + c] = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
 }  // namespace sigamd

@@ -818,7 +818,8 @@ def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
     ((2, 700, 20, 2), {}),                      # few long paths: time slices adding into the output
     ((2, 600, 50, 2), {}), ((1, 300, 36, 2), dict(lead_lag=True)),      # the same with operands staged through LDS
     ((1, 1500, 7, 2), dict(lead_lag=True)), ((70, 6, 65, 2), {}), ((2, 5, 130, 2), dict(time_aug=True)),
-    ((3, 300, 64, 2), {}), ((2, 41, 128, 2), {}), ((2, 150, 100, 2), {}), ((5, 3, 64, 2), {})])     # rows in 16-byte pieces
+    ((3, 300, 64, 2), {}), ((2, 41, 128, 2), {}), ((2, 150, 100, 2), {}), ((5, 3, 64, 2), {}),      # rows in 16-byte pieces
+    ((2, 100, 40, 2), dict(time_aug=True)), ((3, 70, 33, 2), {}), ((1, 1000, 48, 2), {}), ((4, 2, 56, 2), {})])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
     """Degree 2 has a closed form in the path (S2 = U^T Z, pullback through the antisymmetric part of the level-2
