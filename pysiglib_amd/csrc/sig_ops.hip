@@ -20,6 +20,7 @@ namespace sigamd {
 // lead = x[i/2 + (i odd)]; time is the last channel, i * end_time / (len_eff - 1)
 // (siglib/cpsig/cp_path_transforms.h:36-142).  One thread per output element of a path; `dtd` divides by the
 // transformed dimension.
+constexpr int kTransformBatch = 4;      // elements per thread whose loads are in flight together
 template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void transform_path_kernel(
     const T* __restrict__ in, T* __restrict__ out, int64_t batch, I len, I d, DivBy<I> dtd, int time_aug, int lead_lag, T scale)
@@ -30,15 +31,28 @@ __global__ __launch_bounds__(kBlock) void transform_path_kernel(
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* x = in + b * int64_t(len) * int64_t(d);
         T* o = out + b * int64_t(per);
-        for (I e = I(blockIdx.x) * kBlock + threadIdx.x; e < per; e += I(gridDim.x) * kBlock) {
-            const I i = dtd.quot(e);
-            const I c = e - i * td;
-            T v;
-            if (time_aug && c == td - 1) v = T(i) * scale;
-            else if (!lead_lag) v = x[i * d + c];
-            else if (c < d) v = x[(i >> 1) * d + c];
-            else v = x[((i >> 1) + (i & 1)) * d + (c - d)];
-            o[e] = v;
+        // kTransformBatch elements per thread, a grid apart, all loads before the first store
+        const I step = I(gridDim.x) * kBlock;
+        for (I e0 = I(blockIdx.x) * kBlock + threadIdx.x; e0 < per; e0 += kTransformBatch * step) {
+            T v[kTransformBatch];
+#pragma unroll
+            for (int k = 0; k < kTransformBatch; ++k) {
+                const I e = e0 + I(k) * step;
+                const I ec = e < per ? e : per - 1;
+                const I i = dtd.quot(ec);
+                const I c = ec - i * td;
+                // branch-free: the time channel loads element 0 and discards it
+                const bool is_time = time_aug && c == td - 1;
+                const I lag = (i >> 1) * d + c, lead = ((i >> 1) + (i & 1)) * d + (c - d);
+                const I src = is_time ? I(0) : (!lead_lag ? i * d + c : (c < d ? lag : lead));
+                const T raw = x[src];
+                v[k] = is_time ? T(i) * scale : raw;
+            }
+#pragma unroll
+            for (int k = 0; k < kTransformBatch; ++k) {
+                const I e = e0 + I(k) * step;
+                if (e < per) o[e] = v[k];
+            }
         }
     }
 }
@@ -515,7 +529,7 @@ static void transform_path_impl(const T* in, T* out, uint64_t batch, uint64_t di
     hipStream_t stream = nullptr;
     const T scale = tl > 1 ? end_time / T(tl - 1) : T(0);
     (void)total;
-    launch_indexed(tl * td, (tl * td + 3) / 4, batch, [&](auto ix, dim3 grid) {
+    launch_indexed(tl * td, (tl * td + kTransformBatch - 1) / kTransformBatch, batch, [&](auto ix, dim3 grid) {
         using I = decltype(ix);
         hipLaunchKernelGGL((transform_path_kernel<T, I>), grid, dim3(kBlock), 0, stream, in, out, int64_t(batch), I(length),
                            I(dimension), DivBy<I>(td), int(time_aug), int(lead_lag), scale);
