@@ -115,22 +115,24 @@ __global__ __launch_bounds__(kBlock) void sig_coef_kernel(
 // with st_j = ((1/i!) z_0 + c_1/(i-1)!) z_1 + ... (the Horner values of prefix length i),
 //   dz_{i-1} += g_i st_{i-1};  walking j = i-2 .. 0 with sd = g_i z_{i-1} z_{i-2} ..:  dz_j += sd st_j,
 //   g_{j+1} += sd / (i-j-1)!.
-// A block serves the words blockIdx.x * blockDim.x .. of ONE path and walks the steps in lockstep: all its lanes
-// add their increment gradients of a step into per-channel LDS sums (`copies` private sets, chosen by lane, because
-// few channels mean many lanes per word of LDS), and lane j then owns channel j: path point s-1 receives
-// -dz(step s) + dz(step s-1), so the lane carries the first term over to the next step and issues ONE atomic per
-// (block, point, channel).  use_lds = 0 (very wide paths): every lane adds straight to HBM.  `out` is zeroed beforehand.
+// A block serves the words blockIdx.x * blockDim.x .. of ONE path.  Its lanes add their increment gradients into
+// per-step, per-channel LDS sums for a chunk of `chunk` steps (`copies` private sets per step, chosen by lane, because
+// few channels mean many lanes per word of LDS); after the chunk, point p receives G(step p) - G(step p + 1) in one
+// atomic per (block, point, channel), G being zero outside the chunk.  (A flush after every step had the whole block
+// wait at a barrier while d lanes walked the private sets one LDS read at a time: 4400 cycles a step.)
+// use_lds = 0 (very wide paths): every lane adds straight to HBM.  `out` is zeroed beforehand.
 template <typename T, int KMAX, int UF>
-__global__ void sig_coef_bwd_kernel(
+__global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
     const T* __restrict__ path, T* __restrict__ out, const T* __restrict__ coefs, const T* __restrict__ derivs,
-    WordList words, int64_t batch, int64_t d, int64_t len, int64_t row, int use_lds, int copies)
+    WordList words, int64_t batch, int64_t d, int64_t len, int64_t row, int use_lds, int copies, int chunk)
 {
     extern __shared__ double coef_lds_raw[];
-    T* acc = reinterpret_cast<T*>(coef_lds_raw);
+    T* acc = reinterpret_cast<T*>(coef_lds_raw);        // [chunk][copies][d]
     const int64_t w = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     const bool live = w < int64_t(words.count);
     const int k = live ? int(words.degree[w]) : 0;
     const bool active = k > 0 && k <= KMAX;
+    const int64_t slab = int64_t(copies) * d;           // LDS entries of one step
     T* mine = acc + int64_t(threadIdx.x % copies) * d;
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         int64_t let[KMAX];
@@ -152,73 +154,71 @@ __global__ void sig_coef_bwd_kernel(
         }
         if (use_lds) {
             __syncthreads();        // the previous path's sums have been consumed
-            for (int64_t j = threadIdx.x; j < int64_t(copies) * d; j += blockDim.x) acc[j] = T(0);
+            for (int64_t j = threadIdx.x; j < int64_t(chunk) * slab; j += blockDim.x) acc[j] = T(0);
             __syncthreads();
         }
-        T carry = T(0);             // lane j: -dz(step s)[j], still to be added to point s-1
-        for (int64_t s = len - 1; s >= 1; --s) {        // step s-1 -> s
+        for (int64_t s_hi = len - 1; s_hi >= 1; s_hi -= chunk) {        // steps s_lo .. s_hi, downwards
+            const int64_t s_lo = s_hi - chunk + 1 > 1 ? s_hi - chunk + 1 : 1;
             if (active) {
-                const T* xp = x + (s - 1) * d;
+                for (int64_t s = s_hi; s >= s_lo; --s) {                // step s-1 -> s
+                    const T* xp = x + (s - 1) * d;
 #pragma unroll UF
-                for (int i = 0; i < KMAX; ++i) {
-                    const T cur = xp[let[i]];
-                    z[i] = next[i] - cur;
-                    next[i] = cur;
-                }
-                word_step<T, KMAX, UF, -1>(c, z, k);
+                    for (int i = 0; i < KMAX; ++i) {
+                        const T cur = xp[let[i]];
+                        z[i] = next[i] - cur;
+                        next[i] = cur;
+                    }
+                    word_step<T, KMAX, UF, -1>(c, z, k);
 #pragma unroll UF
-                for (int i = 0; i < KMAX; ++i) dz[i] = T(0);
+                    for (int i = 0; i < KMAX; ++i) dz[i] = T(0);
 #pragma unroll UF
-                for (int i = 1; i <= KMAX; ++i) {
-                    if (i <= k) {
-                        st[0] = T(kInvFact[i]);
+                    for (int i = 1; i <= KMAX; ++i) {
+                        if (i <= k) {
+                            st[0] = T(kInvFact[i]);
 #pragma unroll UF
-                        for (int j = 0; j + 1 < i; ++j) st[j + 1] = fmadd(st[j], z[j], c[j + 1] * T(kInvFact[i - j - 1]));
-                        const T gi = g[i];
-                        dz[i - 1] = fmadd(gi, st[i - 1], dz[i - 1]);
-                        T sd = gi * z[i - 1];
+                            for (int j = 0; j + 1 < i; ++j) st[j + 1] = fmadd(st[j], z[j], c[j + 1] * T(kInvFact[i - j - 1]));
+                            const T gi = g[i];
+                            dz[i - 1] = fmadd(gi, st[i - 1], dz[i - 1]);
+                            T sd = gi * z[i - 1];
 #pragma unroll UF
-                        for (int j = i - 2; j >= 0; --j) {
-                            dz[j] = fmadd(sd, st[j], dz[j]);
-                            g[j + 1] = fmadd(sd, T(kInvFact[i - j - 1]), g[j + 1]);
-                            sd *= z[j];
+                            for (int j = i - 2; j >= 0; --j) {
+                                dz[j] = fmadd(sd, st[j], dz[j]);
+                                g[j + 1] = fmadd(sd, T(kInvFact[i - j - 1]), g[j + 1]);
+                                sd *= z[j];
+                            }
                         }
                     }
-                }
 #pragma unroll UF
-                for (int i = 0; i < KMAX; ++i) {
-                    if (i < k) {
-                        if (use_lds) {
-                            lds_add_shared(&mine[let[i]], dz[i]);
-                        } else {
-                            dev_add(&gx[s * d + let[i]], dz[i]);
-                            dev_add(&gx[(s - 1) * d + let[i]], -dz[i]);
+                    for (int i = 0; i < KMAX; ++i) {
+                        if (i < k) {
+                            if (use_lds) {
+                                lds_add_shared(&mine[(s - s_lo) * slab + let[i]], dz[i]);
+                            } else {
+                                dev_add(&gx[s * d + let[i]], dz[i]);
+                                dev_add(&gx[(s - 1) * d + let[i]], -dz[i]);
+                            }
                         }
                     }
                 }
             }
             if (use_lds) {
                 __syncthreads();
-                for (int64_t j = threadIdx.x; j < d; j += blockDim.x) {
+                // point p = s_lo - 1 + q receives the sums of step p (chunk row q - 1) minus those of step p + 1 (row q)
+                const int64_t n = s_hi - s_lo + 1;
+                for (int64_t e = threadIdx.x; e < (n + 1) * d; e += blockDim.x) {
+                    const int64_t q = e / d, j = e - q * d;
                     T sum = T(0);
-                    for (int q = 0; q < copies; ++q) {
-                        sum += acc[int64_t(q) * d + j];
-                        acc[int64_t(q) * d + j] = T(0);
+                    for (int cpy = 0; cpy < copies; ++cpy) {
+                        if (q >= 1) sum += acc[(q - 1) * slab + int64_t(cpy) * d + j];
+                        if (q < n) sum -= acc[q * slab + int64_t(cpy) * d + j];
                     }
-                    // d <= blockDim.x is not required: a lane's `carry` belongs to channel j only when it owns one
-                    // channel, so wider paths add both terms directly
-                    if (d <= int64_t(blockDim.x)) {
-                        dev_add(&gx[s * d + j], sum + carry);
-                        carry = -sum;
-                    } else {
-                        dev_add(&gx[s * d + j], sum);
-                        dev_add(&gx[(s - 1) * d + j], -sum);
-                    }
+                    dev_add(&gx[(s_lo - 1 + q) * d + j], sum);
                 }
+                __syncthreads();
+                for (int64_t j = threadIdx.x; j < n * slab; j += blockDim.x) acc[j] = T(0);
                 __syncthreads();
             }
         }
-        if (use_lds && d <= int64_t(blockDim.x) && int64_t(threadIdx.x) < d && len >= 2) dev_add(&gx[threadIdx.x], carry);
     }
 }
 
@@ -328,13 +328,18 @@ static void sig_coef_backprop_impl(const T* path, T* out, const T* coefs, const 
         const uint64_t gx = (num_words + threads - 1) / threads;
         if (gx > 0x7fffffffull) throw std::runtime_error("sig_coef_backprop_cuda: too many words");
         const int use_lds = dimension <= 4096;
-        const int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(32, 4096 / dimension))) : 1;
-        const size_t lds = use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0;
+        // LDS: `chunk` steps of `copies` private sets of per-channel sums, 32 KB at most
+        int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(8, 4096 / dimension))) : 1;
+        auto steps_for = [&](int cp) { return uint64_t(32768) / (uint64_t(cp) * dimension * sizeof(T)); };
+        while (copies > 1 && steps_for(copies) < 16) copies /= 2;
+        const int chunk = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(64, steps_for(copies)))) : 1;
+        const size_t lds = use_lds ? size_t(chunk) * size_t(copies) * size_t(dimension) * sizeof(T) : 0;
         const dim3 grid{unsigned(gx), unsigned(std::min<uint64_t>(batch, 65535)), 1};
         with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
             constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;
             hipLaunchKernelGGL((sig_coef_bwd_kernel<T, KMAX, UF>), grid, dim3(threads), lds, stream, path, out, coefs, derivs,
-                               words, int64_t(batch), int64_t(dimension), int64_t(length), int64_t(h.row), use_lds, copies);
+                               words, int64_t(batch), int64_t(dimension), int64_t(length), int64_t(h.row), use_lds, copies,
+                               chunk);
         });
         SIG_HIP(hipGetLastError());
         SIG_HIP(hipStreamSynchronize(stream));
