@@ -111,6 +111,88 @@ __global__ __launch_bounds__(kBlock) void sig_coef_kernel(
     }
 }
 
+// The same sweep with the path's points staged through LDS: a block serves up to 256 words of ONE path and copies
+// `chunk` points at a time with coalesced loads; the lanes then pick their letters' channels from LDS, the points of
+// kCoefAhead steps at a time.  (Picked straight from memory, every lane-indexed load occupies the texture addresser
+// for a whole wave whatever it coalesces to: 4 such loads per step were 61 % of a wave's cycles.)
+constexpr int kCoefAhead = 4;
+template <typename T, int KMAX, int UF>
+__global__ __launch_bounds__(kBlock) void sig_coef_staged_kernel(
+    const T* __restrict__ path, T* __restrict__ out, WordList words, int64_t batch, int64_t d, int64_t len, int64_t row,
+    int prefixes, int chunk)
+{
+    extern __shared__ double coef_rows_raw[];
+    T* rows = reinterpret_cast<T*>(coef_rows_raw);      // [chunk][d]
+    const int64_t w = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const bool live = w < int64_t(words.count);
+    const int k = live ? int(words.degree[w]) : 0;
+    const bool active = k > 0 && k <= KMAX;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* x = path + b * len * d;
+        int lo[KMAX];                                   // the letters as offsets into a row
+        T c[KMAX + 1], z[KMAX], prev[KMAX];
+#pragma unroll UF
+        for (int i = 0; i < KMAX; ++i) {
+            lo[i] = (active && i < k) ? int(words.letters[words.start[w] + i]) : 0;
+            prev[i] = len > 0 ? x[lo[i]] : T(0);
+            c[i + 1] = T(0);
+        }
+        c[0] = T(1);
+        for (int64_t s0 = 1; s0 < len; s0 += chunk) {
+            const int n = int(len - s0 < chunk ? len - s0 : chunk);
+            __syncthreads();                            // the chunk before has been consumed
+            for (int64_t e = threadIdx.x; e < int64_t(n) * d; e += blockDim.x) rows[e] = x[s0 * d + e];
+            __syncthreads();
+            if (active) {
+                int r = 0;
+                if constexpr (UF > 1) {
+                    for (; r + kCoefAhead <= n; r += kCoefAhead) {
+                        T cur[kCoefAhead][KMAX];
+#pragma unroll
+                        for (int u = 0; u < kCoefAhead; ++u) {
+#pragma unroll
+                            for (int i = 0; i < KMAX; ++i) cur[u][i] = rows[int64_t(r + u) * d + lo[i]];
+                        }
+#pragma unroll
+                        for (int u = 0; u < kCoefAhead; ++u) {
+#pragma unroll
+                            for (int i = 0; i < KMAX; ++i) {
+                                z[i] = cur[u][i] - prev[i];
+                                prev[i] = cur[u][i];
+                            }
+                            word_step<T, KMAX, UF, 1>(c, z, k);
+                        }
+                    }
+                }
+                for (; r < n; ++r) {
+#pragma unroll UF
+                    for (int i = 0; i < KMAX; ++i) {
+                        const T cur = rows[int64_t(r) * d + lo[i]];
+                        z[i] = cur - prev[i];
+                        prev[i] = cur;
+                    }
+                    word_step<T, KMAX, UF, 1>(c, z, k);
+                }
+            }
+        }
+        if (!live) continue;
+        T* o = out + b * row + (prefixes ? int64_t(words.out_start[w]) : w);
+        if (k == 0) { o[0] = T(1); continue; }
+        if (!active) continue;
+        if (prefixes) {
+#pragma unroll UF
+            for (int i = 1; i <= KMAX; ++i)
+                if (i <= k) o[i - 1] = c[i];
+        } else {
+            T last = c[1];
+#pragma unroll UF
+            for (int i = 2; i <= KMAX; ++i)
+                if (i == k) last = c[i];
+            o[0] = last;
+        }
+    }
+}
+
 // Reverse sweep of one (path, word) pair: coefficients before the step by exp(-z), then the adjoint of the step:
 // with st_j = ((1/i!) z_0 + c_1/(i-1)!) z_1 + ... (the Horner values of prefix length i),
 //   dz_{i-1} += g_i st_{i-1};  walking j = i-2 .. 0 with sd = g_i z_{i-1} z_{i-2} ..:  dz_j += sd st_j,
@@ -295,10 +377,23 @@ static void sig_coef_impl(const T* path, T* out, const uint64_t* multi_idx, uint
     hipStream_t stream = nullptr;
     std::lock_guard<std::mutex> lk(g_ws_mutex);
     const WordList words = upload_words(h, multi_idx, stream);
+    // points staged through LDS (a block per path and 256 words) when a chunk of at least 8 points fits 16 KB
+    const uint64_t fit = uint64_t(16384) / (dimension * sizeof(T));
+    const int chunk = int(std::min<uint64_t>(128, fit));
     with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
         constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;
-        hipLaunchKernelGGL((sig_coef_kernel<T, KMAX, UF>), dim3(grid_for(items)), dim3(kBlock), 0, stream, path, out, words,
-                           int64_t(batch), int64_t(dimension), int64_t(length), int64_t(row), int(prefixes));
+        if (chunk >= 8) {
+            const unsigned threads = num_words <= 64 ? 64u : unsigned(kBlock);
+            const uint64_t gx = (num_words + threads - 1) / threads;
+            if (gx > 0x7fffffffull) throw std::runtime_error("sig_coef_cuda: too many words");
+            const dim3 grid{unsigned(gx), unsigned(std::min<uint64_t>(batch, 65535)), 1};
+            hipLaunchKernelGGL((sig_coef_staged_kernel<T, KMAX, UF>), grid, dim3(threads),
+                               size_t(chunk) * size_t(dimension) * sizeof(T), stream, path, out, words, int64_t(batch),
+                               int64_t(dimension), int64_t(length), int64_t(row), int(prefixes), chunk);
+        } else {
+            hipLaunchKernelGGL((sig_coef_kernel<T, KMAX, UF>), dim3(grid_for(items)), dim3(kBlock), 0, stream, path, out, words,
+                               int64_t(batch), int64_t(dimension), int64_t(length), int64_t(row), int(prefixes));
+        }
     });
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
