@@ -210,6 +210,7 @@ __global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
 {
     extern __shared__ double coef_lds_raw[];
     T* acc = reinterpret_cast<T*>(coef_lds_raw);        // [chunk][copies][d]
+    T* rows = acc + int64_t(chunk) * copies * d;        // use_lds: the points s_lo - 1 .. s_hi of the chunk, [chunk + 1][d]
     const int64_t w = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     const bool live = w < int64_t(words.count);
     const int k = live ? int(words.degree[w]) : 0;
@@ -234,16 +235,24 @@ __global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
                 g[i + 1] = i < k ? grow[i] : T(0);
             }
         }
+        // copies the points of the chunk ending at step s_hi to LDS (coalesced; lane-indexed loads from memory occupy
+        // the texture addresser for a whole wave each)
+        auto stage = [&](int64_t s_hi) {
+            const int64_t s_lo = s_hi - chunk + 1 > 1 ? s_hi - chunk + 1 : 1;
+            const int64_t cnt = (s_hi - s_lo + 2) * d;
+            for (int64_t e = threadIdx.x; e < cnt; e += blockDim.x) rows[e] = x[(s_lo - 1) * d + e];
+        };
         if (use_lds) {
-            __syncthreads();        // the previous path's sums have been consumed
+            __syncthreads();        // the previous path's sums and points have been consumed
             for (int64_t j = threadIdx.x; j < int64_t(chunk) * slab; j += blockDim.x) acc[j] = T(0);
+            if (len >= 2) stage(len - 1);
             __syncthreads();
         }
         for (int64_t s_hi = len - 1; s_hi >= 1; s_hi -= chunk) {        // steps s_lo .. s_hi, downwards
             const int64_t s_lo = s_hi - chunk + 1 > 1 ? s_hi - chunk + 1 : 1;
             if (active) {
                 for (int64_t s = s_hi; s >= s_lo; --s) {                // step s-1 -> s
-                    const T* xp = x + (s - 1) * d;
+                    const T* xp = use_lds ? rows + (s - s_lo) * d : x + (s - 1) * d;
 #pragma unroll UF
                     for (int i = 0; i < KMAX; ++i) {
                         const T cur = xp[let[i]];
@@ -298,6 +307,7 @@ __global__ __launch_bounds__(kBlock) void sig_coef_bwd_kernel(
                 }
                 __syncthreads();
                 for (int64_t j = threadIdx.x; j < n * slab; j += blockDim.x) acc[j] = T(0);
+                if (s_hi - chunk >= 1) stage(s_hi - chunk);
                 __syncthreads();
             }
         }
@@ -422,13 +432,13 @@ static void sig_coef_backprop_impl(const T* path, T* out, const T* coefs, const 
         const unsigned threads = num_words <= 64 ? 64u : unsigned(kBlock);
         const uint64_t gx = (num_words + threads - 1) / threads;
         if (gx > 0x7fffffffull) throw std::runtime_error("sig_coef_backprop_cuda: too many words");
-        const int use_lds = dimension <= 4096;
-        // LDS: `chunk` steps of `copies` private sets of per-channel sums, 32 KB at most
+        const int use_lds = dimension <= 4096 && 3 * dimension * sizeof(T) <= 65536;      // one step's sums + two points fit
+        // LDS: `chunk` steps of `copies` private sets of per-channel sums, 32 KB at most, and the chunk's points
         int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(8, 4096 / dimension))) : 1;
         auto steps_for = [&](int cp) { return uint64_t(32768) / (uint64_t(cp) * dimension * sizeof(T)); };
         while (copies > 1 && steps_for(copies) < 16) copies /= 2;
         const int chunk = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(64, steps_for(copies)))) : 1;
-        const size_t lds = use_lds ? size_t(chunk) * size_t(copies) * size_t(dimension) * sizeof(T) : 0;
+        const size_t lds = use_lds ? (size_t(chunk) * size_t(copies) + size_t(chunk) + 1) * size_t(dimension) * sizeof(T) : 0;
         const dim3 grid{unsigned(gx), unsigned(std::min<uint64_t>(batch, 65535)), 1};
         with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
             constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;

@@ -461,6 +461,26 @@ def test_sig_coef_vs_oracle(P, oracle, aug, dtype, shape):
     assert bwd_err(got, want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("shape", [(2, 9, 300), (2, 6, 2800), (1, 5, 5000), (3, 200, 12)])
+def test_sig_coef_wide_and_long_paths(P, oracle, dtype, shape):
+    """Paths too wide for the LDS staging of the points (forward) or of the per-channel sums (backward) take the
+    kernels that read and add straight from / to memory; a long narrow path crosses several chunks of steps."""
+    rng = np.random.default_rng(shape[1] + shape[2])
+    x = (rng.uniform(size=shape) * 0.5).astype(dtype)
+    d = shape[2]
+    words = [(d - 1,), (0, d - 1), (d // 2, 1, d - 1), (), (d - 1, d - 1, 0), (1, 0, 1, d - 2)] + \
+            [tuple(int(v) for v in rng.integers(0, d, size=3)) for _ in range(70)]
+    cp = oracle.sig_coef(x, words, prefixes=True)
+    got = P.sig_coef(dev(x), words, prefixes=True).cpu().numpy()
+    assert bwd_err(got, cp) < TOL[dtype]
+    g = rng.standard_normal(cp.shape).astype(dtype)
+    want = oracle.sig_coef_backprop(x, words, cp, g)
+    got = P.sig_coef_backprop(dev(x), words, dev(cp), dev(g)).cpu().numpy()
+    assert got.shape == x.shape
+    assert bwd_err(got, want) < TOL[dtype]
+
+
 def bwd_err(got, ref):
     got = got.reshape(ref.shape[0], -1).astype(np.float64)
     ref = ref.reshape(ref.shape[0], -1).astype(np.float64)
