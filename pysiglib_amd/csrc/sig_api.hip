@@ -8,6 +8,8 @@
 // (siglib/shared/last_error.h:22-41).
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include <algorithm>
 #include <atomic>
 #include <charconv>
@@ -488,6 +490,7 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
 // degree 2 in closed form (matrix cores): taken for paths of many channels, where no specialised sweep exists
 // ---------------------------------------------------------------------------
 static Hook g_force_degree2{-1};    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
+static Hook g_degree2_wide{[] { const char* e = std::getenv("CUSIG_AMD_D2_WIDE"); return e ? std::atoi(e) : 1; }()};     // measurement switch
 static Hook g_degree2_staged{1};    // tuning hook: 0 keeps the operands of the degree-2 products out of LDS
 
 // Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
@@ -999,9 +1002,36 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             finish();
             return;
         }
-        hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug)), dim3(kBlock), 0, stream, path, sig_derivs, h,
+        hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug, kWavesPerBlock)), dim3(kBlock), 0, stream, path, sig_derivs, h,
                            int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
                            int64_t(s.stride), sc);
+        if (staged && g_degree2_wide != 0 && s.L >= 1 && !time_aug && !lead_lag) {
+            // more than 64 channels, plain paths: accumulators of a run of rows in registers, channels walked 64 at a
+            // time (with augmentation the per-element evaluation of the points makes it slower than the kernel below)
+            const bool plain = true;
+            const bool vec = plain && dimension % (16 / sizeof(T)) == 0 && reinterpret_cast<uintptr_t>(path) % 16 == 0;
+            const int64_t out_rows = plain ? int64_t(s.L) + 1 : int64_t(s.L);
+            const int64_t run = int64_t(deg2_wide_chunks<T>()) * kDeg2BwdRows;
+            const int64_t parts = (out_rows + run - 1) / run;
+            const int64_t blocks = int64_t(batch) * parts * col_groups;
+            if (blocks > 2147483647LL) throw std::runtime_error("sig_backprop_cuda: launch too large");
+            MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_bwd_f64_wide" : "degree2_bwd_f32_wide", !arena);
+            auto go = [&](auto mode) {
+                constexpr int MODE = decltype(mode)::value;
+                hipLaunchKernelGGL((degree2_bwd_wide_kernel<T, MODE>), dim3(unsigned(blocks)), dim3(kBlock), deg2_bwd_lds_bytes<T>(),
+                                   stream, path, sig_derivs, (const T*)h, MODE ? out : dzinc, int64_t(batch), int64_t(length),
+                                   int(dimension), int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, int(parts),
+                                   col_groups);
+            };
+            if (vec) go(std::integral_constant<int, 2>());
+            else if (plain) go(std::integral_constant<int, 1>());
+            else go(std::integral_constant<int, 0>());
+            timer.stop();
+            if (!plain) launch_path_grad<T>(dzinc, out, batch, length, dimension, time_aug, lead_lag, stream);
+            SIG_HIP(hipGetLastError());
+            finish();
+            return;
+        }
         MainKernelTimer timer(stream, sizeof(T) == 8 ? (staged ? "degree2_bwd_f64_lds" : "degree2_bwd_f64")
                                                      : (staged ? "degree2_bwd_f32_lds" : "degree2_bwd_f32"), !arena);
         if (staged) {

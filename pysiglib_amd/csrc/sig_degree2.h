@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kBlock) void finite_rows_kernel(const T* __restrict
     if (!(chk == T(0))) *nonfinite = 1;
 }
 
-// h[b][c] = G1[c] + sum_e G2[c][e] * S1[e]
+// h[b][c] = G1[c] + sum_e G2[c][e] * S1[e]: one wave per (path, c), its lanes a coalesced walk along the row
 template <typename T>
 __global__ __launch_bounds__(kBlock) void degree2_h_kernel(
     const T* __restrict__ path, const T* __restrict__ gsig, T* __restrict__ h, int64_t batch, int64_t len_raw, int d_raw,
@@ -351,23 +351,21 @@ __global__ __launch_bounds__(kBlock) void degree2_h_kernel(
 {
     const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
     const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
-    for (int64_t e = int64_t(blockIdx.x) * kBlock + threadIdx.x; e < batch * d; e += int64_t(gridDim.x) * kBlock) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t waves = int64_t(gridDim.x) * kWavesPerBlock;
+    for (int64_t e = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6); e < batch * d; e += waves) {
         const int64_t b = e / d;
         const int c = int(e - b * d);
         const T* x = path + b * len_raw * d_raw;
         const T* g = gsig + b * sig_stride + scalar;
-        T s0 = g[c], s1 = T(0);
-        int k = 0;
-        for (; k + 2 <= d; k += 2) {
-            const T v0 = aug_point(x, L, k, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k, d_raw, time_aug, lead_lag, d, time_step);
-            const T v1 = aug_point(x, L, k + 1, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k + 1, d_raw, time_aug, lead_lag, d, time_step);
-            s0 = fmadd(g[d + int64_t(c) * d + k], v0, s0);
-            s1 = fmadd(g[d + int64_t(c) * d + k + 1], v1, s1);
+        const T* grow = g + d + int64_t(c) * d;
+        T s0 = T(0);
+        for (int k = lane; k < d; k += kWave) {
+            const T v = aug_point(x, L, k, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k, d_raw, time_aug, lead_lag, d, time_step);
+            s0 = fmadd(grow[k], v, s0);
         }
-        if (k < d)
-            s0 = fmadd(g[d + int64_t(c) * d + k],
-                       aug_point(x, L, k, d_raw, time_aug, lead_lag, d, time_step) - aug_point(x, 0, k, d_raw, time_aug, lead_lag, d, time_step), s0);
-        h[e] = s0 + s1;
+        s0 = wave_sum(s0);
+        if (lane == 0) h[e] = g[c] + s0;
     }
 }
 
@@ -722,6 +720,186 @@ __global__ __launch_bounds__(kBlock, sizeof(T) == 8 ? 2 : 3) void degree2_bwd_ro
                         else v += hc;
                         o[row * d + c] = v;
                     }
+                }
+            }
+        }
+    }
+}
+
+// Backward for more than 64 channels.  A block serves (path, run of up to RC x 64 output rows, 64 columns) and keeps
+// the RC x kDeg2Cols accumulator tiles of all its rows in registers while it walks the channels 64 at a time: per
+// channel chunk it builds the fragments of the 64 x 64 block of (G2 - G2^T) / 2 once (the two blocks of G2 pass
+// through one LDS tile, one after the other) and then, for each 64-row chunk, copies the points' channels of that
+// chunk to LDS and runs the products as degree2_bwd_rows_kernel does.  h = G1 + G2 S1 comes from degree2_h_kernel.
+// MODE as in degree2_bwd_rows_kernel.
+template <typename T>
+constexpr int deg2_wide_chunks() { return sizeof(T) == 8 ? 2 : 4; }
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kBlock, 2) void degree2_bwd_wide_kernel(
+    const T* __restrict__ path, const T* __restrict__ gsig, const T* __restrict__ h, T* __restrict__ outp, int64_t batch,
+    int64_t len_raw, int d_raw, int time_aug, int lead_lag, T time_step, int64_t sig_stride, int scalar, int parts,
+    int col_groups)
+{
+    using M = Mfma16<T>;
+    using V = typename Vec16<T>::type;
+    constexpr int VN = Vec16<T>::n;
+    constexpr bool DIRECT = MODE != 0;
+    constexpr int HI = DIRECT ? 2 : 1;
+    constexpr int RC = deg2_wide_chunks<T>();
+    extern __shared__ __align__(16) double lds_raw_d2w[];
+    T* Ys = reinterpret_cast<T*>(lds_raw_d2w);
+    T* Gs = Ys + (kDeg2BwdRows + 2) * kDeg2BwdStride;
+    const int d = (lead_lag ? 2 * d_raw : d_raw) + (time_aug ? 1 : 0);
+    const int64_t L = (lead_lag ? 2 * len_raw - 1 : len_raw) - 1;
+    const int64_t out_rows = DIRECT ? L + 1 : L;
+    const int64_t per_path = int64_t(parts) * col_groups;
+    const int64_t b = int64_t(blockIdx.x) / per_path;
+    const int64_t w = int64_t(blockIdx.x) - b * per_path;
+    const int cg = int(w % col_groups);
+    const int64_t row_begin = (w / col_groups) * (RC * kDeg2BwdRows);
+    const int64_t row_end = row_begin + RC * kDeg2BwdRows < out_rows ? row_begin + RC * kDeg2BwdRows : out_rows;
+    if (row_begin >= row_end) return;
+    const T* x = path + b * len_raw * d_raw;
+    const T* g2 = gsig + b * sig_stride + scalar + d;
+    T* o = outp + b * out_rows * d;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int li = lane & 15, lk = lane >> 4;
+    const int c0 = cg * kDeg2Slab;
+    auto point = [&](int64_t t, int c) {
+        if constexpr (DIRECT) return x[t * d_raw + c];
+        else return aug_point(x, t, c, d_raw, time_aug, lead_lag, d, time_step);
+    };
+    constexpr int kVecCols = kDeg2Slab / VN, kVecRows = kBlock / kVecCols;
+    const int vcol = (tid % kVecCols) * VN, vrow0 = tid / kVecCols;
+    const int sc_col = tid % kDeg2Slab, sc_row0 = tid / kDeg2Slab;
+
+    typename M::Acc acc[RC][kDeg2Cols];
+#pragma unroll
+    for (int rc = 0; rc < RC; ++rc) {
+#pragma unroll
+        for (int j = 0; j < kDeg2Cols; ++j) acc[rc][j] = typename M::Acc{T(0), T(0), T(0), T(0)};
+    }
+
+    for (int a0 = 0; a0 < d; a0 += kDeg2Slab) {
+        // fragments of the block (a0 .., c0 ..) of (G2 - G2^T) / 2
+        __syncthreads();        // the products of the channel chunk before are done with Gs and Ys
+        for (int e = tid; e < kDeg2Slab * kDeg2Slab; e += kBlock) {
+            const int a = a0 + e / kDeg2Slab, c = c0 + e % kDeg2Slab;
+            Gs[(e / kDeg2Slab) * kDeg2GStride + e % kDeg2Slab] = (a < d && c < d) ? g2[int64_t(a) * d + c] : T(0);
+        }
+        __syncthreads();
+        T bf[16][kDeg2Cols];
+        if (wave == 0) {
+#pragma unroll
+            for (int kk = 0; kk < 16; ++kk) {
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) bf[kk][j] = Gs[(lk * 16 + kk) * kDeg2GStride + 16 * j + li];
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < kDeg2Slab * kDeg2Slab; e += kBlock) {
+            const int c = c0 + e / kDeg2Slab, a = a0 + e % kDeg2Slab;
+            Gs[(e / kDeg2Slab) * kDeg2GStride + e % kDeg2Slab] = (a < d && c < d) ? g2[int64_t(c) * d + a] : T(0);
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int kk = 0; kk < 16; ++kk) {
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j)
+                    bf[kk][j] = T(0.5) * (bf[kk][j] - Gs[(16 * j + li) * kDeg2GStride + lk * 16 + kk]);
+            }
+        }
+        __syncthreads();
+        T* Bf = Gs;                                     // [kk][lane][j]
+        if (wave == 0) {
+#pragma unroll
+            for (int kk = 0; kk < 16; ++kk) {
+#pragma unroll
+                for (int j = 0; j < kDeg2Cols; ++j) Bf[(kk * kWave + lane) * kDeg2Cols + j] = bf[kk][j];
+            }
+        }
+#pragma unroll
+        for (int rc = 0; rc < RC; ++rc) {
+            const int64_t base = row_begin + int64_t(rc) * kDeg2BwdRows;
+            if (base >= row_end) continue;          // block-uniform
+            __syncthreads();    // the chunk before has been consumed (first pass: Bf is complete)
+            if constexpr (MODE == 2) {
+                const bool v_ok = a0 + vcol < d;
+                const V x0v = v_ok ? *reinterpret_cast<const V*>(x + a0 + vcol) : V(T(0));
+                for (int r = vrow0; r < kDeg2BwdRows + 2; r += kVecRows) {
+                    const int64_t t = base + r - 1;
+                    const int64_t tc = t < 0 ? 0 : (t > L ? L : t);
+                    V v = v_ok ? *reinterpret_cast<const V*>(x + tc * d_raw + a0 + vcol) - x0v : V(T(0));
+                    if (t < 0 || t > L + 1) v = V(T(0));
+                    else if (t == L + 1) v = -v;
+                    *reinterpret_cast<V*>(Ys + r * kDeg2BwdStride + vcol) = v;
+                }
+            } else {
+                constexpr int kRowStep = kBlock / kDeg2Slab;
+                const int a = a0 + sc_col;
+                const T x0s = a < d ? point(0, a) : T(0);
+                for (int r0 = sc_row0; r0 < kDeg2BwdRows + 2; r0 += kRowStep * kDeg2StageBatch) {
+                    T v[kDeg2StageBatch];
+#pragma unroll
+                    for (int k = 0; k < kDeg2StageBatch; ++k) {
+                        const int64_t t = base + r0 + kRowStep * k - (DIRECT ? 1 : 0);
+                        const int64_t tc = t < 0 ? 0 : (t > L ? L : t);
+                        v[k] = a < d ? point(tc, a) - x0s : T(0);
+                        if (t < 0 || t > L + 1 || (!DIRECT && t > L)) v[k] = T(0);
+                        else if (t == L + 1) v[k] = -v[k];
+                    }
+#pragma unroll
+                    for (int k = 0; k < kDeg2StageBatch; ++k) {
+                        const int r = r0 + kRowStep * k;
+                        if (r < kDeg2BwdRows + 2) Ys[r * kDeg2BwdStride + sc_col] = v[k];
+                    }
+                }
+            }
+            __syncthreads();
+            if (base + 16 * wave < row_end) {
+                const T* lo = Ys + (16 * wave + li) * kDeg2BwdStride + lk * 16;
+                const T* hi = lo + HI * kDeg2BwdStride;
+                T u[16];
+#pragma unroll
+                for (int q = 0; q < 16 / VN; ++q) {
+                    const V va = *reinterpret_cast<const V*>(lo + q * VN), vc = *reinterpret_cast<const V*>(hi + q * VN);
+#pragma unroll
+                    for (int e = 0; e < VN; ++e) u[q * VN + e] = DIRECT ? va[e] - vc[e] : va[e] + vc[e];
+                }
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) {
+                    T bq[kDeg2Cols];
+#pragma unroll
+                    for (int q = 0; q < kDeg2Cols / VN; ++q) {
+                        const V v = *reinterpret_cast<const V*>(Bf + (kk * kWave + lane) * kDeg2Cols + q * VN);
+#pragma unroll
+                        for (int e = 0; e < VN; ++e) bq[q * VN + e] = v[e];
+                    }
+#pragma unroll
+                    for (int j = 0; j < kDeg2Cols; ++j) acc[rc][j] = M::mma(u[kk], bq[j], acc[rc][j]);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int rc = 0; rc < RC; ++rc) {
+        const int64_t base = row_begin + int64_t(rc) * kDeg2BwdRows;
+#pragma unroll
+        for (int j = 0; j < kDeg2Cols; ++j) {
+            const int c = c0 + 16 * j + li;
+            if (c >= d) continue;
+            const T hc = h[b * d + c];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t row = base + 16 * wave + M::row(lk, r);
+                if (row < row_end) {
+                    T v = acc[rc][j][r];
+                    if constexpr (DIRECT) v += row == 0 ? -hc : (row == L ? hc : T(0));
+                    else v += hc;
+                    o[row * d + c] = v;
                 }
             }
         }
