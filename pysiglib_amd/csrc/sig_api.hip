@@ -8,8 +8,6 @@
 // (siglib/shared/last_error.h:22-41).
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
-
 #include <algorithm>
 #include <atomic>
 #include <charconv>
@@ -490,7 +488,6 @@ static const KernelEntry* pick_variant(bool backward, const KernelEntry* base, i
 // degree 2 in closed form (matrix cores): taken for paths of many channels, where no specialised sweep exists
 // ---------------------------------------------------------------------------
 static Hook g_force_degree2{-1};    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 2
-static Hook g_degree2_wide{[] { const char* e = std::getenv("CUSIG_AMD_D2_WIDE"); return e ? std::atoi(e) : 1; }()};     // measurement switch
 static Hook g_degree2_staged{1};    // tuning hook: 0 keeps the operands of the degree-2 products out of LDS
 
 // Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
@@ -1005,7 +1002,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         hipLaunchKernelGGL((degree2_h_kernel<T>), dim3(grid_for(batch * s.d_aug, kWavesPerBlock)), dim3(kBlock), 0, stream, path, sig_derivs, h,
                            int64_t(batch), int64_t(length), int(dimension), int(time_aug), int(lead_lag), time_step,
                            int64_t(s.stride), sc);
-        if (staged && g_degree2_wide != 0 && s.L >= 1 && !time_aug && !lead_lag) {
+        if (staged && s.L >= 1 && !time_aug && !lead_lag) {
             // more than 64 channels, plain paths: accumulators of a run of rows in registers, channels walked 64 at a
             // time (with augmentation the per-element evaluation of the points makes it slower than the kernel below)
             const bool plain = true;
