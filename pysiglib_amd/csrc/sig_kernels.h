@@ -1135,6 +1135,36 @@ __device__ __forceinline__ WordPos<I> word_pos(I r, I d)
 // of A, B, C may have different strides and C may carry a leading scalar slot.
 // ---------------------------------------------------------------------------
 
+// LDS copies of the short levels of the two factors of a Chen product (chen_fan<.., LOW = true>): the block copies
+// the first low_n coefficients of each row; barriers on both sides
+template <typename T, typename I>
+__device__ __forceinline__ void stage_low_levels(T* al, T* bl, const T* __restrict__ a, const T* __restrict__ bb, I low_n)
+{
+    __syncthreads();        // the row before is done with the copies
+    for (I j = threadIdx.x; j < low_n; j += kBlock) {
+        al[j] = a[j];
+        bl[j] = bb[j];
+    }
+    __syncthreads();
+}
+// host: how many whole levels fit (two rows, at most 48 KB), never the top level; and the items a thread takes so that
+// the copy is amortised
+inline uint64_t chen_low_count(uint64_t d, uint64_t top, size_t elem_bytes)
+{
+    uint64_t n = 0, size = 1;
+    for (uint64_t t = 1; t < top; ++t) {
+        size *= d;
+        if (2 * (n + size) * elem_bytes > 48 * 1024) break;
+        n += size;
+    }
+    return n;
+}
+inline uint64_t chen_low_items_per_thread(uint64_t low_n)
+{
+    const uint64_t per = (2 * low_n + 255) / 256;       // loads of the copy per thread
+    return per < 1 ? 1 : (per > 8 ? 8 : per);
+}
+
 // The same sums for FAN outputs per thread: the words (a, rest) for FAN consecutive first letters a and one
 // `rest` of t - 1 letters.  Every split pairs a prefix (a, head of rest) with a suffix that does not depend on a, so
 // the suffix factor and all index arithmetic are shared by the outputs; consecutive threads hold consecutive `rest`
@@ -1207,8 +1237,12 @@ __device__ __forceinline__ FanItem<I> fan_item(I item, I d)
     return it;
 }
 
-template <typename T, typename I, int FAN, typename F>
-__device__ __forceinline__ void chen_fan(const T* __restrict__ a, const T* __restrict__ bb, I item, const DivBy<I>& dv, F&& f)
+// LOW: the first `low_n` coefficients of both rows (whole levels) also sit in LDS at `al` / `bl` (stage_low_levels) and
+// are read from there: most factors of a product belong to the short levels, and with all of them coming from memory
+// these kernels are bound by the rate of vector memory instructions, not by bandwidth (texture addresser ~90 % busy).
+template <typename T, typename I, int FAN, bool LOW = false, typename F>
+__device__ __forceinline__ void chen_fan(const T* __restrict__ a, const T* __restrict__ bb, I item, const DivBy<I>& dv, F&& f,
+                                         const T* al = nullptr, const T* bl = nullptr, I low_n = 0)
 {
     constexpr int kChenFan = FAN;
     const I d = I(dv.d);
@@ -1229,12 +1263,23 @@ __device__ __forceinline__ void chen_fan(const T* __restrict__ a, const T* __res
         lev = dv.quot(lev);             // d^k
         a_lo -= lev;
         const I st = dv.quot(lev);      // d^(k-1): distance between the prefixes of consecutive first letters
-        const T bv = bb[b_lo + suf];
-        const T* ap = a + a_lo + pre;
+        T bv;
+        if (LOW && b_lo + suf < low_n) bv = bl[b_lo + suf];
+        else bv = bb[b_lo + suf];
+        if (LOW && a_lo < low_n) {      // a whole level: the same for every lane of the block but at level borders
+            const T* ap = al + a_lo + pre;
 #pragma unroll
-        for (int i = 0; i < kChenFan; ++i) {
-            const I letter = a0 + i < d ? a0 + i : d - 1;      // surplus outputs shadow the last letter
-            acc[i] = fmadd(ap[letter * st], bv, acc[i]);
+            for (int i = 0; i < kChenFan; ++i) {
+                const I letter = a0 + i < d ? a0 + i : d - 1;
+                acc[i] = fmadd(ap[letter * st], bv, acc[i]);
+            }
+        } else {
+            const T* ap = a + a_lo + pre;
+#pragma unroll
+            for (int i = 0; i < kChenFan; ++i) {
+                const I letter = a0 + i < d ? a0 + i : d - 1;      // surplus outputs shadow the last letter
+                acc[i] = fmadd(ap[letter * st], bv, acc[i]);
+            }
         }
         b_lo += pw;
     }
@@ -1247,14 +1292,19 @@ template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void sig_combine_kernel(
     const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int64_t batch, DivBy<I> dv,
     I items /* chen_items(d, degree, FAN) */, int64_t a_stride, int64_t b_stride, int64_t c_stride,
-    int a_off, int b_off, int c_off)
+    int a_off, int b_off, int c_off, I low_n /* chen_low_count: dynamic LDS of 2 * low_n entries; 0 = none */)
 {
+    extern __shared__ double chen_low_raw[];
+    T* al = reinterpret_cast<T*>(chen_low_raw);
+    T* bl = al + low_n;
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * a_stride + a_off;
         const T* bb = B + b * b_stride + b_off;
         T* c = C + b * c_stride;
+        if (low_n) stage_low_levels(al, bl, a, bb, low_n);
         for (I it = I(blockIdx.x) * kBlock + threadIdx.x; it < items; it += I(gridDim.x) * kBlock) {
-            chen_fan<T, I, FAN>(a, bb, it, dv, [&](I r, T sum) { c[c_off + r] = a[r] + bb[r] + sum; });
+            if (low_n) chen_fan<T, I, FAN, true>(a, bb, it, dv, [&](I r, T sum) { c[c_off + r] = a[r] + bb[r] + sum; }, al, bl, low_n);
+            else chen_fan<T, I, FAN>(a, bb, it, dv, [&](I r, T sum) { c[c_off + r] = a[r] + bb[r] + sum; });
             if (c_off && it == 0) c[0] = T(1);
         }
     }

@@ -30,15 +30,21 @@ namespace sigamd {
 template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
     const T* __restrict__ X, const T* __restrict__ Pin, T* __restrict__ Pout, int64_t batch, DivBy<I> dv,
-    I items /* chen_items(d, levels, FAN) */, T inv_k, int64_t stride, int off, int64_t out_stride, int final)
+    I items /* chen_items(d, levels, FAN) */, T inv_k, int64_t stride, int off, int64_t out_stride, int final,
+    I low_n /* chen_low_count: dynamic LDS of 2 * low_n entries; 0 = none */)
 {
+    extern __shared__ double log_low_raw[];
+    T* xl = reinterpret_cast<T*>(log_low_raw);
+    T* pl = xl + low_n;
     for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
         const T* x = X + b * stride + off;
         const T* pin = Pin + b * stride + off;
         T* po = Pout + b * out_stride + off;
+        if (low_n) stage_low_levels(xl, pl, x, pin, low_n);
         for (I it = I(xcd_block_2d().x) * kBlock + threadIdx.x; it < items; it += I(gridDim.x) * kBlock) {
             // the splits after l = 1 .. t-1 letters, several first letters per thread as in the Chen product kernels
-            chen_fan<T, I, FAN>(x, pin, it, dv, [&](I r, T sum) { po[r] = inv_k * x[r] - sum; });
+            if (low_n) chen_fan<T, I, FAN, true>(x, pin, it, dv, [&](I r, T sum) { po[r] = inv_k * x[r] - sum; }, xl, pl, low_n);
+            else chen_fan<T, I, FAN>(x, pin, it, dv, [&](I r, T sum) { po[r] = inv_k * x[r] - sum; });
             if (final && off && it == 0) po[-off] = T(0);
         }
     }
@@ -231,10 +237,13 @@ static void run_tensor_log(const T* sig, T* out, uint64_t batch, uint64_t dimens
             with_chen_fan(dimension, [&](auto fan) {
                 constexpr int FAN = decltype(fan)::value;
                 const uint64_t items = chen_items(dimension, degree - k + 1, FAN);
-                launch_indexed(0, items, batch, [&](auto, dim3 grid) {
-                    hipLaunchKernelGGL((tensor_log_step_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig, pin, pout,
-                                       int64_t(batch), dv, I(items), T(sign) / T(k), int64_t(s.stride), s.off, int64_t(s.stride),
-                                       int(k == 1));
+                // the short levels of x and P_{k+1} in LDS (the step with one level computes no product and needs none)
+                const uint64_t low_n = degree - k + 1 >= 3 ? chen_low_count(dimension, degree - k + 1, sizeof(T)) : 0;
+                const uint64_t per_thread = chen_low_items_per_thread(low_n);
+                launch_indexed(0, (items + per_thread - 1) / per_thread, batch, [&](auto, dim3 grid) {
+                    hipLaunchKernelGGL((tensor_log_step_kernel<T, I, FAN>), grid, dim3(kBlock), 2 * low_n * sizeof(T), stream, sig,
+                                       pin, pout, int64_t(batch), dv, I(items), T(sign) / T(k), int64_t(s.stride), s.off,
+                                       int64_t(s.stride), int(k == 1), I(low_n));
                 });
             });
         }

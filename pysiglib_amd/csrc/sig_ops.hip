@@ -350,11 +350,14 @@ static void sig_combine_impl(const T* sig1, const T* sig2, T* out, uint64_t batc
         with_chen_fan(dimension, [&](auto fan) {
             constexpr int FAN = decltype(fan)::value;
             const uint64_t items = chen_items(dimension, degree, FAN);
-            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+            // the short levels of both factors in LDS; a thread then takes several items, so that the copy is amortised
+            const uint64_t low_n = chen_low_count(dimension, degree, sizeof(T));
+            const uint64_t per_thread = chen_low_items_per_thread(low_n);
+            launch_indexed(s.n_coef, (items + per_thread - 1) / per_thread, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
-                hipLaunchKernelGGL((sig_combine_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig1, sig2, out, int64_t(batch),
-                                   DivBy<I>(dimension), I(items), int64_t(s.stride), int64_t(s.stride), int64_t(s.stride),
-                                   s.off, s.off, s.off);
+                hipLaunchKernelGGL((sig_combine_kernel<T, I, FAN>), grid, dim3(kBlock), 2 * low_n * sizeof(T), stream, sig1, sig2, out,
+                                   int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), int64_t(s.stride),
+                                   int64_t(s.stride), s.off, s.off, s.off, I(low_n));
             });
         });
     }
