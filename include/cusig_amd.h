@@ -259,6 +259,9 @@ CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) CUSIG_AMD_NOEXCEPT;
  * backward, time-split sig_backprop): 0 = streaming kernels for rows of 4096 coefficients or more, 1 = streaming
  * kernels wherever they apply, 2 = item-per-word kernels only. */
 CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) CUSIG_AMD_NOEXCEPT;
+/* Test hook: the Chen product kernels of sig_combine and of the tensor logarithm can keep the factors' short levels in
+ * LDS: 0 = never, 1 (default) = for float64 rows of large launches, 2 = always. */
+CUSIG_AMD_API void cusig_amd_set_chen_low_levels(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Stream-ordered mode (no counterpart in the reference, off by default).  When enabled, signature_cuda_{f,d} and
  * sig_backprop_cuda_{f,d} enqueue their kernels on the null stream and return without waiting, and do not wait for
  * other streams on entry: inputs must be ordered before, and consumers after, the null stream (true for PyTorch's

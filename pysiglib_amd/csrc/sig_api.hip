@@ -192,6 +192,7 @@ struct Workspace {
 };
 std::atomic<int> g_force_wide_index{0};
 std::atomic<int> g_chen_adjoint_mode{0};
+std::atomic<int> g_chen_low_levels{1};
 std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
@@ -1353,6 +1354,7 @@ CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = 
 
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
 CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) noexcept { g_chen_adjoint_mode = mode; }
+CUSIG_AMD_API void cusig_amd_set_chen_low_levels(int enabled) noexcept { g_chen_low_levels = enabled; }
 
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
 

@@ -1147,22 +1147,28 @@ __device__ __forceinline__ void stage_low_levels(T* al, T* bl, const T* __restri
     }
     __syncthreads();
 }
-// host: how many whole levels fit (two rows, at most 48 KB), never the top level; and the items a thread takes so that
-// the copy is amortised
-inline uint64_t chen_low_count(uint64_t d, uint64_t top, size_t elem_bytes)
+// host: how many whole levels are copied, never the top level: at most 1536 coefficients per row (a longer copy costs a
+// block more than its reads save).  Only for 8-byte elements (measured: +8..30 % for float64 rows, -9..+10 % for
+// float32) and only when the launch keeps at least 4096 blocks after every thread has taken several items to amortise
+// the copy (`blocks` = blocks of the launch at one item per thread).
+extern std::atomic<int> g_chen_low_levels;      // test hook (defined in sig_api.hip): 0 = no copies, 1 = automatic, 2 = always
+inline uint64_t chen_low_items_per_thread(uint64_t low_n, uint64_t blocks)
 {
+    const uint64_t per = (2 * low_n + 255) / 256;       // loads of the copy per thread
+    const uint64_t room = g_chen_low_levels == 2 ? per : blocks / 4096;
+    const uint64_t take = per < room ? per : room;
+    return take < 1 ? 1 : (take > 8 ? 8 : take);
+}
+inline uint64_t chen_low_count(uint64_t d, uint64_t top, size_t elem_bytes, uint64_t blocks)
+{
+    if (!g_chen_low_levels || (g_chen_low_levels != 2 && (elem_bytes < 8 || blocks < 8192))) return 0;
     uint64_t n = 0, size = 1;
     for (uint64_t t = 1; t < top; ++t) {
         size *= d;
-        if (2 * (n + size) * elem_bytes > 48 * 1024) break;
+        if (n + size > 1536) break;
         n += size;
     }
     return n;
-}
-inline uint64_t chen_low_items_per_thread(uint64_t low_n)
-{
-    const uint64_t per = (2 * low_n + 255) / 256;       // loads of the copy per thread
-    return per < 1 ? 1 : (per > 8 ? 8 : per);
 }
 
 // The same sums for FAN outputs per thread: the words (a, rest) for FAN consecutive first letters a and one

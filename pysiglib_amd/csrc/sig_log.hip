@@ -238,8 +238,9 @@ static void run_tensor_log(const T* sig, T* out, uint64_t batch, uint64_t dimens
                 constexpr int FAN = decltype(fan)::value;
                 const uint64_t items = chen_items(dimension, degree - k + 1, FAN);
                 // the short levels of x and P_{k+1} in LDS (the step with one level computes no product and needs none)
-                const uint64_t low_n = degree - k + 1 >= 3 ? chen_low_count(dimension, degree - k + 1, sizeof(T)) : 0;
-                const uint64_t per_thread = chen_low_items_per_thread(low_n);
+                const uint64_t blocks = (items + kBlock - 1) / kBlock * batch;
+                const uint64_t low_n = degree - k + 1 >= 3 ? chen_low_count(dimension, degree - k + 1, sizeof(T), blocks) : 0;
+                const uint64_t per_thread = low_n ? chen_low_items_per_thread(low_n, blocks) : 1;
                 launch_indexed(0, (items + per_thread - 1) / per_thread, batch, [&](auto, dim3 grid) {
                     hipLaunchKernelGGL((tensor_log_step_kernel<T, I, FAN>), grid, dim3(kBlock), 2 * low_n * sizeof(T), stream, sig,
                                        pin, pout, int64_t(batch), dv, I(items), T(sign) / T(k), int64_t(s.stride), s.off,

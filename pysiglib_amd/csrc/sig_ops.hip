@@ -351,8 +351,9 @@ static void sig_combine_impl(const T* sig1, const T* sig2, T* out, uint64_t batc
             constexpr int FAN = decltype(fan)::value;
             const uint64_t items = chen_items(dimension, degree, FAN);
             // the short levels of both factors in LDS; a thread then takes several items, so that the copy is amortised
-            const uint64_t low_n = chen_low_count(dimension, degree, sizeof(T));
-            const uint64_t per_thread = chen_low_items_per_thread(low_n);
+            const uint64_t blocks = (items + kBlock - 1) / kBlock * batch;
+            const uint64_t low_n = chen_low_count(dimension, degree, sizeof(T), blocks);
+            const uint64_t per_thread = low_n ? chen_low_items_per_thread(low_n, blocks) : 1;
             launch_indexed(s.n_coef, (items + per_thread - 1) / per_thread, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
                 hipLaunchKernelGGL((sig_combine_kernel<T, I, FAN>), grid, dim3(kBlock), 2 * low_n * sizeof(T), stream, sig1, sig2, out,

@@ -43,6 +43,18 @@ def chen_mode(request):
     L.CUSIG.cusig_amd_force_chen_adjoint(0)
 
 
+@pytest.fixture(params=[1, 2], ids=["low-auto", "low-lds"])
+def chen_low(request):
+    """Chen product kernels (sig_combine, tensor logarithm): automatic choice, then the factors' short levels kept in LDS
+    for every shape and element type."""
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_set_chen_low_levels.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_chen_low_levels.restype = None
+    L.CUSIG.cusig_amd_set_chen_low_levels(request.param)
+    yield request.param
+    L.CUSIG.cusig_amd_set_chen_low_levels(1)
+
+
 def dev(a, dtype=None):
     return torch.tensor(np.ascontiguousarray(a, dtype=dtype), device=DEV)
 
@@ -66,7 +78,7 @@ def test_combine_kats(P):
                                          (37, 2, 5), (2, 14, 2), (4, 4, 9), (6, 3, 5), (11, 3, 3), (13, 3, 5), (9, 4, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_combine_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
+def test_combine_vs_oracle(P, oracle, chen_low, d, deg, batch, dtype, scalar_term):
     rng = np.random.default_rng(100 * d + deg)
     n = oracle.sig_length(d, deg) - 1
     scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
@@ -589,7 +601,7 @@ def test_log_sig_backprop_golden(P, fixtures, deg, dtype):
                                          (40, 2, 3), (2, 12, 2), (6, 4, 3), (13, 3, 2)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_sig_to_log_sig_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, scalar_term):
+def test_sig_to_log_sig_vs_oracle(P, oracle, chen_mode, chen_low, d, deg, batch, dtype, scalar_term):
     rng = np.random.default_rng(3 * d + deg)
     n = oracle.sig_length(d, deg) - 1
     scale = np.concatenate([np.full(d ** k, 0.5 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)]) if deg else np.zeros(0)
