@@ -135,15 +135,27 @@ __global__ __launch_bounds__(kBlock) void linear_sig_kernel(
 // append: the products of trailing letters are shared, the prefixes (a, head of rest) differ by d^(t-k-1) per letter;
 // prepend: every term with k >= 1 carries the factor z[a] and otherwise depends on `rest` only, so
 //   out_t[(a, rest)] = A_t[(a, rest)] + z[a] * C(rest),   C = sum_{k=1..t} z[r_1] .. z[r_{k-1}] / k! * A_{t-k}[r_k .. r_{t-1}].
+// low_n > 0 (append form): the block keeps the first low_n coefficients of A (whole levels) and the d letters' values in
+// LDS (dynamic, low_n + d entries) and reads the prefixes of those levels from there, as the Chen product kernels do.
 template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void sig_join_kernel(
     const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I items,
-    int64_t stride, int off, int prepend)
+    int64_t stride, int off, int prepend, I low_n)
 {
+    extern __shared__ double join_low_raw[];
+    T* al = reinterpret_cast<T*>(join_low_raw);
+    T* zl = al + low_n;
     const I d = I(dv.d);
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * stride + off;
         const T* z = disp + b * int64_t(d);
+        if (low_n) {
+            __syncthreads();        // the row before is done with the copies
+            for (I j = threadIdx.x; j < low_n; j += kBlock) al[j] = a[j];
+            for (I j = threadIdx.x; j < d; j += kBlock) zl[j] = z[j];
+            __syncthreads();
+            z = zl;
+        }
         T* o = out + b * stride;
         for (I item = I(blockIdx.x) * kBlock + threadIdx.x; item < items; item += I(gridDim.x) * kBlock) {
             const FanItem<I> fi = fan_item<I, FAN>(item, d);
@@ -162,11 +174,20 @@ __global__ __launch_bounds__(kBlock) void sig_join_kernel(
                     lev = dv.quot(lev);            // d^(t-k)
                     lo -= lev;
                     const I st = dv.quot(lev);     // d^(t-k-1): distance between the prefixes of consecutive first letters
-                    const T* ap = a + lo + head;
+                    if (lo < low_n) {           // a whole level: the same for every lane but at level borders
+                        const T* ap = al + lo + head;
 #pragma unroll
-                    for (int i = 0; i < FAN; ++i) {
-                        const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
-                        acc[i] = fmadd(ap[letter * st], ek, acc[i]);
+                        for (int i = 0; i < FAN; ++i) {
+                            const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
+                            acc[i] = fmadd(ap[letter * st], ek, acc[i]);
+                        }
+                    } else {
+                        const T* ap = a + lo + head;
+#pragma unroll
+                        for (int i = 0; i < FAN; ++i) {
+                            const I letter = fi.a0 + i < d ? fi.a0 + i : d - 1;
+                            acc[i] = fmadd(ap[letter * st], ek, acc[i]);
+                        }
                     }
                 }
                 // k = t: the empty prefix (A_0 = 1) and the whole word's product
@@ -432,10 +453,14 @@ static void sig_join_impl(const T* sig, const T* disp, T* out, uint64_t batch, u
         with_chen_fan(dimension, [&](auto fan) {
             constexpr int FAN = decltype(fan)::value;
             const uint64_t items = chen_items(dimension, degree, FAN);
-            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+            const uint64_t blocks = (items + kBlock - 1) / kBlock * batch;
+            const uint64_t low_n = prepend ? 0 : chen_low_count(dimension, degree, sizeof(T), blocks);
+            const uint64_t per_thread = low_n ? chen_low_items_per_thread(low_n, blocks) : 1;
+            launch_indexed(s.n_coef, (items + per_thread - 1) / per_thread, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
-                hipLaunchKernelGGL((sig_join_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, sig, disp, out, int64_t(batch),
-                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, int(prepend));
+                hipLaunchKernelGGL((sig_join_kernel<T, I, FAN>), grid, dim3(kBlock), low_n ? (low_n + dimension) * sizeof(T) : 0,
+                                   stream, sig, disp, out, int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), s.off,
+                                   int(prepend), I(low_n));
             });
         });
     }

@@ -308,7 +308,7 @@ def test_linear_sig_vs_oracle(P, oracle, d, deg, batch, dtype, scalar_term):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("prepend", [False, True])
 @pytest.mark.parametrize("scalar_term", [False, True])
-def test_sig_join_vs_oracle(P, oracle, chen_mode, d, deg, batch, dtype, prepend, scalar_term):
+def test_sig_join_vs_oracle(P, oracle, chen_mode, chen_low, d, deg, batch, dtype, prepend, scalar_term):
     rng = np.random.default_rng(5 * d + deg)
     n = oracle.sig_length(d, deg) - 1
     scale = np.concatenate([np.full(d ** k, 1.0 / np.sqrt(float(d) ** k)) for k in range(1, deg + 1)])
