@@ -128,6 +128,86 @@ __global__ __launch_bounds__(kBlock) void linear_sig_kernel(
     }
 }
 
+// The same rows with a level per block: a thread takes one word `rest` of t - 1 letters and writes the d words
+// (a, rest): one product per d outputs, and the level, its size and its start are block-uniform (scalar arithmetic),
+// where the item form above spends ~60 instructions per output on finding them per thread.  Stores stay coalesced
+// (consecutive threads, consecutive `rest`).  The block keeps z in LDS (dynamic, d entries) when z_lds is set.
+struct LevelBlocks {
+    int top;
+    uint32_t first[kExpMaxDegree + 2];      // first block of level t, t = 1 .. top; first[top + 1] = number of blocks
+};
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void linear_sig_levels_kernel(
+    const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, LevelBlocks lb, int64_t stride, int off,
+    int z_lds)
+{
+    extern __shared__ double linear_lds_raw[];
+    T* zl = reinterpret_cast<T*>(linear_lds_raw);
+    const I d = I(dv.d);
+    int t = 1;
+    while (t < lb.top && blockIdx.x >= lb.first[t + 1]) ++t;
+    I size = 1, lo = 0;                     // d^(t-1), start of level t
+    T scale = T(1);                         // 1 / t!
+    for (int k = 1; k < t; ++k) {
+        lo += size * d;
+        size *= d;
+    }
+    for (int k = 1; k <= t; ++k) scale *= rcp_of<T>(k);
+    const I rest = I(blockIdx.x - lb.first[t]) * kBlock + threadIdx.x;
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* z = disp + b * int64_t(d);
+        if (z_lds) {
+            __syncthreads();                // the row before is done with the copy
+            for (I j = threadIdx.x; j < d; j += kBlock) zl[j] = z[j];
+            __syncthreads();
+            z = zl;
+        }
+        T* o = out + b * stride;
+        if (rest < size) {
+            T v = scale;
+            I idx = rest;
+            for (int k = t - 1; k >= 1; --k) {      // letters of rest from the right
+                const I q = dv.quot(idx);
+                v *= z[idx - q * d];
+                idx = q;
+            }
+            T* dst = o + off + lo + rest;
+            for (I a = 0; a < d; ++a) dst[a * size] = v * z[a];
+        }
+        if (off && blockIdx.x == 0 && threadIdx.x == 0) o[0] = T(1);
+    }
+}
+// host: the launch of linear_sig_levels_kernel for rows of `top` levels; false when the blocks do not fit a grid
+static bool level_blocks(uint64_t d, uint64_t top, LevelBlocks& lb)
+{
+    if (top > uint64_t(kExpMaxDegree)) return false;
+    lb.top = int(top);
+    uint64_t blocks = 0, size = 1;
+    for (uint64_t t = 1; t <= top; ++t) {
+        lb.first[t] = uint32_t(blocks);
+        blocks += (size + kBlock - 1) / kBlock;
+        if (blocks > 0x7fffffffull) return false;
+        size *= d;
+    }
+    lb.first[top + 1] = uint32_t(blocks);
+    return true;
+}
+template <typename T>
+static bool launch_linear_sig_levels(const T* disp, T* out, uint64_t batch, uint64_t dimension, uint64_t top, uint64_t n_coef,
+                                     int64_t stride, int off, hipStream_t stream)
+{
+    LevelBlocks lb;
+    if (top < 1 || !level_blocks(dimension, top, lb)) return false;
+    const int z_lds = dimension * sizeof(T) <= 32768;
+    const dim3 grid{lb.first[top + 1], unsigned(std::min<uint64_t>(batch, 65535)), 1};
+    launch_indexed(n_coef, 1, 1, [&](auto ix, dim3) {
+        using I = decltype(ix);
+        hipLaunchKernelGGL((linear_sig_levels_kernel<T, I>), grid, dim3(kBlock), z_lds ? size_t(dimension) * sizeof(T) : 0, stream,
+                           disp, out, int64_t(batch), DivBy<I>(dimension), lb, stride, off, z_lds);
+    });
+    return true;
+}
+
 // out = A (x) exp(z) (append) or exp(z) (x) A (prepend):
 //   append : out_t[w] = sum_{k=0..t} A_{t-k}[w_1..w_{t-k}] * z[w_{t-k+1}] ... z[w_t] / k!
 //   prepend: out_t[w] = sum_{k=0..t} z[w_1] ... z[w_k] / k! * A_{t-k}[w_{k+1}..w_t]          (A_0 = 1)
@@ -422,15 +502,16 @@ static void linear_sig_impl(const T* disp, T* out, uint64_t batch, uint64_t dime
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch)), dim3(kBlock), 0, stream, out, int64_t(batch),
                                int64_t(1), 1);
     } else {
-        with_chen_fan(dimension, [&](auto fan) {
-            constexpr int FAN = decltype(fan)::value;
-            const uint64_t items = chen_items(dimension, degree, FAN);
-            launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
-                using I = decltype(ix);
-                hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, out, int64_t(batch),
-                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+        if (!launch_linear_sig_levels<T>(disp, out, batch, dimension, degree, s.n_coef, int64_t(s.stride), s.off, stream))
+            with_chen_fan(dimension, [&](auto fan) {
+                constexpr int FAN = decltype(fan)::value;
+                const uint64_t items = chen_items(dimension, degree, FAN);
+                launch_indexed(s.n_coef, items, batch, [&](auto ix, dim3 grid) {
+                    using I = decltype(ix);
+                    hipLaunchKernelGGL((linear_sig_kernel<T, I, FAN>), grid, dim3(kBlock), 0, stream, disp, out, int64_t(batch),
+                                       DivBy<I>(dimension), I(items), int64_t(s.stride), s.off);
+                });
             });
-        });
     }
     SIG_HIP(hipGetLastError());
     SIG_HIP(hipStreamSynchronize(stream));
@@ -490,7 +571,7 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
     T* E = static_cast<T*>(workspace(4, bytes));
     T* dE = static_cast<T*>(workspace(5, bytes));
     // exp(z) up to level degree - 1: the adjoint never multiplies with a factor's top level
-    if (degree >= 2)
+    if (degree >= 2 && !launch_linear_sig_levels<T>(disp, E, batch, dimension, degree - 1, s.n_coef, int64_t(s.stride), s.off, stream))
         with_chen_fan(dimension, [&](auto fan) {
             constexpr int FAN = decltype(fan)::value;
             const uint64_t items = chen_items(dimension, degree - 1, FAN);
