@@ -399,7 +399,8 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
     int best = 1;
     double best_t = estimate(1);
     const double whole = best_t;
-    for (int g : {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32}) {
+    // (one very long path of few channels: hundreds of pieces, each further doubling one more 10 us fold)
+    for (int g : {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024}) {
         if (L / g < 48 || uint64_t(g) * sig_bytes_all_paths > (uint64_t(256) << 20)) break;
         const double t = estimate(g);
         if (t < best_t) { best = g; best_t = t; }
@@ -445,7 +446,7 @@ static int choose_bwd_segments(int64_t waves, int64_t L, int waves_per_simd, uin
     int best = 1;
     double best_t = estimate(1);
     const double whole = best_t;
-    for (int g : {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64}) {
+    for (int g : {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512}) {
         if (L / g < 32 || uint64_t(g) * sig_bytes_all_paths > (uint64_t(64) << 20)) break;
         const double t = estimate(g);
         if (t < best_t) { best = g; best_t = t; }

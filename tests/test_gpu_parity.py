@@ -675,6 +675,7 @@ def test_time_segmented_backward(P, oracle, segments):
     ((2, 5, 98, 2), np.float64), ((2, 4, 350, 2), np.float32), ((1, 3, 1000, 2), np.float64),     # wide paths, low degree
     ((70000, 3, 2, 2), np.float32), ((66000, 4, 3, 3), np.float64),                                # batch beyond 65535
     ((3, 2000, 2, 4), np.float64), ((1, 20001, 3, 3), np.float64),                                 # long paths
+    ((1, 100000, 3, 6), np.float64), ((1, 65536, 2, 10), np.float64), ((2, 16000, 5, 5), np.float64),      # hundreds of time pieces
     ((2, 6, 2, 16), np.float64), ((1, 4, 3, 11), np.float64),                                      # highest compiled degrees
     ((2, 6, 2, 20), np.float64), ((1, 5, 2, 24), np.float64), ((1, 4, 3, 17), np.float64),         # run-time-degree sweeps
     ((2, 5, 2, 18), np.float32),
