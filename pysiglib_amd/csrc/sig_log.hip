@@ -50,6 +50,24 @@ __global__ __launch_bounds__(kBlock) void tensor_log_step_kernel(
     }
 }
 
+// The same step evaluated only at the `count` coefficients listed in `index` (positions in a scalar-free row): the last
+// step of the recursion when only the Lyndon words' coordinates of the logarithm are wanted (a fifth of the row at
+// d = 10, degree 5).  With one output per work item the item number of the Chen product kernels IS the coefficient's
+// position, so the listed positions are fed to chen_fan directly.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void tensor_log_step_at_kernel(
+    const T* __restrict__ X, const T* __restrict__ Pin, T* __restrict__ Pout, int64_t batch, DivBy<I> dv,
+    const uint64_t* __restrict__ index, int64_t count, T inv_k, int64_t stride, int off, int64_t out_stride)
+{
+    for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
+        const T* x = X + b * stride + off;
+        const T* pin = Pin + b * stride + off;
+        T* po = Pout + b * out_stride + off;
+        for (int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x; i < count; i += int64_t(gridDim.x) * kBlock)
+            chen_fan<T, I, 1>(x, pin, I(index[i]), dv, [&](I r, T sum) { po[r] = inv_k * x[r] - sum; });
+    }
+}
+
 // after the adjoint of x (x) P_{k+1} with -P_{k+1} as the left factor's partner (tmpB w.r.t. P_{k+1}; w.r.t. x:
 // -tmpA, which the k = 1 call has already added to g inside dx and the later calls leave in `neg_a`):
 //   g_next = -tmpB,   dx += neg_a + g_next / (k + 1)      over the `count_next` coefficients of levels <= N - k
@@ -276,7 +294,18 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
     const uint64_t elems = batch * s.stride;
     // Lyndon coordinates are read off the expanded logarithm, which then lives in a scratch copy
     T* expanded = method ? static_cast<T*>(workspace(14, bytes)) : out;
-    run_tensor_log<T>(sig, expanded, batch, dimension, degree, s, stream, [&](uint64_t k) { return ws + (k & 1) * elems; });
+    if (method && degree >= 2) {
+        // only the Lyndon words' coordinates are read below: the last step, most of the work, is evaluated at those
+        run_tensor_log<T>(sig, expanded, batch, dimension, degree, s, stream, [&](uint64_t k) { return ws + (k & 1) * elems; }, 2);
+        launch_indexed(s.n_coef, lyn.count, batch, [&](auto ix, dim3 grid) {
+            using I = decltype(ix);
+            hipLaunchKernelGGL((tensor_log_step_at_kernel<T, I>), grid, dim3(kBlock), 0, stream, sig, (const T*)(ws + (2 & 1) * elems),
+                               expanded, int64_t(batch), DivBy<I>(dimension), (const uint64_t*)lyn.index, int64_t(lyn.count), T(1),
+                               int64_t(s.stride), s.off, int64_t(s.stride));
+        });
+    } else {
+        run_tensor_log<T>(sig, expanded, batch, dimension, degree, s, stream, [&](uint64_t k) { return ws + (k & 1) * elems; });
+    }
     if (method) {
         launch_indexed(0, lyn.count, batch, [&](auto, dim3 grid) {
             hipLaunchKernelGGL((lyndon_compress_kernel<T>), grid, dim3(kBlock), 0, stream, (const T*)expanded, out, int64_t(batch),
