@@ -121,10 +121,12 @@ struct DeviceLyndon {
     uint64_t* index = nullptr;                           // their positions in a scalar-free row
     uint64_t *row_ptr = nullptr, *t_row_ptr = nullptr;   // strictly lower part of M^-1 and of its transpose (CSR)
     uint32_t *col = nullptr, *t_col = nullptr;
+    uint64_t* col_pos = nullptr;                         // index[col[k]]: the row position the k-th entry of M^-1 reads
     int32_t *val = nullptr, *t_val = nullptr;
     void release() noexcept
     {
-        for (void* p : {(void*)index, (void*)row_ptr, (void*)t_row_ptr, (void*)col, (void*)t_col, (void*)val, (void*)t_val})
+        for (void* p : {(void*)index, (void*)row_ptr, (void*)t_row_ptr, (void*)col, (void*)t_col, (void*)val, (void*)t_val,
+                        (void*)col_pos})
             if (p) (void)hipFree(p);
         *this = DeviceLyndon();
     }
@@ -164,6 +166,9 @@ static void prepare_lyndon(uint64_t dimension, uint64_t degree, int method)
             fresh.t_row_ptr = upload(t.t_row_ptr);
             fresh.col = upload(t.col);
             fresh.t_col = upload(t.t_col);
+            std::vector<uint64_t> pos(t.col.size());
+            for (size_t k = 0; k < pos.size(); ++k) pos[k] = t.index[t.col[k]];
+            fresh.col_pos = upload(pos);
             fresh.val = upload(t.val);
             fresh.t_val = upload(t.t_val);
         }
@@ -199,11 +204,12 @@ static DeviceLyndon find_lyndon(uint64_t dimension, uint64_t degree, int method)
     return it->second;
 }
 
-// out[b][i] = x[b][index[i]] (method 1) plus sum_k val[k] * x[b][index[col[k]]] over the row's entries (method 2)
+// out[b][i] = x[b][index[i]] (method 1) plus sum_k val[k] * x[b][col_pos[k]] over the row's entries (method 2;
+// col_pos[k] = index[col[k]], resolved when the tables are prepared)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void lyndon_compress_kernel(
     const T* __restrict__ expanded, T* __restrict__ out, int64_t batch, int64_t count, int64_t stride, int off,
-    const uint64_t* __restrict__ index, const uint64_t* __restrict__ row_ptr, const uint32_t* __restrict__ col,
+    const uint64_t* __restrict__ index, const uint64_t* __restrict__ row_ptr, const uint64_t* __restrict__ col_pos,
     const int32_t* __restrict__ val)
 {
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
@@ -211,7 +217,7 @@ __global__ __launch_bounds__(kBlock) void lyndon_compress_kernel(
         for (int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x; i < count; i += int64_t(gridDim.x) * kBlock) {
             T acc = x[index[i]];
             if (row_ptr)
-                for (uint64_t k = row_ptr[i]; k < row_ptr[i + 1]; ++k) acc = fmadd(T(val[k]), x[index[col[k]]], acc);
+                for (uint64_t k = row_ptr[i]; k < row_ptr[i + 1]; ++k) acc = fmadd(T(val[k]), x[col_pos[k]], acc);
             out[b * count + i] = acc;
         }
     }
@@ -310,7 +316,7 @@ static void sig_to_log_sig_impl(const T* sig, T* out, uint64_t batch, uint64_t d
         launch_indexed(0, lyn.count, batch, [&](auto, dim3 grid) {
             hipLaunchKernelGGL((lyndon_compress_kernel<T>), grid, dim3(kBlock), 0, stream, (const T*)expanded, out, int64_t(batch),
                                int64_t(lyn.count), int64_t(s.stride), s.off, (const uint64_t*)lyn.index,
-                               (const uint64_t*)(method == 2 ? lyn.row_ptr : nullptr), (const uint32_t*)lyn.col,
+                               (const uint64_t*)(method == 2 ? lyn.row_ptr : nullptr), (const uint64_t*)lyn.col_pos,
                                (const int32_t*)lyn.val);
         });
     }
