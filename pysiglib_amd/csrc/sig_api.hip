@@ -988,6 +988,9 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_bwd_f64_rows" : "degree2_bwd_f32_rows", !arena);
             auto go = [&](auto mode) {
                 constexpr int MODE = decltype(mode)::value;
+                if (deg2_bwd_lds_bytes<T>() > 64 * 1024)       // above the default limit of dynamic LDS
+                    SIG_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&degree2_bwd_rows_kernel<T, MODE>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, int(deg2_bwd_lds_bytes<T>())));
                 hipLaunchKernelGGL((degree2_bwd_rows_kernel<T, MODE>), dim3(unsigned(blocks)), dim3(kBlock), deg2_bwd_lds_bytes<T>(),
                                    stream, path, sig_derivs, MODE ? out : dzinc, int64_t(batch), int64_t(length), int(dimension),
                                    int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, int(parts), part_rows);
@@ -1017,6 +1020,9 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree2_bwd_f64_wide" : "degree2_bwd_f32_wide", !arena);
             auto go = [&](auto mode) {
                 constexpr int MODE = decltype(mode)::value;
+                if (deg2_bwd_lds_bytes<T>() > 64 * 1024)
+                    SIG_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&degree2_bwd_wide_kernel<T, MODE>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, int(deg2_bwd_lds_bytes<T>())));
                 hipLaunchKernelGGL((degree2_bwd_wide_kernel<T, MODE>), dim3(unsigned(blocks)), dim3(kBlock), deg2_bwd_lds_bytes<T>(),
                                    stream, path, sig_derivs, (const T*)h, MODE ? out : dzinc, int64_t(batch), int64_t(length),
                                    int(dimension), int(time_aug), int(lead_lag), time_step, int64_t(s.stride), sc, int(parts),
