@@ -437,8 +437,10 @@ static void sig_coef_backprop_impl(const T* path, T* out, const T* coefs, const 
         int copies = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(8, 4096 / dimension))) : 1;
         auto steps_for = [&](int cp) { return uint64_t(32768) / (uint64_t(cp) * dimension * sizeof(T)); };
         while (copies > 1 && steps_for(copies) < 16) copies /= 2;
-        const int chunk = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(64, steps_for(copies)))) : 1;
-        const size_t lds = use_lds ? (size_t(chunk) * size_t(copies) + size_t(chunk) + 1) * size_t(dimension) * sizeof(T) : 0;
+        int chunk = use_lds ? int(std::max<uint64_t>(1, std::min<uint64_t>(64, steps_for(copies)))) : 1;
+        auto lds_for = [&](int ch) { return (size_t(ch) * size_t(copies) + size_t(ch) + 1) * size_t(dimension) * sizeof(T); };
+        while (chunk > 1 && lds_for(chunk) > 65536) --chunk;       // sums and points together within 64 KB
+        const size_t lds = use_lds ? lds_for(chunk) : 0;
         const dim3 grid{unsigned(gx), unsigned(std::min<uint64_t>(batch, 65535)), 1};
         with_degree_bucket(h.max_degree, [&](auto kc, auto uc) {
             constexpr int KMAX = decltype(kc)::value, UF = decltype(uc)::value;

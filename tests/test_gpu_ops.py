@@ -474,7 +474,7 @@ def test_sig_coef_vs_oracle(P, oracle, aug, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
-@pytest.mark.parametrize("shape", [(2, 9, 300), (2, 6, 2800), (1, 5, 5000), (3, 200, 12)])
+@pytest.mark.parametrize("shape", [(2, 9, 300), (2, 6, 2000), (2, 6, 2800), (1, 5, 5000), (3, 200, 12)])
 def test_sig_coef_wide_and_long_paths(P, oracle, dtype, shape):
     """Paths too wide for the LDS staging of the points (forward) or of the per-channel sums (backward) take the
     kernels that read and add straight from / to memory; a long narrow path crosses several chunks of steps."""
