@@ -813,6 +813,37 @@ def test_degree_three_matrix_form(P, oracle, shape, aug, dtype, scalar_term):
     assert bwd_rel_err(sweep, want) <= TOL[dtype], shape
 
 
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_degree_two_pointers_aligned_to_the_element_only(dtype):
+    """The C ABI promises nothing beyond element alignment: the degree-2 kernels that copy rows in 16-byte pieces must
+    fall back to element-wise copies for such pointers and return the same bits."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    tdt = torch.float64 if dtype == "float64" else torch.float32
+    real = L.DTYPES[dtype]
+    b, length, d = 9, 70, 64
+    n = d + d * d
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    x = (torch.randn((b, length, d), dtype=tdt, generator=gen).cumsum(1) * 0.05).to(DEV)
+    g = torch.randn((b, n), dtype=tdt, generator=gen).to(DEV)
+    esz = x.element_size()
+    res = []
+    for shift in (0, 1):
+        xs = torch.zeros(x.numel() + 4, dtype=tdt, device=DEV)
+        xs[shift:shift + x.numel()] = x.flatten()
+        gs = torch.zeros(g.numel() + 4, dtype=tdt, device=DEV)
+        gs[shift:shift + g.numel()] = g.flatten()
+        sig = torch.zeros(b * n + 4, dtype=tdt, device=DEV)
+        gx = torch.zeros(x.numel() + 4, dtype=tdt, device=DEV)
+        ptr = lambda t: ctypes.cast(t.data_ptr() + shift * esz, ctypes.POINTER(real))
+        assert L.CUSIG_SIGNATURE[dtype](ptr(xs), ptr(sig), b, d, length, 2, False, False, 1.0, True, False, None, 0, 0, 0) == 0
+        assert L.CUSIG_SIG_BACKPROP[dtype](ptr(xs), ptr(gx), ptr(gs), ptr(sig), b, d, length, 2, False, False, 1.0, False,
+                                           None, 0, 0, 0) == 0
+        res.append((sig[shift:shift + b * n].clone(), gx[shift:shift + x.numel()].clone()))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    assert float(res[0][0].abs().max()) > 0 and float(res[0][1].abs().max()) > 0
+
+
 @pytest.mark.parametrize("shape,aug", [
     ((3, 9, 2, 2), {}), ((2, 30, 5, 2), {}), ((4, 17, 16, 2), {}), ((2, 21, 17, 2), dict(time_aug=True)),
     ((2, 13, 31, 2), dict(lead_lag=True)), ((3, 12, 33, 2), dict(time_aug=True, lead_lag=True)), ((1, 2, 70, 2), {}),
