@@ -407,12 +407,12 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
             }
         }
         if (use_lds) {
+            // the private sets fold into the first one with the whole block at work (d lanes walking them one read at
+            // a time would take longer than the block's items), then one atomic per letter
             __syncthreads();
-            for (I j = threadIdx.x; j < d; j += kBlock) {
-                T sum = T(0);
-                for (int c = 0; c < copies; ++c) sum += acc[I(c) * d + j];
-                dev_add(&out[j], sum);
-            }
+            for (I e = d + threadIdx.x; e < I(copies) * d; e += kBlock) lds_add_shared(&acc[e % d], acc[e]);
+            __syncthreads();
+            for (I j = threadIdx.x; j < d; j += kBlock) dev_add(&out[j], acc[j]);
         }
     }
 }
