@@ -340,12 +340,17 @@ __global__ __launch_bounds__(kBlock) void exp_pullback_kernel(
     // `copies` private sets of d accumulators, chosen by lane: few letters mean many lanes adding to one word
     T* mine = acc + (threadIdx.x % copies) * d;
     for (int64_t b = xcd_block_2d().y; b < batch; b += gridDim.y) {
+        const T* z = disp + b * int64_t(d);
         if (use_lds) {
+            // the accumulators and, behind them, the row's d letter values (picked per lane: from memory every such
+            // load would occupy the texture addresser for a whole wave)
+            T* zl = acc + I(copies) * d;
             __syncthreads();
             for (I j = threadIdx.x; j < I(copies) * d; j += kBlock) acc[j] = T(0);
+            for (I j = threadIdx.x; j < d; j += kBlock) zl[j] = z[j];
             __syncthreads();
+            z = zl;
         }
-        const T* z = disp + b * int64_t(d);
         const T* g = dE + b * stride + off;
         T* out = dz + b * int64_t(d);
         auto add = [&](I letter, T v) {
@@ -605,7 +610,7 @@ static void sig_join_backprop_impl(const T* d_out, T* d_sig, T* d_disp, const T*
                 auto go = [&](auto tmax) {
                     constexpr int TMAX = decltype(tmax)::value;
                     hipLaunchKernelGGL((exp_pullback_kernel<T, I, FAN, TMAX>), grid, dim3(kBlock),
-                                       use_lds ? size_t(copies) * size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp,
+                                       use_lds ? (size_t(copies) + 1) * size_t(dimension) * sizeof(T) : 0, stream, (const T*)dE, disp,
                                        d_disp, int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, use_lds,
                                        copies);
                 };
