@@ -220,7 +220,7 @@ static bool launch_linear_sig_levels(const T* disp, T* out, uint64_t batch, uint
 template <typename T, typename I, int FAN>
 __global__ __launch_bounds__(kBlock) void sig_join_kernel(
     const T* __restrict__ A, const T* __restrict__ disp, T* __restrict__ out, int64_t batch, DivBy<I> dv, I items,
-    int64_t stride, int off, int prepend, I low_n)
+    int64_t stride, int off, int prepend, I low_n, int z_lds)
 {
     extern __shared__ double join_low_raw[];
     T* al = reinterpret_cast<T*>(join_low_raw);
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(kBlock) void sig_join_kernel(
     for (int64_t b = blockIdx.y; b < batch; b += gridDim.y) {
         const T* a = A + b * stride + off;
         const T* z = disp + b * int64_t(d);
-        if (low_n) {
+        if (low_n || z_lds) {       // z_lds: the letters' values alone (both forms pick them per lane)
             __syncthreads();        // the row before is done with the copies
             for (I j = threadIdx.x; j < low_n; j += kBlock) al[j] = a[j];
             for (I j = threadIdx.x; j < d; j += kBlock) zl[j] = z[j];
@@ -544,9 +544,10 @@ static void sig_join_impl(const T* sig, const T* disp, T* out, uint64_t batch, u
             const uint64_t per_thread = low_n ? chen_low_items_per_thread(low_n, blocks) : 1;
             launch_indexed(s.n_coef, (items + per_thread - 1) / per_thread, batch, [&](auto ix, dim3 grid) {
                 using I = decltype(ix);
-                hipLaunchKernelGGL((sig_join_kernel<T, I, FAN>), grid, dim3(kBlock), low_n ? (low_n + dimension) * sizeof(T) : 0,
-                                   stream, sig, disp, out, int64_t(batch), DivBy<I>(dimension), I(items), int64_t(s.stride), s.off,
-                                   int(prepend), I(low_n));
+                const int z_lds = dimension * sizeof(T) <= 32768;
+                hipLaunchKernelGGL((sig_join_kernel<T, I, FAN>), grid, dim3(kBlock),
+                                   (low_n || z_lds) ? (low_n + dimension) * sizeof(T) : 0, stream, sig, disp, out, int64_t(batch),
+                                   DivBy<I>(dimension), I(items), int64_t(s.stride), s.off, int(prepend), I(low_n), z_lds);
             });
         });
     }
