@@ -18,12 +18,20 @@ import os
 
 MAX_GENERIC_N = 16
 GENERIC_K = 4
-# Paths of many channels (beyond the specialised dimensions) at low degree: run-time-dimension kernels with more
-# letters per lane, (D, K) per direction; D = -1 is the wide layout.  Measured on MI355X for d = 18 .. 100:
-# forward: wide K 8 is fastest wherever it applies (degree >= 3; degree 2 of that many channels runs in closed
-# form); backward: packed K 16.
-MANY_CHANNELS_MAX_N = 5
-MANY_CHANNELS = {"fwd": ((-1, 8),), "bwd": ((0, 16),)}
+# Shapes beyond the specialised table: run-time-dimension kernels with more letters per lane (the chain work of a lane
+# is shared by more top-level updates), (D, K) per direction and degree range; D = -1 is the wide layout (one letter
+# group of one path per wave, the group's increments arriving through scalar loads), D = 0 the packed one.  Measured on
+# MI355X (d = 41 .. 80 at degree 4, 21 .. 32 at degree 5, 9 .. 16 at degree 6, 6 .. 8 at degree 7, 5 .. 6 at degree 8,
+# 4 at degree 9 and 10): the wide layout wins wherever it applies except in the backward of 4 channels; forward K 8 up
+# to 8 channels, K 32 where 32 divides the channel count (single precision), else K 16; backward K 8 up to 8 channels, 16 up to 32, 32
+# beyond; the packed K 16 backward is kept for single precision at 9 .. 15 channels.
+MANY_CHANNELS_MAX_N = 10
+def many_channels(direction, N):
+    if N <= 5:
+        return ((-1, 16), (-1, 32)) if direction == "fwd" else ((0, 16), (-1, 16), (-1, 32))
+    if N <= 8:
+        return ((-1, 8), (-1, 16)) if direction == "fwd" else ((0, 16), (-1, 8), (-1, 16))
+    return ((-1, 8),) if direction == "fwd" else ()
 
 # value budgets (signature values held per lane); backward holds state + adjoint
 BUDGET = {("f64", "fwd"): 100, ("f64", "bwd"): 60, ("f32", "fwd"): 170, ("f32", "bwd"): 100}
@@ -195,7 +203,7 @@ def main():
             for direction in ("fwd", "bwd"):
                 insts.append((T, 0, N, 1, GENERIC_K, direction, 1, 0))
                 if N <= MANY_CHANNELS_MAX_N:
-                    for (dd, kk) in MANY_CHANNELS[direction]:
+                    for (dd, kk) in many_channels(direction, N):
                         insts.append((T, dd, N, 1, kk, direction, 0, 0))
 
     # balance files by a rough compile-cost estimate

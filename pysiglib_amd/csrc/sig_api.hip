@@ -90,24 +90,36 @@ static const KernelEntry* choose_entry(bool backward, bool f64, uint64_t d, uint
 }
 
 // Shapes without a specialised instance run a run-time-dimension kernel.  Its default carries few depth-1 letters
-// per lane, which suits small dimensions and high degrees.  Paths of many channels at low degree have variants
-// with more letters per lane (the chain work of a lane is shared by more top-level updates): for the backward a
-// packed 16-letter variant, for the forward a wide-layout 8-letter variant (one letter group of one path per wave,
-// the group's increments arriving through scalar loads) for paths with at least 48 word prefixes.  Measured for
-// d = 18 .. 100: forward 2-3x, backward 1.6-2x faster than the default.
+// per lane in the packed layout, which suits the few lanes of small shapes.  Up to degree 10 there are variants with
+// more letters per lane (the chain work of a lane is shared by more top-level updates), most of them in the wide
+// layout (one letter group of one path per wave, the group's increments arriving through scalar loads), which needs
+// at least 48 word prefixes.  Measured for d = 41 .. 80 at degree 4, 21 .. 32 at degree 5, 9 .. 16 at degree 6,
+// 6 .. 8 at degree 7 and 5 .. 6 at degree 8: 2-16x faster forward, 1.5-5x backward than the default.
 static const KernelEntry* pick_run_time_entry(bool backward, bool f64, int d, int degree)
 {
     const auto& m = backward ? table().bwd : table().fwd;
     auto packed = m.find(std::make_tuple(int(f64), 0, degree));
     if (packed == m.end() || packed->second.empty()) return nullptr;
     const KernelEntry* best = packed->second.front();
-    if (d < 12) return best;
+    const KernelEntry* packed_many = nullptr;
     for (const KernelEntry* e : packed->second)
-        if (e->k > best->k && !e->staged) best = e;       // the many-letter variant, if this degree has one
-    if (backward) return best;
+        if (e->k > best->k && !e->staged && (!packed_many || e->k > packed_many->k)) packed_many = e;
     auto wide = m.find(std::make_tuple(int(f64), -1, degree));
-    if (wide != m.end() && !wide->second.empty() && ipow64(d, degree - 1) >= 48) best = wide->second.front();
-    return best;
+    if (wide == m.end() || wide->second.empty() || ipow64(d, degree - 1) < 48)
+        return d >= 12 && packed_many ? packed_many : best;
+    // single precision backward at 9 .. 15 channels: the packed 16-letter variant is ~10 % ahead of the wide one,
+    // whose only letter group is then partly empty
+    if (backward && !f64 && d > 8 && d < 16 && packed_many) return packed_many;
+    // letters per lane: a partly empty last group costs more than the longer chain share of a smaller K
+    // (forward, 32 letters: single precision only -- a double-precision row of 32 does not fit the scalar registers twice)
+    const int want = d <= 8 ? 8 : backward ? (d <= 32 ? 16 : 32) : (d % 32 == 0 && !f64 ? 32 : 16);
+    const KernelEntry* pick = nullptr;
+    for (const KernelEntry* e : wide->second) {
+        if (e->staged) continue;
+        // the largest letter count up to `want`, else the smallest there is
+        if (!pick || (e->k <= want ? (pick->k > want || e->k > pick->k) : (pick->k > want && e->k < pick->k))) pick = e;
+    }
+    return pick ? pick : best;
 }
 
 static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64_t degree)

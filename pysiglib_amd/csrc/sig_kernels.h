@@ -29,6 +29,8 @@ struct LaneCtx {
     using Tr = Tree<T, D, N, TAIL, K>;
     static constexpr int M = Tr::M;
     static constexpr bool WIDE = D > 0 ? ipow64(D > 0 ? D : 1, M) >= 48 : D < 0;
+    static constexpr bool kWholeGroups = D > 0 && D % K == 0;     // no letter group reaches past the row
+    static constexpr bool kRunTimeWide = D < 0;
     int d;
     TreeGeom G;
     LaneId id;
@@ -56,20 +58,39 @@ struct LaneCtx {
             p[l] = int(q % d);
             q /= d;
         }
-        a0 = id.g * K;
+        a0 = kRunTimeWide ? __builtin_amdgcn_readfirstlane(id.g * K) : id.g * K;      // wave-uniform: say so
     }
 
+    // GUARD: every read of the group is bounds-tested instead (no read past the row, no merged loads)
+    template <bool GUARD = false>
     __device__ __forceinline__ void load_inc(typename Tr::Inc& in, const T* __restrict__ row) const
     {
         if constexpr (TAIL >= 2) {
 #pragma unroll
             for (int j = 0; j < Tr::DD; ++j) in.z[j] = row[j];
         }
+        // Run-time dimension, wide layout: the group is wave-uniform and its K reads merge into a few wide scalar loads,
+        // provided none of them is guarded.  The last group of a row then reads on into the next row (the increment
+        // buffer continues for more than K elements past its last row) and mask_inc drops what lies beyond the row.
+        if constexpr (kWholeGroups || (D < 0 && !GUARD)) {
 #pragma unroll
-        for (int a = 0; a < K; ++a) in.zs[a] = (a0 + a < d) ? row[a0 + a] : T(0);
+            for (int a = 0; a < K; ++a) in.zs[a] = row[a0 + a];
+        } else {
+#pragma unroll
+            for (int a = 0; a < K; ++a) in.zs[a] = (a0 + a < d) ? row[a0 + a] : T(0);
+        }
 #pragma unroll
         for (int l = 0; l < M; ++l) in.pz[l] = row[p[l]];
     }
+
+    // Zeroes the letters that load_inc read past the end of the row; needed by the waves of a row's last group when the
+    // dimension is not a multiple of K (partial_group()).
+    __device__ __forceinline__ void mask_inc(typename Tr::Inc& in) const
+    {
+#pragma unroll
+        for (int a = 0; a < K; ++a) in.zs[a] = (a0 + a < d) ? in.zs[a] : T(0);
+    }
+    __device__ __forceinline__ bool partial_group() const { return D < 0 && a0 + K > d; }      // wave-uniform
 
     // offset of level `lev` (1-based) inside a signature row
     __device__ __forceinline__ int64_t level_off(int lev, int scalar) const
@@ -230,26 +251,51 @@ __device__ __forceinline__ const T* opaque_lds(const T* p)
 // scalar path.  WAIT_ALL: end every step with a full wait for outstanding loads (cheapest schedule when the
 // step issues no stores); the backward must not do that, because a full wait would also wait for the
 // acknowledgement of the global atomics it fires, so there the compiler's per-register waits are used.
-template <int DIR, bool WAIT_ALL, typename Cx, typename Inc, typename T, typename StepFn>
-__device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
-                                             StepFn&& step)
+template <int DIR, bool WAIT_ALL, bool MASK, typename Cx, typename Inc, typename T, typename StepFn>
+__device__ __forceinline__ void sweep_direct_rows(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
+                                                  StepFn&& step)
 {
+    // MASK: the wave's letter group reaches past the row.  The forward reads it whole and zeroes the excess when the
+    // row is used; the backward, short of registers, keeps bounds-tested reads there.
+    constexpr bool GUARD = MASK && !WAIT_ALL;
+    constexpr bool ZERO = MASK && !GUARD;
+    // Scalar loads return out of order, so the only wait there is for them is "all landed".  The row a step uses was
+    // requested a whole step ago: waiting for it before the next row is requested costs nothing, while any later first
+    // use would also wait for the row just requested.  (The forward's full wait at the end of a step does the same.)
+    constexpr bool ROW_WAIT = Cx::kRunTimeWide && !GUARD && !WAIT_ALL;
     const int d = cx.d;
     Inc za, zb;
-    cx.load_inc(za, row);
+    cx.template load_inc<GUARD>(za, row);
+    if constexpr (Cx::kRunTimeWide && WAIT_ALL) wait_all_loads();
     int64_t i = 0;
     for (; i + 2 <= count; i += 2) {
-        cx.load_inc(zb, row + DIR * d);
+        if constexpr (ROW_WAIT) wait_lds();
+        cx.template load_inc<GUARD>(zb, row + DIR * d);
         loads_issued();
+        if constexpr (ZERO) cx.mask_inc(za);
         step(za, first + DIR * i, IntC<-1>{}, IntC<0>{});
         if constexpr (WAIT_ALL) wait_all_loads();
-        cx.load_inc(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
+        if constexpr (ROW_WAIT) wait_lds();
+        cx.template load_inc<GUARD>(za, row + 2 * DIR * d);        // at most one row past the path: a zero guard row
         loads_issued();
+        if constexpr (ZERO) cx.mask_inc(zb);
         step(zb, first + DIR * (i + 1), IntC<-1>{}, IntC<1>{});
         if constexpr (WAIT_ALL) wait_all_loads();
         row += 2 * DIR * d;
     }
-    if (i < count) step(za, first + DIR * i, IntC<-1>{}, IntC<0>{});
+    if (i < count) {
+        if constexpr (ZERO) cx.mask_inc(za);
+        step(za, first + DIR * i, IntC<-1>{}, IntC<0>{});
+    }
+}
+
+// run-time-dimension wide kernels hold the loop twice, and each wave takes the one its letter group needs
+template <int DIR, bool WAIT_ALL, typename Cx, typename Inc, typename T, typename StepFn>
+__device__ __forceinline__ void sweep_direct(const Cx& cx, const T* __restrict__ row, int64_t first, int64_t count,
+                                             StepFn&& step)
+{
+    if (Cx::kRunTimeWide && cx.partial_group()) sweep_direct_rows<DIR, WAIT_ALL, true, Cx, Inc>(cx, row, first, count, step);
+    else sweep_direct_rows<DIR, WAIT_ALL, false, Cx, Inc>(cx, row, first, count, step);
 }
 
 // staged path; G0 >= 0: the depth-1 letters start at the compile-time letter G0

@@ -738,7 +738,9 @@ def test_run_time_degree_sweeps(P, oracle, shape, dtype):
     (3, 9, 13, 4), (2, 12, 20, 3), (5, 7, 30, 2), (2, 6, 32, 3), (3, 8, 50, 2), (4, 9, 40, 2), (2, 5, 18, 5), (2, 6, 100, 2),
     (70, 5, 12, 2), (2, 7, 27, 3), (2, 6, 33, 3), (1, 30, 64, 2),
     (2, 6, 70, 3), (1, 5, 34, 4), (2, 5, 17, 5), (3, 40, 65, 3),
-    (2, 6, 130, 3), (2, 7, 97, 3), (1, 5, 41, 4), (2, 5, 21, 5), (1, 4, 200, 3)])        # beyond the specialised table: run-time dimension
+    (2, 6, 130, 3), (2, 7, 97, 3), (1, 5, 41, 4), (2, 5, 21, 5), (1, 4, 200, 3),        # beyond the specialised table: run-time dimension
+    (1, 4, 48, 4), (1, 3, 24, 5), (2, 5, 9, 6), (2, 6, 10, 6), (1, 4, 12, 6), (1, 4, 6, 7), (1, 4, 7, 7), (1, 4, 8, 7),
+    (1, 4, 5, 8), (1, 3, 6, 8), (1, 3, 4, 9), (1, 3, 4, 10)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_many_channel_shapes(P, oracle, shape, dtype):
     """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
@@ -771,6 +773,55 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
     refa = oracle.signature(xa, min(deg, 3), n_jobs=-1, **aug)
     da = (2 * xa.shape[2] if aug["lead_lag"] else xa.shape[2]) + 1
     assert level_rel_err(P.sig(dev(xa), min(deg, 3), **aug).cpu().numpy(), refa, da, min(deg, 3)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("shape", [(2, 6, 41, 4), (1, 5, 48, 4), (2, 5, 21, 5), (2, 6, 9, 6), (1, 5, 12, 6), (1, 5, 7, 7),
+                                   (1, 4, 8, 7), (2, 5, 5, 8), (1, 4, 4, 9), (1, 4, 4, 10)])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_every_run_time_dimension_variant(P, oracle, shape, dtype):
+    """The run-time-dimension kernels exist with 4 letters per lane in the packed layout for every degree and, up to
+    degree 10 (backward: 8), with 8, 16 or 32 letters per lane in the packed or the wide layout; the choice among them follows the
+    channel count.  Here every compiled variant of a degree is forced onto one shape (letter groups that fill the row
+    exactly, reach past it, or hold it in one partly empty group) and checked against the oracle in both directions."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    C = L.CUSIG
+    C.cusig_amd_force_partition.argtypes = (ctypes.c_int, ctypes.c_int)
+    C.cusig_amd_force_partition.restype = None
+    C.cusig_amd_force_run_time_wide.argtypes = (ctypes.c_int,)
+    C.cusig_amd_force_run_time_wide.restype = None
+    b, length, d, deg = shape
+    if deg <= 5:
+        variants = {False: [(0, 4), (1, 16), (1, 32)], True: [(0, 4), (0, 16), (1, 16), (1, 32)]}
+    elif deg <= 8:
+        variants = {False: [(0, 4), (1, 8), (1, 16)], True: [(0, 4), (0, 16), (1, 8), (1, 16)]}
+    else:
+        variants = {False: [(0, 4), (1, 8)], True: [(0, 4)]}
+    rng = np.random.default_rng(d * 100 + deg)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * 0.3).astype(dtype)
+    ref = oracle.signature(x, deg, n_jobs=-1)
+    g = rng.standard_normal(ref.shape).astype(dtype)
+    want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
+    try:
+        C.cusig_amd_set_profiling(1)
+        for backward in (False, True):
+            for (wide, k) in variants[backward]:
+                C.cusig_amd_force_run_time_wide(wide)
+                C.cusig_amd_force_partition(1, k)
+                if backward:
+                    got = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
+                else:
+                    got = P.sig(dev(x), deg).cpu().numpy()
+                name = C.cusig_amd_last_kernel_name().decode()
+                assert ("_d0w_" if wide else "_d0_") in name and name.endswith("_t1_k%d" % k), (name, wide, k)
+                if backward:
+                    assert bwd_rel_err(got, want) <= TOL[dtype], (shape, name)
+                else:
+                    assert level_rel_err(got, ref, d, deg) <= TOL[dtype], (shape, name)
+    finally:
+        C.cusig_amd_force_partition(0, 0)
+        C.cusig_amd_force_run_time_wide(0)
+        C.cusig_amd_set_profiling(0)
 
 
 @pytest.mark.parametrize("shape,aug", [
