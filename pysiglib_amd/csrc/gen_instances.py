@@ -83,8 +83,9 @@ if os.environ.get("SIGAMD_EXTRA_PARTITIONS"):
 
 def spec_shapes():
     """(D, N) pairs that get specialised kernels."""
-    caps = {2: 12, 3: 12, 4: 8, 5: 7, 6: 6, 7: 6, 8: 6}
+    caps = {2: 12, 3: 12, 4: 10, 5: 8, 6: 7, 7: 7, 8: 7}
     caps.update({d: 5 for d in range(9, 21)})
+    caps.update({d: 6 for d in range(9, 13)})
     caps.update({d: 4 for d in range(21, 41)})
     caps.update({d: 3 for d in range(41, 129)})
     out = []
