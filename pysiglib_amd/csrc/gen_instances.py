@@ -83,7 +83,7 @@ if os.environ.get("SIGAMD_EXTRA_PARTITIONS"):
 
 def spec_shapes():
     """(D, N) pairs that get specialised kernels."""
-    caps = {2: 12, 3: 12, 4: 10, 5: 8, 6: 7, 7: 7, 8: 7}
+    caps = {2: 16, 3: 14, 4: 10, 5: 9, 6: 8, 7: 7, 8: 7}
     caps.update({d: 5 for d in range(9, 21)})
     caps.update({d: 6 for d in range(9, 13)})
     caps.update({d: 4 for d in range(21, 41)})
