@@ -11,7 +11,7 @@ a register budget, and writes
 D = 0 denotes the run-time-dimension kernel (TAIL = 1), instantiated for every
 degree 2..MAX_GENERIC_N; it serves every shape that has no specialised entry.
 
-Usage: python gen_instances.py [--out gen] [--files 8]
+Usage: python gen_instances.py [--out gen] [--files 24]
 """
 import argparse
 import os
