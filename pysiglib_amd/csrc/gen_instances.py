@@ -179,7 +179,7 @@ def choose(D, N, dtype, direction):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "gen"))
-    ap.add_argument("--files", type=int, default=8)
+    ap.add_argument("--files", type=int, default=24)
     ap.add_argument("--quick", action="store_true", help="small table (fast builds while developing)")
     args = ap.parse_args()
     os.makedirs(args.out, exist_ok=True)
