@@ -332,31 +332,33 @@ def main():
                             "roofline_frac": mm_flops / (kms * 1e-3) / 1e12 / PEAK_TFLOPS["float32"]}
         del xp, sg, gg, gx
         torch.cuda.empty_cache()
-        # degree 3 on paths of many channels: the backward as two library matrix products around a scan (not one of the
-        # five benchmark workloads); flops are the sweep's operation count, as for the other workloads
-        tb, tl, td = 512, 256, 80
-        xp = (torch.randn((tb, tl, td), dtype=torch.float32, device="cuda:0").cumsum(1) * 0.03).contiguous()
-        sg = torch.empty((tb, td + td * td + td ** 3), dtype=torch.float32, device="cuda:0")
-        gg = torch.randn_like(sg)
-        gx = torch.empty_like(xp)
+        # further f32 legs, none of them one of the five benchmark workloads: degree 3 on paths of many channels (the
+        # backward as two library matrix products around a scan), a shape the instance table reaches at degree 6, and
+        # one beyond the table (run-time-dimension kernels); flops are the sweep's operation count, as for the workloads
+        for prefix, tb, tl, td, tdeg in (("D3", 512, 256, 80, 3), ("T6", 64, 200, 10, 6), ("R4", 32, 200, 48, 4)):
+            xp = (torch.randn((tb, tl, td), dtype=torch.float32, device="cuda:0").cumsum(1) * (0.5 / tl ** 0.5)).contiguous()
+            sg = torch.empty((tb, int(loader.CUSIG.cusig_amd_sig_length(td, tdeg)) - 1), dtype=torch.float32, device="cuda:0")
+            gg = torch.randn_like(sg)
+            gx = torch.empty_like(xp)
 
-        def d3_fwd():
-            loader.CUSIG_SIGNATURE["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), tb, td, tl, 3,
-                                              False, False, 1.0, True, False, None, 0, 0, 0)
+            def leg_fwd():
+                loader.CUSIG_SIGNATURE["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), tb, td, tl,
+                                                  tdeg, False, False, 1.0, True, False, None, 0, 0, 0)
 
-        def d3_bwd():
-            loader.CUSIG_SIG_BACKPROP["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(gx.data_ptr(), fp),
-                                                 ctypes.cast(gg.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), tb, td, tl,
-                                                 3, False, False, 1.0, False, None, 0, 0, 0)
+            def leg_bwd():
+                loader.CUSIG_SIG_BACKPROP["float32"](ctypes.cast(xp.data_ptr(), fp), ctypes.cast(gx.data_ptr(), fp),
+                                                     ctypes.cast(gg.data_ptr(), fp), ctypes.cast(sg.data_ptr(), fp), tb, td, tl,
+                                                     tdeg, False, False, 1.0, False, None, 0, 0, 0)
 
-        for tag, fn, fl in (("D3 fwd f32 (512,256,80) deg 3", d3_fwd, cfgmod.flops_fwd(td, 3)),
-                            ("D3 bwd f32 (512,256,80) deg 3", d3_bwd, cfgmod.flops_bwd(td, 3))):
-            wall, kms, name = time_calls(fn, torch, loader, 2, 5)
-            tf = tb * (tl - 1) * fl / (kms * 1e-3) / 1e12
-            configs[tag] = {"signatures_per_s": tb / wall, "call_ms": wall * 1e3, "kernel": name, "kernel_ms": kms, "tflops": tf,
-                            "roofline_frac": tf / PEAK_TFLOPS["float32"]}
-        del xp, sg, gg, gx
-        torch.cuda.empty_cache()
+            shape = "f32 (%d,%d,%d) deg %d" % (tb, tl, td, tdeg)
+            for tag, fn, fl in (("%s fwd %s" % (prefix, shape), leg_fwd, cfgmod.flops_fwd(td, tdeg)),
+                                ("%s bwd %s" % (prefix, shape), leg_bwd, cfgmod.flops_bwd(td, tdeg))):
+                wall, kms, name = time_calls(fn, torch, loader, 2, 5)
+                tf = tb * (tl - 1) * fl / (kms * 1e-3) / 1e12
+                configs[tag] = {"signatures_per_s": tb / wall, "call_ms": wall * 1e3, "kernel": name, "kernel_ms": kms,
+                                "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS["float32"]}
+            del xp, sg, gg, gx
+            torch.cuda.empty_cache()
 
     def step():
         r1.forward()
