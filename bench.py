@@ -335,7 +335,7 @@ def main():
         # further f32 legs, none of them one of the five benchmark workloads: degree 3 on paths of many channels (the
         # backward as two library matrix products around a scan), a shape the instance table reaches at degree 6, and
         # one beyond the table (run-time-dimension kernels); flops are the sweep's operation count, as for the workloads
-        for prefix, tb, tl, td, tdeg in (("D3", 512, 256, 80, 3), ("T6", 64, 200, 10, 6), ("R4", 32, 200, 48, 4)):
+        for prefix, tb, tl, td, tdeg in (("D3", 512, 256, 80, 3), ("T6", 64, 200, 10, 6), ("R4", 16, 200, 64, 4)):
             xp = (torch.randn((tb, tl, td), dtype=torch.float32, device="cuda:0").cumsum(1) * (0.5 / tl ** 0.5)).contiguous()
             sg = torch.empty((tb, int(loader.CUSIG.cusig_amd_sig_length(td, tdeg)) - 1), dtype=torch.float32, device="cuda:0")
             gg = torch.randn_like(sg)

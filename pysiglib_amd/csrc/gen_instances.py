@@ -21,7 +21,7 @@ GENERIC_K = 4
 # Shapes beyond the specialised table: run-time-dimension kernels with more letters per lane (the chain work of a lane
 # is shared by more top-level updates), (D, K) per direction and degree range; D = -1 is the wide layout (one letter
 # group of one path per wave, the group's increments arriving through scalar loads), D = 0 the packed one.  Measured on
-# MI355X (d = 41 .. 80 at degree 4, 21 .. 32 at degree 5, 9 .. 16 at degree 6, 6 .. 8 at degree 7, 5 .. 6 at degree 8,
+# MI355X before the table grew (d = 41 .. 80 at degree 4, 21 .. 32 at degree 5, 9 .. 16 at degree 6, 6 .. 8 at degree 7, 5 .. 6 at degree 8,
 # 4 at degree 9 and 10): the wide layout wins wherever it applies except in the backward of 4 channels; forward K 8 up
 # to 8 channels, K 32 where 32 divides the channel count (single precision), else K 16; backward K 8 up to 8 channels, 16 up to 32, 32
 # beyond; the packed K 16 backward is kept for single precision at 9 .. 15 channels.
@@ -86,8 +86,9 @@ def spec_shapes():
     caps = {2: 16, 3: 14, 4: 10, 5: 9, 6: 8, 7: 7, 8: 7}
     caps.update({d: 5 for d in range(9, 21)})
     caps.update({d: 6 for d in range(9, 13)})
-    caps.update({d: 4 for d in range(21, 41)})
-    caps.update({d: 3 for d in range(41, 129)})
+    caps.update({d: 4 for d in range(21, 49)})
+    caps.update({d: 5 for d in range(21, 25)})
+    caps.update({d: 3 for d in range(49, 129)})
     out = []
     for d, nmax in sorted(caps.items()):
         for n in range(2, nmax + 1):
@@ -152,7 +153,7 @@ def choose(D, N, dtype, direction):
             return (2, 2) if D <= 100 else (2, 1)
     if N == 4 and D > 32:
         if direction == "fwd":
-            return (1, D) if dtype == "f32" else (1, D // 2)
+            return (1, D) if dtype == "f32" else (1, D // 2 if D <= 40 else (D + 1) // 2)     # beyond 40: two groups also for odd D
         return (2, 3)
     if dtype == "f64" and direction == "fwd" and D >= 24 and N == 3:
         # measured on MI355X (d = 24, 32, 48 at degree 3): the f64 forward runs 1.1-1.8x faster with one subtree level

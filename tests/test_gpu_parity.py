@@ -740,7 +740,7 @@ def test_run_time_degree_sweeps(P, oracle, shape, dtype):
     (2, 6, 70, 3), (1, 5, 34, 4), (2, 5, 17, 5), (3, 40, 65, 3),
     (2, 6, 130, 3), (2, 7, 97, 3), (1, 5, 41, 4), (2, 5, 21, 5), (1, 4, 200, 3),        # beyond the specialised table: run-time dimension
     (1, 4, 48, 4), (1, 3, 24, 5), (2, 5, 9, 6), (2, 6, 10, 6), (1, 4, 12, 6), (1, 4, 6, 7), (1, 4, 7, 7), (1, 4, 8, 7),
-    (1, 4, 5, 8), (1, 3, 6, 8), (1, 3, 4, 9), (1, 3, 4, 10), (1, 4, 13, 6), (1, 3, 9, 7), (1, 3, 5, 9), (1, 3, 7, 8)])
+    (1, 4, 5, 8), (1, 3, 6, 8), (1, 3, 4, 9), (1, 3, 4, 10), (1, 4, 13, 6), (1, 3, 9, 7), (1, 3, 5, 9), (1, 3, 7, 8), (1, 4, 49, 4), (1, 3, 25, 5)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_many_channel_shapes(P, oracle, shape, dtype):
     """Dimensions beyond the specialised instances run the run-time-dimension kernels, which come in several
@@ -775,7 +775,7 @@ def test_many_channel_shapes(P, oracle, shape, dtype):
     assert level_rel_err(P.sig(dev(xa), min(deg, 3), **aug).cpu().numpy(), refa, da, min(deg, 3)) <= TOL[dtype]
 
 
-@pytest.mark.parametrize("shape", [(2, 6, 41, 4), (1, 5, 48, 4), (2, 5, 21, 5), (1, 5, 13, 6), (1, 4, 9, 7), (1, 3, 7, 8),
+@pytest.mark.parametrize("shape", [(1, 5, 49, 4), (1, 4, 52, 4), (1, 4, 25, 5), (1, 5, 13, 6), (1, 4, 9, 7), (1, 3, 7, 8),
                                    (1, 3, 6, 9), (1, 3, 5, 10)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_every_run_time_dimension_variant(P, oracle, shape, dtype):
@@ -947,7 +947,7 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_every_specialised_dimension_above_12(P, oracle, dtype):
     """One small forward + backward per compiled (dimension, degree) instance that the grid above does not reach:
-    dimensions 13..64 at degree 3, 13..32 at degree 4, 9..16 at degree 5, 7..12 at degree 6, 6..8 at degree 7, 5..6 at
+    dimensions 13..64 at degree 3, 13..32 and 41..48 at degree 4, 9..16 and 21..24 at degree 5, 7..12 at degree 6, 6..8 at degree 7, 5..6 at
     degree 8, 4..5 at degree 9, 4 at degree 10, 2 at degrees 13..16, 3 at degrees 13 and 14."""
     import ctypes
     from pysiglib_amd import _loader as L
@@ -955,7 +955,8 @@ def test_every_specialised_dimension_above_12(P, oracle, dtype):
     C.cusig_amd_force_partition.argtypes = (ctypes.c_int, ctypes.c_int)
     C.cusig_amd_force_partition.restype = None
     rng = np.random.default_rng(5)
-    shapes = ([(d, 3) for d in range(13, 65)] + [(d, 4) for d in range(13, 33)] + [(d, 5) for d in range(9, 17)] +
+    shapes = ([(d, 3) for d in range(13, 65)] + [(d, 4) for d in range(13, 33)] + [(d, 4) for d in range(41, 49)] +
+              [(d, 5) for d in range(9, 17)] + [(d, 5) for d in range(21, 25)] +
               [(7, 6), (8, 6), (9, 6), (10, 6), (11, 6), (12, 6), (6, 7), (7, 7), (8, 7), (5, 8), (6, 8), (4, 9), (5, 9), (4, 10),
                (2, 13), (2, 14), (2, 15), (2, 16), (3, 13), (3, 14)])
     tail, k, spec = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
