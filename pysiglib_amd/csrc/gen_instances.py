@@ -154,7 +154,9 @@ def choose(D, N, dtype, direction):
     if N == 4 and D > 32:
         if direction == "fwd":
             return (1, D) if dtype == "f32" else (1, D // 2 if D <= 40 else (D + 1) // 2)     # beyond 40: two groups also for odd D
-        return (2, 3)
+        # f64 beyond 40 channels: three letters per lane no longer fit the registers (d = 48: 65.8 ms, two letters 19.5;
+        # d = 44: 23.7 / 14.8; d = 41: 13.0 / 13.2)
+        return (2, 2) if dtype == "f64" and D > 40 else (2, 3)
     if dtype == "f64" and direction == "fwd" and D >= 24 and N == 3:
         # measured on MI355X (d = 24, 32, 48 at degree 3): the f64 forward runs 1.1-1.8x faster with one subtree level
         # per lane and all (or half of) the letters than with the two-level subtrees the model picks
