@@ -42,6 +42,9 @@ OVERRIDES = {
     ("f32", 5, 7, "fwd"): (4, 1),
     ("f64", 3, 12, "fwd"): (5, 1),      # 24.1 ms; (4, 3) 25.3, (3, 3) and (4, 1) 31.7
     ("f32", 17, 4, "fwd"): (2, 6),      # staged 0.66 ms; (1, 17) direct 0.96, (2, 9) staged 0.79, (2, 3) staged 0.91
+    # the per-level Horner values of a 12-letter chain leave no room for a depth-4 subtree (256 paths of 200 steps)
+    ("f64", 2, 15, "bwd"): (3, 2),      # 9.4 ms; (4, 2) 13.6, (2, 2) 16.1
+    ("f64", 2, 16, "bwd"): (3, 2),      # 29.0 ms; (4, 2) 58.3, (2, 2) 42.2, (5, 2) 85.8
 }
 
 
