@@ -142,20 +142,6 @@ __device__ __forceinline__ void wait_all_loads()
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <typename T, int D, int N, int TAIL, int K>
-__device__ __forceinline__ typename Tree<T, D, N, TAIL, K>::Inc negate(const typename Tree<T, D, N, TAIL, K>::Inc& in)
-{
-    using Tr = Tree<T, D, N, TAIL, K>;
-    typename Tr::Inc o;
-#pragma unroll
-    for (int j = 0; j < Tr::DD; ++j) o.z[j] = -in.z[j];
-#pragma unroll
-    for (int a = 0; a < K; ++a) o.zs[a] = -in.zs[a];
-#pragma unroll
-    for (int l = 0; l < Tr::M; ++l) o.pz[l] = -in.pz[l];
-    return o;
-}
-
 
 // ---------------------------------------------------------------------------
 // Sweep drivers: feed the increments of steps first, first + DIR, ... (count
@@ -681,6 +667,10 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     // The tile is flushed when `limit` steps sit in it.  The first chunk takes the remainder of count / CH, so that
     // all later chunks are full and the last flush falls on the last step: the test is one 32-bit compare per step.
     int limit = tiled ? (count % CH == 0 ? CH : int(count % CH)) : 0;
+    // The four waves of a block run in step, and four flushes at once queue up in the one LDS unit of the CU.  Each
+    // wave therefore closes its first chunk at a different fill (the last chunk is then partial and flushed after the
+    // sweep), which spreads the flushes of a block over the steps: 2 % of the sweep at batch 32, length 1000, d = 10.
+    if (tiled) limit = (limit - 1 + (wave_in_block * CH) / kWavesPerBlock) % CH + 1;
 
     auto reduce_chunk = [&](int n_slots) {
         wave_lds_sync();
@@ -728,12 +718,23 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         wave_lds_sync();
     };
 
+    // PAIR: word of each chain letter within a step's rows (row and half-wave of the letter, column of this lane in that half)
+    int chain_off[M];
+    if constexpr (PAIR) {
+        constexpr int H = (Tr::DD + 1) / 2;
+#pragma unroll
+        for (int l = 0; l < M; ++l) {
+            const int hi = cx.p[l] >= H ? 1 : 0;
+            chain_off[l] = (cx.p[l] - H * hi) * kRedStride + 32 * hi + (lane & 31);
+        }
+    }
     auto do_step = [&](const typename Tr::Inc& z, int64_t t, auto g0c, auto posc) {
         constexpr int G0 = decltype(g0c)::value;
         constexpr bool FOLD = Ad::template kFoldDepth1<G0>;     // depth-1 pieces already sit in dz.dj
         // position 0 of the reverse sweep is the last step of an even-length range: an odd step
         using Act = std::conditional_t<LL == 0, AllLetters, LeadLagLetters<Tr::DD, 1 - decltype(posc)::value, G0>>;
-        S.template fwd_step<Act>(negate<T, D, N, TAIL, K>(z));     // state before the step
+        typename Tr::Chain unmul;
+        S.template fwd_step<Act, true>(z, &unmul);     // state before the step
         typename Ad::DInc dz;
 #pragma unroll
         for (int j = 0; j < Tr::DD; ++j) dz.dj[j] = T(0);
@@ -741,7 +742,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
         for (int a = 0; a < K; ++a) dz.da[a] = T(0);
 #pragma unroll
         for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
-        A.template pullback<G0, Act>(S, z, dz);
+        A.template pullback<G0, Act>(S, z, dz, Tr::kLockstep ? &unmul : nullptr);
 
         if (tiled) {
             // Idle lanes need no predicate: their adjoints were loaded as zero, so every piece they produce is zero.
@@ -752,13 +753,9 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
 #pragma unroll
                 for (int r = 0; r < H; ++r)
                     col[r * kRedStride] = pair_sum32(dz.dj[r], r + H < Tr::DD ? dz.dj[r + H < Tr::DD ? r + H : 0] : T(0));
-                // chain letters: row and half-wave of the letter, column of this lane within that half
-                T* base = wbuf + cs * (RS * kRedStride) + (lane & 31);
+                T* base = wbuf + cs * (RS * kRedStride);
 #pragma unroll
-                for (int l = 0; l < M; ++l) {
-                    const int hi = cx.p[l] >= H ? 1 : 0;
-                    lds_add_shared(&base[(cx.p[l] - H * hi) * kRedStride + 32 * hi], dz.dc[l]);
-                }
+                for (int l = 0; l < M; ++l) lds_add_shared(&base[chain_off[l]], dz.dc[l]);
             } else if constexpr (TAIL >= 2) {
 #pragma unroll
                 for (int j = 0; j < Tr::DD; ++j) col[j * kRedStride] = dz.dj[j];
@@ -884,6 +881,7 @@ __global__ __launch_bounds__(kBlock) void tree_bwd_kernel(
     } else {
         sweep_direct<-1, false, Cx, typename Tr::Inc>(cx, row, count - 1, count, do_step);
     }
+    if (tiled && cs > 0) reduce_chunk(cs);      // what the staggered first chunk left over
 }
 
 // ---------------------------------------------------------------------------

@@ -34,8 +34,23 @@ __host__ __device__ constexpr int64_t ipow64(int64_t b, int e)
     return r;
 }
 
+// 1 / k.  Reciprocals that are no inline constant of the instruction set (k > 2) are handed out in scalar registers,
+// set once per kernel: as a literal, a multiply-add by such a number has to overwrite its addend, and the compiler
+// then copies the addend first whenever it lives on (one more issue slot per use).
 template <typename T>
-__device__ __forceinline__ constexpr T rcp(int k) { return T(1) / T(k); }
+__device__ __forceinline__ T rcp(int k)
+{
+    T v = T(1) / T(k);
+#ifndef SIGAMD_LITERAL_RCP
+    if (k > 2 && (k & (k - 1)) == 0) asm("" : "+s"(v));
+#endif
+    return v;
+}
+
+// the increment as a step sees it: NEG steps run on the negated increment.  Negating an operand where it is used costs
+// nothing (an operand modifier), while products of the increment itself stay common to a step and its negated twin.
+template <bool NEG, typename T>
+__device__ __forceinline__ T sgn(T x) { return NEG ? -x : x; }
 
 template <typename T>
 __device__ __forceinline__ T fmadd(T a, T b, T c) { return __builtin_fma(a, b, c); }
@@ -220,6 +235,7 @@ struct Tree {
     static constexpr bool kLockstep = M <= 4;
     struct Chain {
         T u[N + 1][M];
+        T q[N + 1][M];      // q[t][l] = z[p_{l+1}] / (t - l), l >= 1: the scaled prefix letters the chains multiply by
     };
 
     // Keeps the instruction scheduler from re-serialising what the source interleaves: the compiler's machine
@@ -228,17 +244,31 @@ struct Tree {
     __device__ __forceinline__ static void pin() { __builtin_amdgcn_sched_barrier(0); }
 
     // All chains of one step in lockstep over the depth; every value is computed from the state before the step.
-    __device__ __forceinline__ void chain_all(const Inc& in, Chain& ch) const
+    // reuse (may be null): the chains of the step with the negated increment taken from the state AFTER that step, i.e.
+    // from this state's successor.  Its value at depth t - 1 of target level t is the integral of the level's node
+    // along the segment, the same number from either end, so those entries are taken over instead of computed
+    // (levels up to kReuseMax, the ones the negated step evaluates).
+    static constexpr int kReuseMax = M + 1 < N - 1 ? M + 1 : N - 1;
+    template <bool NEG = false>
+    __device__ __forceinline__ void chain_all(const Inc& in, Chain& ch, const Chain* reuse = nullptr) const
     {
-        T q[N + 1];     // q[t] = z[p_{l+1}] / (t - l) of the current row
 #pragma unroll
         for (int l = 0; l < M; ++l) {
 #pragma unroll
-            for (int t = l + 2; t <= N; ++t)
-                ch.u[t][l] = (l == 0) ? fmadd(in.pz[0], rcp<T>(t), c[0]) : fmadd(ch.u[t][l - 1], q[t], c[l]);
+            for (int t = l + 2; t <= N; ++t) {
+                if (reuse && t == l + 2 && t <= kReuseMax) ch.u[t][l] = reuse->u[t][l];
+                // the sign goes to the chain value: the negated product would be folded into a constant of the other sign
+                else ch.u[t][l] = (l == 0) ? fmadd(sgn<NEG>(in.pz[0]), rcp<T>(t), c[0]) : fmadd(sgn<NEG>(ch.u[t][l - 1]), ch.q[t][l], c[l]);
+            }
             if (l + 1 < M) {
 #pragma unroll
-                for (int t = l + 3; t <= N; ++t) q[t] = in.pz[l + 1] * rcp<T>(t - l - 1);
+                for (int t = l + 3; t <= N; ++t) {
+                    if (reuse && t <= N - 1) {
+                        ch.q[t][l + 1] = reuse->q[t][l + 1];        // the negated step's products: the same numbers
+                    } else {
+                        ch.q[t][l + 1] = in.pz[l + 1] * rcp<T>(t - l - 1);
+                    }
+                }
             }
             pin();
         }
@@ -247,12 +277,12 @@ struct Tree {
     // Level-by-level form, used for long prefixes: U_t at chain depth `depth` (1 <= depth <= min(t-1, M)):
     //   U(1) = z[p_1]/t + S_1[p_1];  U(l+1) = U(l) * z[p_{l+1}] / (t-l) + S_{l+1}[..]
     // All intermediate values are returned in u[0..depth).
-    template <int t, int depth>
+    template <int t, int depth, bool NEG = false>
     __device__ __forceinline__ void chain_u(const Inc& in, T (&u)[M > 0 ? M : 1]) const
     {
-        u[0] = fmadd(in.pz[0], rcp<T>(t), c[0]);
+        u[0] = fmadd(sgn<NEG>(in.pz[0]), rcp<T>(t), c[0]);
 #pragma unroll
-        for (int l = 1; l < depth; ++l) u[l] = fmadd(u[l - 1] * rcp<T>(t - l), in.pz[l], c[l]);
+        for (int l = 1; l < depth; ++l) u[l] = fmadd(u[l - 1] * rcp<T>(t - l), sgn<NEG>(in.pz[l]), c[l]);
     }
 
     template <int E>
@@ -271,7 +301,7 @@ struct Tree {
         if (E == 1) return ACT::G0 < 0 || ACT::on(ACT::G0 + ch);
         return ACT::on(ch);
     }
-    template <int E, int I, typename ACT = AllLetters>
+    template <int E, int I, typename ACT = AllLetters, bool NEG = false>
     __device__ __forceinline__ void fwd_desc(const Inc& in, T upar, int pidx)
     {
         constexpr int NCH = (E == 1) ? K : DD;
@@ -279,64 +309,67 @@ struct Tree {
 #pragma unroll
             for (int ch = 0; ch < NCH; ++ch)
                 if (letter_on<E, ACT>(ch))
-                    s[off(E) + pidx * NCH + ch] = fmadd(upar, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]);
+                    s[off(E) + pidx * NCH + ch] = fmadd(upar, sgn<NEG>(zc<E>(in, ch)), s[off(E) + pidx * NCH + ch]);
         } else {
             // the children's Horner values first, their consumers afterwards: no FMA directly follows its producer
             const T ur = upar * rcp<T>(I - E + 1);
             T uc[NCH];
 #pragma unroll
             for (int ch = 0; ch < NCH; ++ch)
-                uc[ch] = letter_on<E, ACT>(ch) ? fmadd(ur, zc<E>(in, ch), s[off(E) + pidx * NCH + ch]) : s[off(E) + pidx * NCH + ch];
+                uc[ch] = letter_on<E, ACT>(ch) ? fmadd(ur, sgn<NEG>(zc<E>(in, ch)), s[off(E) + pidx * NCH + ch]) : s[off(E) + pidx * NCH + ch];
             if constexpr (NCH >= 4) pin();      // narrow fans: the regions between pins would be too small to fill
 #pragma unroll
-            for (int ch = 0; ch < NCH; ++ch) fwd_desc<E + 1, I, ACT>(in, uc[ch], pidx * NCH + ch);
+            for (int ch = 0; ch < NCH; ++ch) fwd_desc<E + 1, I, ACT, NEG>(in, uc[ch], pidx * NCH + ch);
         }
     }
 
     // subtree target levels t, t-1, ..., M+1: descending, so that every read of a shallower depth still sees the
     // value from before the step
-    template <int t, typename ACT = AllLetters>
+    template <int t, typename ACT = AllLetters, bool NEG = false>
     __device__ __forceinline__ void fwd_subtree(const Inc& in, const Chain& ch)
     {
         if constexpr (t > M) {
-            fwd_desc<1, t - M, ACT>(in, ch.u[t][M - 1], 0);
-            fwd_subtree<t - 1, ACT>(in, ch);
+            fwd_desc<1, t - M, ACT, NEG>(in, ch.u[t][M - 1], 0);
+            fwd_subtree<t - 1, ACT, NEG>(in, ch);
         }
     }
 
-    template <int t, typename ACT = AllLetters>
+    template <int t, typename ACT = AllLetters, bool NEG = false>
     __device__ __forceinline__ void fwd_level(const Inc& in)
     {
         if constexpr (t == 1) {
-            c[0] += in.pz[0];
+            c[0] += sgn<NEG>(in.pz[0]);
         } else if constexpr (t <= M) {
             T u[M > 0 ? M : 1];
-            chain_u<t, t - 1>(in, u);
-            c[t - 1] = fmadd(u[t - 2], in.pz[t - 1], c[t - 1]);
+            chain_u<t, t - 1, NEG>(in, u);
+            c[t - 1] = fmadd(u[t - 2], sgn<NEG>(in.pz[t - 1]), c[t - 1]);
         } else {
             T u[M > 0 ? M : 1];
-            chain_u<t, M>(in, u);
-            fwd_desc<1, t - M, ACT>(in, u[M - 1], 0);
+            chain_u<t, M, NEG>(in, u);
+            fwd_desc<1, t - M, ACT, NEG>(in, u[M - 1], 0);
         }
-        if constexpr (t > 1) fwd_level<t - 1, ACT>(in);
+        if constexpr (t > 1) fwd_level<t - 1, ACT, NEG>(in);
     }
 
     // S <- S (x) exp(z): target levels in descending order so that every read of
     // a lower level still sees the value from before the step
     // (siglib/cpsig/cp_signature.h:464-499).
-    template <typename ACT = AllLetters>
-    __device__ __forceinline__ void fwd_step(const Inc& in)
+    // NEG: the step with the negated increment, S <- S (x) exp(-z) (the reverse sweep's un-multiply).
+    // keep (lockstep chains only, may be null): receives the chains of this step, for TreeAdj::pullback to take over.
+    template <typename ACT = AllLetters, bool NEG = false>
+    __device__ __forceinline__ void fwd_step(const Inc& in, Chain* keep = nullptr)
     {
         if constexpr (!kLockstep) {
-            fwd_level<N, ACT>(in);
+            fwd_level<N, ACT, NEG>(in);
             return;
         }
         Chain ch;
-        chain_all(in, ch);
-        fwd_subtree<N, ACT>(in, ch);
+        chain_all<NEG>(in, ch);
+        fwd_subtree<N, ACT, NEG>(in, ch);
 #pragma unroll
-        for (int t = M; t >= 2; --t) c[t - 1] = fmadd(ch.u[t][t - 2], in.pz[t - 1], c[t - 1]);
-        c[0] += in.pz[0];
+        for (int t = M; t >= 2; --t) c[t - 1] = fmadd(ch.u[t][t - 2], sgn<NEG>(in.pz[t - 1]), c[t - 1]);
+        c[0] += sgn<NEG>(in.pz[0]);
+        if (keep) *keep = ch;
     }
 };
 
@@ -377,7 +410,7 @@ struct TreeAdj {
     __device__ __forceinline__ T bwd_desc(const Tr& S, const typename Tr::Inc& in, DInc& dz, T upar, int pidx)
     {
         constexpr int NCH = (E == 1) ? K : DD;
-        constexpr T sc = rcp<T>(I - E + 1);
+        const T sc = rcp<T>(I - E + 1);
         const T v = (I - E + 1 == 1) ? upar : upar * sc;
         T red = T(0);
         T uc[NCH];
@@ -463,15 +496,18 @@ struct TreeAdj {
     // the state BEFORE the step.  Target levels ascend so that the adjoint of
     // level t is consumed before higher levels add into it
     // (siglib/cpsig/cp_signature.h:1147-1187).
+    // unmul (lockstep chains only, may be null): the chains of the step with the negated increment that produced S
+    // from its successor (Tree::fwd_step<ACT, true>), see Tree::chain_all.
     template <int G0 = -1, typename ACT = AllLetters>
-    __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz)
+    __device__ __forceinline__ void pullback(const Tr& S, const typename Tr::Inc& in, DInc& dz,
+                                             const typename Tr::Chain* unmul = nullptr)
     {
         if constexpr (!Tr::kLockstep) {
             bwd_level<1, G0, ACT>(S, in, dz);
             return;
         }
         typename Tr::Chain ch;
-        S.chain_all(in, ch);
+        S.template chain_all<false>(in, ch, unmul);
         // Every target level t reads the adjoint of its own chain node as it was before the step and adds into
         // shallower nodes only, so all starting adjoints are taken first and the walks to the root run in
         // lockstep over the depth (consecutive instructions belong to different levels).
@@ -491,13 +527,22 @@ struct TreeAdj {
                 dz.dc[l] = fmadd(a[t], v, dz.dc[l]);
                 a[t] = a[t] * (in.pz[l] * rcp<T>(t - l));
             }
+            if (l == 1) {
+                // the root letter's piece starts from the level-1 adjoint as it was before the step: taken here, ahead
+                // of the sums into that adjoint, it needs no copy
+                dz.dc[0] += gc[0];
+#pragma unroll
+                for (int t = 2; t <= N; ++t) dz.dc[0] = fmadd(a[t], rcp<T>(t), dz.dc[0]);
+            }
 #pragma unroll
             for (int t = l + 1; t <= N; ++t) gc[l - 1] += a[t];
             Tr::pin();
         }
-        dz.dc[0] += g1;
+        if constexpr (M == 1) {
+            dz.dc[0] += g1;
 #pragma unroll
-        for (int t = 2; t <= N; ++t) dz.dc[0] = fmadd(a[t], rcp<T>(t), dz.dc[0]);
+            for (int t = 2; t <= N; ++t) dz.dc[0] = fmadd(a[t], rcp<T>(t), dz.dc[0]);
+        }
     }
 };
 
