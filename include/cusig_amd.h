@@ -235,6 +235,19 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
  * kernels that store the result set the flag, so a caller who must warn about overflow (pysiglib/sig.py:299-311
  * scans the result for NaN and Inf) needs no pass of its own over the output.  No counterpart in the reference. */
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) CUSIG_AMD_NOEXCEPT;
+/* The tuning and test hooks declared from here on (cusig_amd_force_*, cusig_amd_set_point_fed, _set_lead_lag_sparse,
+ * _set_chen_low_levels, _set_degree2_staged, _set_alloc_limit) are process-wide switches for offline sweeps and for the
+ * test-suite.  They are ignored until cusig_amd_enable_test_hooks(1) has been called; cusig_amd_enable_test_hooks(0)
+ * restores every default.  No counterpart in the reference. */
+CUSIG_AMD_API void cusig_amd_enable_test_hooks(int enabled) CUSIG_AMD_NOEXCEPT;
+/* Test hook: workspace requests of more than `bytes` bytes fail as if the device were out of memory (0: no limit), which
+ * exercises the retry on halves of the batch (siglib/cusig/cu_runtime_utils.h:103-105,212-235) and the fall-back of the
+ * degree-3 matrix form to the sweeps.  cusig_amd_alloc_retries counts the splits since the library was loaded. */
+CUSIG_AMD_API void cusig_amd_set_alloc_limit(uint64_t bytes) CUSIG_AMD_NOEXCEPT;
+CUSIG_AMD_API int cusig_amd_alloc_retries(void) CUSIG_AMD_NOEXCEPT;
+/* Bytes the library's grow-only workspace pool holds on the current device (released by cusig_shutdown).  A host-side
+ * query; no counterpart in the reference. */
+CUSIG_AMD_API uint64_t cusig_amd_workspace_bytes(void) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the forward sweep splits every path into (0 = automatic). */
 CUSIG_AMD_API void cusig_amd_force_segments(int segments) CUSIG_AMD_NOEXCEPT;
 /* Number of time segments per path in the last forward sweep on this thread (0 if no sweep kernel ran). */
@@ -272,7 +285,8 @@ CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_force_degree2(int mode) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: degree 3 as rocBLAS matrix products around a scan kernel (backward: two products, forward: one):
  * -1 automatic (backward from 48 channels in float32 and 36 in float64, forward from 112, given enough paths to fill
- * the chip and a librocblas that can be opened), 0 never, 1 whenever the degree is 3. */
+ * the chip, a librocblas that can be opened and a device that can hold the extra rows buffer of up to 1 GiB; otherwise
+ * the sweeps serve the shape), 0 never, 1 whenever the degree is 3 and one path's rows fit the buffer. */
 CUSIG_AMD_API void cusig_amd_force_degree3(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: 1 routes every sweep of 2, 3 or 4 augmented channels that the run-time-degree kernels can serve
  * (degree >= 5, 4, 3 respectively) to them; by default they only serve degrees 17 .. 64. */

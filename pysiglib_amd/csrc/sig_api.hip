@@ -58,6 +58,9 @@ struct Table {
 // Process-wide hooks (tuning, tests, measurement) may be set by one thread while another is inside a call: atomics,
 // read once where a call needs a consistent value.
 using Hook = std::atomic<int>;
+// the tuning and test hooks below only take effect after cusig_amd_enable_test_hooks(1): a caller that merely links
+// the library cannot reroute the kernels of other threads by accident
+static Hook g_test_hooks{0};
 // tuning hook: when set (tail > 0), prefer the compiled partition with this (tail, k)
 static Hook g_force_tail{0}, g_force_k{0};
 static Hook g_force_run_time_wide{0};   // with a forced partition: take the run-time-dimension kernel in the wide layout
@@ -208,6 +211,10 @@ std::atomic<int> g_chen_low_levels{1};
 std::mutex g_ws_mutex;
 static std::map<std::pair<int, int>, Workspace> g_ws;   // (device, slot)
 
+// test hook: workspace requests above this many bytes fail as if the device were out of memory (0: no limit)
+static std::atomic<uint64_t> g_alloc_limit{0};
+static std::atomic<int> g_alloc_retries{0};     // calls split in two after a failed workspace allocation
+
 void* workspace(int slot, size_t bytes)
 {
     int dev = 0;
@@ -220,7 +227,8 @@ void* workspace(int slot, size_t bytes)
             w.bytes = 0;
         }
         const size_t want = (bytes + bytes / 8 + 255) & ~size_t(255);
-        if (hipMalloc(&w.ptr, want) != hipSuccess) {
+        const uint64_t limit = g_alloc_limit;
+        if ((limit && want > limit) || hipMalloc(&w.ptr, want) != hipSuccess) {
             (void)hipGetLastError();
             w.ptr = nullptr;
             throw std::bad_alloc();
@@ -507,7 +515,8 @@ static Hook g_degree2_staged{1};    // tuning hook: 0 keeps the operands of the 
 // Measured against the sweeps for d = 3 .. 256: the backward wins everywhere (1.4x at d = 4, 20x at d = 64), the
 // forward from about 12 channels on and for small dimensions whenever the sweeps cannot fill the chip.
 static Hook g_force_degree3{-1};    // tuning hook: -1 automatic, 0 never, 1 whenever the degree is 3
-constexpr uint64_t kDeg3BufBytes = uint64_t(4) << 30;
+// rows buffer [paths of a chunk][L][d^2] of the degree-3 matrix form: paths are taken in chunks that fit this many bytes
+constexpr uint64_t kDeg3BufBytes = uint64_t(1) << 30;
 
 // degree 3 as library matrix products around a scan (sig_degree3.h): two products backward, one forward.  Measured against the sweep kernels at
 // batch 512, length 256: float32 1.3x faster from 48 channels (4.6x at 80, 11x at 128), float64 from 36 (10x at 80);
@@ -515,6 +524,8 @@ constexpr uint64_t kDeg3BufBytes = uint64_t(4) << 30;
 static bool want_degree3_gemm(uint64_t d_aug, uint64_t degree, uint64_t L, uint64_t batch, bool f64, bool backward)
 {
     if (degree != 3 || d_aug < 2 || d_aug > uint64_t(kDeg3MaxDim) || L > 0x7fffffff) return false;
+    // one path's rows must fit the buffer (longer paths stay with the sweeps, which need B * L * d elements)
+    if (L > kDeg3BufBytes / (d_aug * d_aug * (f64 ? 8 : 4))) return false;
     if (g_force_degree3 >= 0) return g_force_degree3 != 0;
     const uint64_t waves = ((d_aug + kWave - 1) / kWave) * ((d_aug + kDeg3RowsPerThread - 1) / kDeg3RowsPerThread) * batch;
     const uint64_t from = backward ? (f64 ? 36u : 48u) : 112u;      // forward: 1.3x at 128 channels, slower at 80
@@ -604,6 +615,41 @@ static void compute_increments(const T* path, T* inc, uint64_t batch, uint64_t d
     SIG_HIP(hipGetLastError());
 }
 
+// Everything the degree-3 matrix form needs from the device, taken before anything is launched: when the device
+// cannot provide it (or rocBLAS cannot create its handle) `ok` stays false and the caller sweeps the shape instead,
+// which needs B * L * d elements of workspace where this form needs up to kDeg3BufBytes more.
+template <typename T>
+struct Degree3Buffers {
+    bool ok = false;
+    uint64_t chunk = 0;     // paths per pass over the rows buffer
+    T* inc = nullptr;
+    T* dzinc = nullptr;     // backward only
+    T* r1 = nullptr;        // backward only
+    T* rows = nullptr;
+    RocBlas::Handle handle = nullptr;
+
+    void acquire(uint64_t batch, const Shape& s, hipStream_t stream, bool backward)
+    {
+        try {
+            const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
+            const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
+            const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
+            if (per_path == 0 || per_path > kDeg3BufBytes) return;
+            chunk = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(batch, 65535), kDeg3BufBytes / per_path));
+            inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
+            if (backward) {
+                dzinc = static_cast<T*>(workspace(1, checked_mul(dz_elems, sizeof(T), "increments")));
+                r1 = static_cast<T*>(workspace(18, checked_mul(dz_elems, sizeof(T), "increments")));
+            }
+            rows = static_cast<T*>(workspace(19, checked_mul(chunk, per_path, "level-2 rows")));
+            handle = rocblas_handle_for(stream);
+            ok = true;
+        } catch (const std::bad_alloc&) {
+        } catch (const std::runtime_error&) {       // no rocBLAS handle
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------
 // forward  (dispatch mirrors siglib/cpsig/cp_signature.h:740-851 and
 // siglib/cusig/cu_signature.cu:2592-2657)
@@ -634,6 +680,9 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
     }
 
     const int sc = scalar_term ? 1 : 0;
+    Degree3Buffers<T> d3;
+    if (s.len_aug > 1 && s.d_aug > 1 && want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, false) && rocblas_ready())
+        d3.acquire(batch, s, stream, false);
     if (s.len_aug <= 1) {
         if (s.stride)
             hipLaunchKernelGGL((fill_trivial_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
@@ -650,16 +699,14 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         hipLaunchKernelGGL((degree_one_fwd_kernel<T>), dim3(grid_for(batch * s.stride)), dim3(kBlock), 0, stream,
                            path, out, int64_t(batch), int64_t(length), int(dimension), int(time_aug),
                            int(lead_lag), time_step, sc, flag);
-    } else if (want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, false) && rocblas_ready()) {
+    } else if (d3.ok) {
         const int d = int(s.d_aug);
         const int64_t L = int64_t(s.L);
-        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
-        const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
-        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(batch, 65535), kDeg3BufBytes / per_path));
-        T* inc = static_cast<T*>(workspace(0, checked_mul(inc_elems, sizeof(T), "increments")));
-        T* rows = static_cast<T*>(workspace(19, checked_mul(chunk, per_path, "level-2 rows")));
+        const uint64_t chunk = d3.chunk;
+        T* inc = d3.inc;
+        T* rows = d3.rows;
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
-        RocBlas::Handle h = rocblas_handle_for(stream);
+        RocBlas::Handle h = d3.handle;
         tl_last_segments = 1;
         MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree3_fwd_gemm_f64" : "degree3_fwd_gemm_f32");
         const int64_t dd = int64_t(d) * d;
@@ -920,11 +967,12 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
     auto finish = [&] { if (!arena) exit_sync(stream); };
     std::unique_lock<std::mutex> lk(g_ws_mutex, std::defer_lock);
     auto lock_pool = [&] { if (!arena && !lk.owns_lock()) lk.lock(); };
-    bool degree3 = !arena && s.len_aug > 1 && want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, true);
-    if (degree3) {
+    Degree3Buffers<T> d3;
+    if (!arena && s.len_aug > 1 && want_degree3_gemm(s.d_aug, degree, s.L, batch, sizeof(T) == 8, true)) {
         lock_pool();
-        degree3 = rocblas_ready();
+        if (rocblas_ready()) d3.acquire(batch, s, stream, true);
     }
+    const bool degree3 = d3.ok;
 
     if (s.len_aug <= 1 || degree == 0) {
         if (out_elems)
@@ -937,17 +985,15 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
     } else if (degree3) {
         const int d = int(s.d_aug);
         const int64_t L = int64_t(s.L);
-        const uint64_t inc_elems = checked_mul(checked_mul(batch, s.L + 2, "increments"), s.d_aug, "increments");
         const uint64_t dz_elems = checked_mul(checked_mul(batch, s.L, "increments"), s.d_aug, "increments");
-        const uint64_t per_path = checked_mul(checked_mul(s.L, s.d_aug * s.d_aug, "level-2 rows"), sizeof(T), "level-2 rows");
-        const uint64_t chunk = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(batch, 65535), kDeg3BufBytes / per_path));
-        T* inc = static_cast<T*>(buffer(0, checked_mul(inc_elems, sizeof(T), "increments")));
-        T* dzinc = static_cast<T*>(buffer(1, checked_mul(dz_elems, sizeof(T), "increments")));
-        T* r1 = static_cast<T*>(buffer(18, checked_mul(dz_elems, sizeof(T), "increments")));
-        T* rows = static_cast<T*>(buffer(19, checked_mul(chunk, per_path, "level-2 rows")));
+        const uint64_t chunk = d3.chunk;
+        T* inc = d3.inc;
+        T* dzinc = d3.dzinc;
+        T* r1 = d3.r1;
+        T* rows = d3.rows;
         compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream, dzinc, dz_elems);
         hipLaunchKernelGGL((zero_kernel<T>), dim3(grid_for(dz_elems)), dim3(kBlock), 0, stream, r1, int64_t(dz_elems));
-        RocBlas::Handle h = rocblas_handle_for(stream);
+        RocBlas::Handle h = d3.handle;
         MainKernelTimer timer(stream, sizeof(T) == 8 ? "degree3_bwd_gemm_f64" : "degree3_bwd_gemm_f32", true);
         const int64_t dd = int64_t(d) * d;
         const int groups = (d + kDeg3RowsPerThread - 1) / kDeg3RowsPerThread;
@@ -1268,9 +1314,43 @@ static void* scratch_of_current_device()
     return ptr;
 }
 
+void note_alloc_retry() noexcept { ++g_alloc_retries; }
+
 }  // namespace sigamd
 
 using namespace sigamd;
+
+// signature_cuda_* with the batch taken in halves when the device cannot hold the workspace of the whole call
+template <typename T>
+static void signature_entry(const T* path, T* out, uint64_t batch, uint64_t dimension, uint64_t length, uint64_t degree,
+                            bool time_aug, bool lead_lag, T end_time, bool horner, bool scalar_term, const T* correction,
+                            uint64_t correction_len)
+{
+    int nonfinite = 0;
+    split_on_bad_alloc(batch, "signature", [&](uint64_t first, uint64_t count) {
+        uint64_t stride = 0;
+        if (first) stride = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term).stride;
+        signature_impl<T>(path + first * length * dimension, out + first * stride, count, dimension, length, degree, time_aug,
+                          lead_lag, end_time, horner, scalar_term, correction, correction_len);
+        const int f = tl_sig_nonfinite;
+        nonfinite = (nonfinite < 0 || f < 0) ? -1 : (nonfinite | f);
+    });
+    if (batch) tl_sig_nonfinite = nonfinite;
+}
+
+template <typename T>
+static void sig_backprop_entry(const T* path, T* out, const T* sig_derivs, const T* sig, uint64_t batch, uint64_t dimension,
+                               uint64_t length, uint64_t degree, bool time_aug, bool lead_lag, T end_time, bool scalar_term,
+                               const T* correction, uint64_t correction_len)
+{
+    split_on_bad_alloc(batch, "sig_backprop", [&](uint64_t first, uint64_t count) {
+        uint64_t stride = 0;
+        if (first) stride = make_shape(dimension, length, degree, time_aug, lead_lag, scalar_term).stride;
+        sig_backprop_impl<T>(path + first * length * dimension, out + first * length * dimension, sig_derivs + first * stride,
+                             sig + first * stride, count, dimension, length, degree, time_aug, lead_lag, end_time, scalar_term,
+                             correction, correction_len);
+    });
+}
 
 extern "C" {
 
@@ -1280,8 +1360,8 @@ CUSIG_AMD_API int signature_cuda_f(const float* path, float* out, uint64_t batch
                                    uint64_t correction_len, uint64_t, uint64_t) noexcept
 {
     return guarded([&] {
-        signature_impl<float>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
-                              horner, scalar_term, correction, correction_len);
+        signature_entry<float>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
+                               horner, scalar_term, correction, correction_len);
     });
 }
 
@@ -1291,8 +1371,8 @@ CUSIG_AMD_API int signature_cuda_d(const double* path, double* out, uint64_t bat
                                    uint64_t correction_len, uint64_t, uint64_t) noexcept
 {
     return guarded([&] {
-        signature_impl<double>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
-                               horner, scalar_term, correction, correction_len);
+        signature_entry<double>(path, out, batch_size, dimension, length, degree, time_aug, lead_lag, end_time,
+                                horner, scalar_term, correction, correction_len);
     });
 }
 
@@ -1303,8 +1383,8 @@ CUSIG_AMD_API int sig_backprop_cuda_f(const float* path, float* out, const float
                                       uint64_t) noexcept
 {
     return guarded([&] {
-        sig_backprop_impl<float>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
-                                 lead_lag, end_time, scalar_term, correction, correction_len);
+        sig_backprop_entry<float>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
+                                  lead_lag, end_time, scalar_term, correction, correction_len);
     });
 }
 
@@ -1315,8 +1395,8 @@ CUSIG_AMD_API int sig_backprop_cuda_d(const double* path, double* out, const dou
                                       uint64_t correction_len, uint64_t, uint64_t) noexcept
 {
     return guarded([&] {
-        sig_backprop_impl<double>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
-                                  lead_lag, end_time, scalar_term, correction, correction_len);
+        sig_backprop_entry<double>(path, out, sig_derivs, sig, batch_size, dimension, length, degree, time_aug,
+                                   lead_lag, end_time, scalar_term, correction, correction_len);
     });
 }
 
@@ -1362,37 +1442,75 @@ CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) noexcept
     return name;
 }
 
-CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { g_force_segments = segments; }
+CUSIG_AMD_API void cusig_amd_force_segments(int segments) noexcept { if (g_test_hooks) g_force_segments = segments; }
 CUSIG_AMD_API int cusig_amd_last_segments(void) noexcept { return tl_last_segments; }
-CUSIG_AMD_API void cusig_amd_set_point_fed(int on) noexcept { g_point_fed = on; }
-CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) noexcept { g_lead_lag_sparse = on; }
+CUSIG_AMD_API void cusig_amd_set_point_fed(int on) noexcept { if (g_test_hooks) g_point_fed = on; }
+CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) noexcept { if (g_test_hooks) g_lead_lag_sparse = on; }
 
-CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { g_force_bwd_segments = segments; }
+CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { if (g_test_hooks) g_force_bwd_segments = segments; }
 
-CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { g_force_staged = mode; }
+CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { if (g_test_hooks) g_force_staged = mode; }
 
-CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { g_force_wide_index = enabled; }
-CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) noexcept { g_chen_adjoint_mode = mode; }
-CUSIG_AMD_API void cusig_amd_set_chen_low_levels(int enabled) noexcept { g_chen_low_levels = enabled; }
+CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { if (g_test_hooks) g_force_wide_index = enabled; }
+CUSIG_AMD_API void cusig_amd_force_chen_adjoint(int mode) noexcept { if (g_test_hooks) g_chen_adjoint_mode = mode; }
+CUSIG_AMD_API void cusig_amd_set_chen_low_levels(int enabled) noexcept { if (g_test_hooks) g_chen_low_levels = enabled; }
 
 CUSIG_AMD_API void cusig_amd_set_stream_ordered(int enabled) noexcept { g_stream_ordered = enabled; }
 
 CUSIG_AMD_API int cusig_amd_last_sig_nonfinite(void) noexcept { return tl_sig_nonfinite; }
 
-CUSIG_AMD_API void cusig_amd_force_degree2(int mode) noexcept { g_force_degree2 = mode; }
-CUSIG_AMD_API void cusig_amd_force_degree3(int mode) noexcept { g_force_degree3 = mode; }
+CUSIG_AMD_API void cusig_amd_force_degree2(int mode) noexcept { if (g_test_hooks) g_force_degree2 = mode; }
+CUSIG_AMD_API void cusig_amd_force_degree3(int mode) noexcept { if (g_test_hooks) g_force_degree3 = mode; }
 
-CUSIG_AMD_API void cusig_amd_force_deep(int enabled) noexcept { g_force_deep = enabled; }
+CUSIG_AMD_API void cusig_amd_force_deep(int enabled) noexcept { if (g_test_hooks) g_force_deep = enabled; }
 
-CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) noexcept { g_degree2_staged = enabled; }
+CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) noexcept { if (g_test_hooks) g_degree2_staged = enabled; }
 
-CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { g_force_run_time_wide = enabled; }
+CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { if (g_test_hooks) g_force_run_time_wide = enabled; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
 {
+    if (!g_test_hooks) return;
     g_force_tail = tail;
     g_force_k = k;
 }
+
+CUSIG_AMD_API void cusig_amd_enable_test_hooks(int enabled) noexcept
+{
+    g_test_hooks = enabled != 0;
+    if (enabled) return;
+    // back to the defaults
+    g_force_segments = 0;
+    g_point_fed = 1;
+    g_lead_lag_sparse = 1;
+    g_force_bwd_segments = 0;
+    g_force_staged = -1;
+    g_force_wide_index = 0;
+    g_chen_adjoint_mode = 0;
+    g_chen_low_levels = 1;
+    g_force_degree2 = -1;
+    g_force_degree3 = -1;
+    g_force_deep = 0;
+    g_degree2_staged = 1;
+    g_force_run_time_wide = 0;
+    g_force_tail = 0;
+    g_force_k = 0;
+    g_alloc_limit = 0;
+}
+
+CUSIG_AMD_API uint64_t cusig_amd_workspace_bytes(void) noexcept
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    uint64_t total = 0;
+    for (const auto& kv : g_ws)
+        if (kv.first.first == dev) total += kv.second.bytes;
+    return total;
+}
+
+CUSIG_AMD_API void cusig_amd_set_alloc_limit(uint64_t bytes) noexcept { if (g_test_hooks) g_alloc_limit = bytes; }
+CUSIG_AMD_API int cusig_amd_alloc_retries(void) noexcept { return g_alloc_retries; }
 
 CUSIG_AMD_API int cusig_amd_kernel_choice(int backward, int is_f64, uint64_t dimension, uint64_t degree,
                                           int* tail, int* k, int* specialised) noexcept

@@ -38,6 +38,36 @@ struct HipFailure : std::runtime_error {
         if (e__ != hipSuccess) throw ::sigamd::HipFailure(e__, #call); \
     } while (0)
 
+// Out of device memory, like the reference (siglib/cusig/cu_runtime_utils.h:103-105,212-235): a call whose workspace
+// the device cannot hold is retried on halves of its batch; only when a single path does not fit does the call fail,
+// as a device error (status 100000 + hipErrorOutOfMemory).  run(first, count) handles `count` batch items from
+// `first` on and throws std::bad_alloc when a workspace cannot be had.  A half that failed may already have written
+// part of its outputs; the retry overwrites them.
+void note_alloc_retry() noexcept;      // counts the splits (defined in sig_api.hip)
+template <typename F>
+void split_on_bad_alloc(uint64_t batch, const char* who, F&& run)
+{
+    struct Range {
+        uint64_t first, count;
+    };
+    Range stack[70];        // depth of a binary split of 2^64 items
+    int top = 0;
+    stack[top++] = Range{0, batch};
+    while (top) {
+        const Range r = stack[--top];
+        try {
+            run(r.first, r.count);
+        } catch (const std::bad_alloc&) {
+            if (r.count <= 1)
+                throw HipFailure(hipErrorOutOfMemory, (std::string(who) + ": the workspace of a single batch item does not fit the device").c_str());
+            note_alloc_retry();
+            const uint64_t half = r.count / 2;
+            stack[top++] = Range{r.first + half, r.count - half};
+            stack[top++] = Range{r.first, half};
+        }
+    }
+}
+
 // a runtime error that carries its own status code (siglib/shared/errors.h: 5 = prepared cache not found)
 struct CodedError : std::runtime_error {
     int code;

@@ -758,8 +758,12 @@ CUSIG_AMD_API int sig_join_backprop_cuda_f(const float* d_out, float* d_sig, flo
                                            uint64_t degree, bool prepend, bool scalar_term) noexcept
 {
     return guarded([&] {
-        sig_join_backprop_impl<float>(d_out, d_sig, d_displacement, sig, displacement, batch_size, dimension, degree, prepend,
+        split_on_bad_alloc(batch_size, "sig_join_backprop", [&](uint64_t first, uint64_t count) {
+            const uint64_t stride = first ? sig_shape(dimension, degree, scalar_term, "sig_join_backprop_cuda").stride : 0;
+            sig_join_backprop_impl<float>(d_out + first * stride, d_sig + first * stride, d_displacement + first * dimension,
+                                      sig + first * stride, displacement + first * dimension, count, dimension, degree, prepend,
                                       scalar_term);
+        });
     });
 }
 CUSIG_AMD_API int sig_join_backprop_cuda_d(const double* d_out, double* d_sig, double* d_displacement, const double* sig,
@@ -767,8 +771,12 @@ CUSIG_AMD_API int sig_join_backprop_cuda_d(const double* d_out, double* d_sig, d
                                            uint64_t degree, bool prepend, bool scalar_term) noexcept
 {
     return guarded([&] {
-        sig_join_backprop_impl<double>(d_out, d_sig, d_displacement, sig, displacement, batch_size, dimension, degree, prepend,
+        split_on_bad_alloc(batch_size, "sig_join_backprop", [&](uint64_t first, uint64_t count) {
+            const uint64_t stride = first ? sig_shape(dimension, degree, scalar_term, "sig_join_backprop_cuda").stride : 0;
+            sig_join_backprop_impl<double>(d_out + first * stride, d_sig + first * stride, d_displacement + first * dimension,
+                                       sig + first * stride, displacement + first * dimension, count, dimension, degree, prepend,
                                        scalar_term);
+        });
     });
 }
 

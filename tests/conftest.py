@@ -23,3 +23,19 @@ def kats():
     import json
     with open(os.path.join(ROOT, "tests", "golden", "kats.json")) as fh:
         return json.load(fh)
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _library_test_hooks():
+    """The library ignores its tuning and test hooks (cusig_amd_force_*, ...) until they are switched on."""
+    import ctypes
+    try:
+        from pysiglib_amd import _loader as L
+    except Exception:       # no built library: the tests that need it fail on their own
+        yield
+        return
+    L.CUSIG.cusig_amd_enable_test_hooks.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_enable_test_hooks.restype = None
+    L.CUSIG.cusig_amd_enable_test_hooks(1)
+    yield
+    L.CUSIG.cusig_amd_enable_test_hooks(0)

@@ -123,6 +123,36 @@ def test_kernel_table(lib):
             assert fn(bwd, f64, 2, 40, tail, k, spec) == 0                           # served by the run-time-degree sweeps, not by the table
 
 
+def test_hooks_need_to_be_switched_on(lib):
+    """The tuning and test hooks are ignored until cusig_amd_enable_test_hooks(1); switching them off restores the defaults
+    (seen through the kernel table, a host-side query)."""
+    fn = lib.cusig_amd_kernel_choice
+    fn.argtypes = (ctypes.c_int, ctypes.c_int, ctypes.c_uint64, ctypes.c_uint64) + (ctypes.POINTER(ctypes.c_int),) * 3
+    lib.cusig_amd_force_partition.argtypes = (ctypes.c_int, ctypes.c_int)
+    lib.cusig_amd_force_partition.restype = None
+    lib.cusig_amd_enable_test_hooks.argtypes = (ctypes.c_int,)
+    lib.cusig_amd_enable_test_hooks.restype = None
+    tail, k, spec = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+
+    def letters_per_lane():
+        assert fn(0, 0, 150, 3, tail, k, spec) == 1
+        return k.value
+
+    try:
+        lib.cusig_amd_enable_test_hooks(0)
+        default = letters_per_lane()
+        assert default != 4
+        lib.cusig_amd_force_partition(1, 4)
+        assert letters_per_lane() == default          # ignored
+        lib.cusig_amd_enable_test_hooks(1)
+        lib.cusig_amd_force_partition(1, 4)
+        assert letters_per_lane() == 4
+        lib.cusig_amd_enable_test_hooks(0)
+        assert letters_per_lane() == default          # defaults restored
+    finally:
+        lib.cusig_amd_enable_test_hooks(1)            # the session fixture's state
+
+
 def test_wrapper_argument_errors():
     import pysiglib_amd as P
     x = torch.zeros(3, 4, 2)
