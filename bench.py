@@ -4,8 +4,9 @@ A "step" is one forward + one backward pass of the headline workload
 (batch 32, length 1000, dimension 10, degree 5, float64; path points iid N(0,1))
 through the library's C ABI with all buffers resident in HBM.  Prints ONE JSON line.
 
-Order of a run: every other leg first (configs 2-4, the degree-2 case, stream-ordered mode, per-kernel timings), then the
-headline: W untimed warm-up steps, K timed steps, each step timed on its own (both calls are synchronous).
+Order of a run: every other leg first (configs 2-4, the extra shapes, stream-ordered mode, per-kernel timings), then the
+headline: W untimed warm-up steps, K timed steps, each step timed on its own (both calls are synchronous); after it the
+same calls through the Python wrappers and the measured FMA ceilings.
 `ms_per_step` is the median step, `ms_per_step_mean` the mean over the same K steps; `value` follows the median.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all-configs]
@@ -24,16 +25,44 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"float64": 78.6, "float32": 157.3}
 
-# HBM bytes per launch of the sweep kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
-# known size (profiles/sweep_kernels_hbm_traffic.txt).  Keyed by kernel instance so that a re-tuned partition
-# reports null instead of a stale figure.
-TRAFFIC_BYTES = {
-    "fwd_f64_d10_n5_t2_k5_lds": 35.8e6,
-    "bwd_f64_d10_n5_t2_k5_lds": 149.3e6,
-    "fwd_f32_d5_n7_t4_k1_lds": 163.4e6,    # swept in three time pieces: three segment signature sets are written
-    "fwd_f64_d3_n12_t5_k1": 478.7e6,
-    "fwd_f32_d17_n4_t2_k6_lds_ll": 114.4e6,
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "sweep_kernels_hbm_traffic.txt")
+
+
+def traffic_bytes(instance):
+    """HBM bytes per launch of a sweep kernel as measured with rocprofv3 (FETCH_SIZE / WRITE_SIZE scaled by a plain copy
+    of known size), read from the committed summary; None when the summary has no row for this instance, e.g. after a
+    partition was re-tuned.  `instance` is the library's name, e.g. bwd_f64_d10_n5_t2_k5_lds[_ll]."""
+    import re
+    m = re.match(r"^(fwd|bwd)_(f64|f32)_d(\d+)_n(\d+)_t(\d+)_k(\d+)(_lds)?(_ll)?$", instance)
+    if not m or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    d = int(m.group(3))
+    ll = 0 if not m.group(8) else (1 if d % 2 else 2)
+    row = "tree_%s_kernel<%s, %d, %s, %s, %s, %s, %d>" % (m.group(1), "double" if m.group(2) == "f64" else "float", d, m.group(4),
+                                                           m.group(5), m.group(6), "true" if m.group(7) else "false", ll)
+    with open(TRAFFIC_PROFILE) as fh:
+        for line in fh:
+            if line.startswith(row):
+                cols = line[len(row):].split()
+                if len(cols) >= 3:
+                    return float(cols[2]) * 1e6      # columns: FETCH KiB, WRITE KiB, traffic MB, algorithmic MB
+    return None
+
+
+def measured_peaks(loader):
+    """Independent FMAs and nothing else, at 1 / 2 / 8 waves per SIMD (a kernel of the library): the ceiling the chip
+    reaches against the nominal peak.  The headline sweeps run one wave per SIMD."""
+    fn = loader.CUSIG.cusig_amd_measure_fma_peak
+    fn.argtypes = (ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double))
+    fn.restype = ctypes.c_int
+    out = {}
+    for name, is_f64 in (("f64", 1), ("f32_unpacked", 0)):
+        out[name] = {}
+        for waves in (1, 2, 8):
+            v = ctypes.c_double()
+            rc = fn(is_f64, waves, ctypes.byref(v))
+            out[name]["%d_waves_per_simd" % waves] = v.value if rc == 0 else None
+    return out
 
 
 def parse():
@@ -357,6 +386,11 @@ def main():
                 tf = tb * (tl - 1) * fl / (kms * 1e-3) / 1e12
                 configs[tag] = {"signatures_per_s": tb / wall, "call_ms": wall * 1e3, "kernel": name, "kernel_ms": kms,
                                 "tflops": tf, "roofline_frac": tf / PEAK_TFLOPS["float32"]}
+                if "degree3" in name:
+                    configs[tag]["note"] = ("runs as matrix products on the matrix cores around a scan: tflops is the sweep's "
+                                            "operation count over the time (a sweep-equivalent rate), and roofline_frac sets "
+                                            "it against the vector FP32 peak the sweep would be bound by; neither is a "
+                                            "utilisation of the matrix pipe")
             del xp, sg, gg, gx
             torch.cuda.empty_cache()
 
@@ -364,12 +398,14 @@ def main():
         r1.forward()
         r5.backward()
 
-    # the same steps with the library in stream-ordered mode: calls only enqueue, the host syncs once at the end
+    # the same steps with the library in stream-ordered mode (calls only enqueue, the host syncs once at the end).  The
+    # legs before it end with long kernels that leave the clocks low: it gets a longer warm-up of its own, and in turn
+    # leaves the device in the state the headline is measured in.
     loader.CUSIG.cusig_amd_set_stream_ordered.argtypes = (ctypes.c_int,)
     loader.CUSIG.cusig_amd_set_stream_ordered.restype = None
     loader.CUSIG.cusig_amd_set_stream_ordered(1)
     try:
-        for _ in range(args.warmup):
+        for _ in range(max(args.warmup, 50)):
             step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -381,20 +417,39 @@ def main():
         loader.CUSIG.cusig_amd_set_stream_ordered(0)
         torch.cuda.synchronize()
 
-    # per-kernel figures (HIP events inside the library, on the launch stream)
-    wall_f, kms_f, name_f = time_calls(r1.forward, torch, loader, 1, max(5, args.steps))
-    wall_b, kms_b, name_b = time_calls(r5.backward, torch, loader, 1, max(5, args.steps))
+    # per-kernel figures of the same two calls (HIP events inside the library, on the launch stream)
+    wall_f, kms_f, name_f = time_calls(r1.forward, torch, loader, 3, max(5, args.steps))
+    wall_b, kms_b, name_b = time_calls(r5.backward, torch, loader, 3, max(5, args.steps))
     tf_f = r1.flops_fwd / (kms_f * 1e-3) / 1e12
     tf_b = r5.flops_bwd / (kms_b * 1e-3) / 1e12
-    # the headline comes last, after every other leg of this run, so that it is timed on a device in steady state
+    # the headline comes after every other leg on the sweep kernels, so that it is timed on a device in steady state
     ms_per_step, ms_mean = time_steps(step, torch, args.warmup, args.steps)
     value = r1.c["batch"] / (ms_per_step * 1e-3)
+
+
+    # the Python wrappers on the same device tensors: argument checks, output allocation, the overflow report
+    import pysiglib_amd
+    x1, g5, s5 = r1.path, r5.gsig, r5.sig
+
+    def wrapped(fn):
+        for _ in range(5):
+            fn()
+        each = []
+        for _ in range(max(10, min(args.steps, 100))):
+            t0 = time.perf_counter()
+            fn()
+            each.append(time.perf_counter() - t0)
+        return statistics.median(each) * 1e3
+
+    wrap_f = wrapped(lambda: pysiglib_amd.sig(x1, r1.c["degree"]))
+    wrap_b = wrapped(lambda: pysiglib_amd.sig_backprop(x1, s5, g5, r5.c["degree"]))
+    peaks = measured_peaks(loader)      # last: its sustained full-rate kernels leave the clocks lower than they found them
     dominant = {"kernel": name_b, "ms": kms_b, "tflops": tf_b} if kms_b >= kms_f else {"kernel": name_f, "ms": kms_f, "tflops": tf_f}
     headline = {
-        "C1": {"signatures_per_s": r1.c["batch"] / wall_f, "call_ms": wall_f * 1e3, "kernel": name_f,
-               "kernel_ms": kms_f, "tflops": tf_f, "roofline_frac": tf_f / peak},
-        "C5": {"signatures_per_s": r5.c["batch"] / wall_b, "call_ms": wall_b * 1e3, "kernel": name_b,
-               "kernel_ms": kms_b, "tflops": tf_b, "roofline_frac": tf_b / peak},
+        "C1": {"signatures_per_s": r1.c["batch"] / wall_f, "call_ms": wall_f * 1e3, "python_wrapper_call_ms": wrap_f,
+               "kernel": name_f, "kernel_ms": kms_f, "tflops": tf_f, "roofline_frac": tf_f / peak},
+        "C5": {"signatures_per_s": r5.c["batch"] / wall_b, "call_ms": wall_b * 1e3, "python_wrapper_call_ms": wrap_b,
+               "kernel": name_b, "kernel_ms": kms_b, "tflops": tf_b, "roofline_frac": tf_b / peak},
     }
     headline.update(configs)
     configs = headline
@@ -419,7 +474,13 @@ def main():
             "bound": "vector_fp64", "pipe": "vector FP64 FMA (per-path rank-1 updates and GEMVs: no MFMA tile applies)",
             "kernel": dominant["kernel"], "achieved": dominant["tflops"], "peak": peak, "unit": "TFLOP/s",
             "frac": dominant["tflops"] / peak, "kernel_ms": dominant["ms"],
-            "traffic": TRAFFIC_BYTES.get(dominant["kernel"]),
+            "traffic": traffic_bytes(dominant["kernel"]),
+            # measured ceilings (independent FMAs only): the chip's best, and what one wave per SIMD, the regime of
+            # this workload's 1024 waves, can issue
+            "measured_peak": dict(peaks, unit="TFLOP/s"),
+            "frac_of_measured": (dominant["tflops"] / peaks["f64"]["8_waves_per_simd"]) if peaks["f64"]["8_waves_per_simd"] else None,
+            "frac_of_measured_one_wave_per_simd": (dominant["tflops"] / peaks["f64"]["1_waves_per_simd"])
+            if peaks["f64"]["1_waves_per_simd"] else None,
             "fwd_bwd_combined_frac": (r1.flops_fwd + r5.flops_bwd) / ((kms_f + kms_b) * 1e-3) / 1e12 / peak,
             # the whole synchronous step as timed above (launches and host waits included)
             "step_frac": (r1.flops_fwd + r5.flops_bwd) / (ms_per_step * 1e-3) / 1e12 / peak,

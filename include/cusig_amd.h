@@ -230,6 +230,10 @@ CUSIG_AMD_API uint64_t cusig_amd_sig_length(uint64_t dimension, uint64_t degree)
 CUSIG_AMD_API void cusig_amd_set_profiling(int enabled) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API float cusig_amd_last_kernel_ms(void) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API const char* cusig_amd_last_kernel_name(void) CUSIG_AMD_NOEXCEPT;
+/* Measured ceiling of the vector multiply-add pipe: runs a kernel of independent FMAs (float64 or float32, unpacked) with
+ * `waves_per_simd` (1..8) waves on every SIMD of the current device and stores the achieved TFLOP/s.  The benchmark
+ * reports it beside the nominal peak.  Synchronous; returns a status like the operators.  No counterpart in the reference. */
+CUSIG_AMD_API int cusig_amd_measure_fma_peak(int is_f64, int waves_per_simd, double* tflops) CUSIG_AMD_NOEXCEPT;
 /* Whether the last signature_cuda_* call on this thread stored a NaN or an infinity: 1 yes, 0 no, -1 not
  * reported (the call failed, or ran in stream-ordered mode, where the answer is not known at return).  The
  * kernels that store the result set the flag, so a caller who must warn about overflow (pysiglib/sig.py:299-311
