@@ -267,6 +267,11 @@ CUSIG_AMD_API void cusig_amd_set_point_fed(int on) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: number of time segments the backward sweep splits every path into (0 = automatic, 1 = never). */
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT;
+/* Test hook: 1 (default) lets single-precision backward sweeps of 33 and more augmented channels at degrees 3 .. 8 that
+ * the compiled instance table does not cover run the by-row reverse sweep (a wave holds its tile of top-level adjoints
+ * both by prefix and by letter, so no per-step reduction across lanes is left); 0 sends them to the general run-time
+ * kernels. */
+CUSIG_AMD_API void cusig_amd_set_rows_backward(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: how increments reach the waves: -1 automatic, 0 scalar loads, 1 LDS-staged where compiled. */
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only

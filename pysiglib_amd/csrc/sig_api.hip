@@ -24,6 +24,7 @@
 #include "../../include/cusig_amd.h"
 #include "sig_chen_adjoint.h"
 #include "sig_deep.h"
+#include "sig_rows.h"
 #include "sig_degree2.h"
 #include "sig_degree3.h"
 #include "sig_host.h"
@@ -433,6 +434,7 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
 // with the remaining segments.  That costs a segmented forward sweep, two chains of Chen products and one product
 // adjoint, all over (path, segment) rows.
 static Hook g_force_bwd_segments{0};   // tuning hook (0 = automatic)
+static Hook g_rows_backward{1};        // test hook: 0 = shapes beyond the table never take the by-row reverse sweep (sig_rows.hip)
 
 // g pieces are chosen by the same kind of model as for the forward sweep (fullest SIMD, `pair_rate`, lane_step(g) =
 // seconds per step of a lone wave).  The extra work is larger here: the segmented forward sweep (a third of the
@@ -1158,7 +1160,10 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         // lead-lag sweeps that skip the letters a step cannot move read a step's parity off its position in the
         // segment: segments start on even steps (a lead-lag path has an even number of steps)
         const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
-        int nseg = (arena || !ef || degree > uint64_t(kCombMaxLevels)) ? 1
+        // many channels beyond the compiled table: the by-row sweep, whole paths only (its launches fill the chip)
+        const bool by_rows = !arena && e->D <= 0 && g_rows_backward != 0 && g_force_tail == 0 &&
+                             rows_bwd_supported(sizeof(T), s.d_aug, degree) && rows_bwd_fits(s.d_aug, degree, batch);
+        int nseg = (arena || by_rows || !ef || degree > uint64_t(kCombMaxLevels)) ? 1
                    : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
                                               : choose_bwd_segments(
                                                     total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
@@ -1179,7 +1184,7 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         // Whole-path staged sweeps of plain narrow paths form the increments themselves while staging the points: no
         // pre-pass launch, so the accumulator comes from the pair that takes turns (cleared by the previous call).
         const KernelEntry* e_run = pick_variant(true, e, total_waves(geom, int64_t(batch) * nseg), sparse_ll);
-        const bool point_fed = !arena && nseg == 1 && e_run->staged && !time_aug && !lead_lag && e_run->D > 0 &&
+        const bool point_fed = !arena && !by_rows && nseg == 1 && e_run->staged && !time_aug && !lead_lag && e_run->D > 0 &&
                                e_run->D <= kPointFedMaxDim && g_point_fed != 0;
         T* inc = nullptr;
         T* dzinc = nullptr;
@@ -1259,11 +1264,16 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
             p.batch = int64_t(rows); p.nseg = nseg; p.lseg = lseg;
         }
         e = e_run;
-        const bool use_ll = sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
-        const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
+        const bool use_ll = !by_rows && sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
+        const std::string shown = by_rows ? "rows_bwd_f32_n" + std::to_string(degree)
+                                  : use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str(), !arena);
         if (turn) turn->dirty[mine] = dz_bytes;        // from here on the accumulator holds sums
-        SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
+        if (by_rows) {
+            if constexpr (sizeof(T) == 4) SIG_HIP(launch_rows_bwd_f32(p, int(degree)));
+        } else {
+            SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
+        }
         timer.stop();
         if (turn) {
             // the same launch clears what the other accumulator still holds: it is the next call's
@@ -1449,6 +1459,8 @@ CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) noexcept { if (g_test_h
 
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { if (g_test_hooks) g_force_bwd_segments = segments; }
 
+CUSIG_AMD_API void cusig_amd_set_rows_backward(int on) noexcept { if (g_test_hooks) g_rows_backward = on; }
+
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { if (g_test_hooks) g_force_staged = mode; }
 
 CUSIG_AMD_API void cusig_amd_force_wide_index(int enabled) noexcept { if (g_test_hooks) g_force_wide_index = enabled; }
@@ -1484,6 +1496,7 @@ CUSIG_AMD_API void cusig_amd_enable_test_hooks(int enabled) noexcept
     g_point_fed = 1;
     g_lead_lag_sparse = 1;
     g_force_bwd_segments = 0;
+    g_rows_backward = 1;
     g_force_staged = -1;
     g_force_wide_index = 0;
     g_chen_adjoint_mode = 0;

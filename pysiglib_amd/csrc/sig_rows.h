@@ -1,0 +1,19 @@
+// Reverse sweep for many channels (more than 32) at degrees beyond the compiled instance table; defined in sig_rows.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sig_registry.h"
+
+namespace sigamd {
+
+// whether launch_rows_bwd serves (element size, augmented dimension, degree)
+bool rows_bwd_supported(size_t elem_bytes, uint64_t d, uint64_t degree);
+
+// whether a launch for `batch` paths fits the grid limits (to be checked before anything is enqueued)
+bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch);
+
+// whole-path reverse sweeps (p.nseg must be 1, p.inc holds increments); p.d is the augmented dimension
+hipError_t launch_rows_bwd_f32(const BwdParams& p, int degree);
+
+}  // namespace sigamd

@@ -1,0 +1,357 @@
+// Reverse signature sweep for paths of many channels (33 and more) at degrees the compiled instance table does not
+// reach, single precision.
+//
+// Arithmetic: siglib/cpsig/cp_signature.h:1137-1187 (per step: un-multiply the state by exp(-z), pull the adjoint back
+// through the step, emit the increment gradient), regrouped per word as in sig_tree.h with a subtree of depth 1: a
+// lane owns a word prefix p of N - 1 letters, the chain S_1[p_1] .. S_{N-1}[p], and the top-level adjoints G[p, a].
+//
+// What bounds such sweeps is the sum over the prefixes: the gradient of letter a in a step is
+//   dz[a] += sum_p G[p, a] * U[p]          (U[p]: Horner value of p towards the top level, one per lane)
+// which lanes that each hold one prefix can only form through a reduction across the wave, once per letter and step.
+// The top-level adjoints never change during the sweep, so a wave holds its tile of them twice:
+//   by prefix:  lane = prefix, registers over the letters:  red[p] = sum_a G[p, a] * z[a] stays inside the lane
+//               (z[a] wave-uniform, from scalar loads);
+//   by letter:  lane = letter, registers over the prefixes: dz[a] = sum_p G[p, a] * U[p] stays inside the lane too,
+//               U[p] handed from lane p to all lanes through LDS.
+// No reduction is left but the one over the waves, which the atomic adds into the gradient rows perform.
+//
+// Tile of a wave: the 64 prefixes (r, 64 blk + lane) that share their first N - 2 letters r, times the 64 letters
+// [64 ga, 64 ga + 64); paths of d channels have ceil(d / 64) values of blk and of ga.  The first N - 2 prefix letters
+// are wave-uniform: their increments come from scalar loads and their gradient pieces need one sum over the wave; the
+// last prefix letter differs from lane to lane and its pieces go to the gradient row directly.  The chain and its
+// adjoint run through the code of the compiled kernels (Tree / TreeAdj with a one-letter subtree whose adjoint is 1 and
+// whose "increment" is red[p]: the pullback then sees exactly the contraction it would have formed itself).
+#include <hip/hip_runtime.h>
+
+#include "sig_rows.h"
+#include "sig_launch.h"
+
+namespace sigamd {
+
+namespace {
+
+constexpr int kRowLetters = 64;
+constexpr int kRowsMinDim = 33;         // below, the compiled table or the other run-time kernels are faster
+constexpr int kRowsMinDegree = 3;
+constexpr int kRowsMaxDegree = 8;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+// sum over the 64 lanes, valid in every lane
+__device__ __forceinline__ float wave_sum_rows(float v)
+{
+    v = dpp_add<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+    v = dpp_add<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+    v = dpp_add<0x141>(v);      // row_half_mirror
+    v = dpp_add<0x140>(v);      // row_mirror: every lane holds the sum of its row of 16
+    const float s0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float s1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float s2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float s3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (s0 + s1) + (s2 + s3);
+}
+
+constexpr int kRowsWaves = 8;                       // waves per block: one block fills a CU at two waves per SIMD
+constexpr int kRowsBlock = kRowsWaves * kWave;
+constexpr int kRowsMaxChunk = 4;                    // steps a block collects before it adds them to the gradient
+constexpr int kRowsTileElems = 4096;                // per buffer: chunk steps * d stays below this (32 KB for both buffers)
+constexpr int kRowsPriv = 2 * kRowLetters;          // a wave's own words per step: by-letter sums, last-prefix-letter pieces
+
+inline int rows_chunk_steps(int d)
+{
+    const int c = kRowsTileElems / d;
+    return c < 1 ? 1 : c > kRowsMaxChunk ? kRowsMaxChunk : c;
+}
+
+template <int N>
+__global__ __launch_bounds__(kRowsBlock) void rows_bwd_kernel(
+    const float* __restrict__ inc, const float* __restrict__ sig, const float* __restrict__ gsig,
+    float* __restrict__ dzinc, int64_t batch, int64_t L, int d, int64_t sig_stride, int scalar, int64_t rows /* d^(N-2) */,
+    int nblk /* ceil(d / 64) */, int64_t blocks_per_path, int chunk /* rows_chunk_steps(d) */)
+{
+    using T = float;
+    using Tr = Tree<T, -1, N, 1, 1>;
+    using Ad = TreeAdj<T, -1, N, 1, 1>;
+    constexpr int M = N - 1;
+    static_assert(M >= 2, "degree 3 and up");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
+
+    // ---- the wave's tile (all wave-uniform) ------------------------------
+    // The waves of a block belong to one path: they share the block's gradient tile.  Surplus waves of a path's last
+    // block shadow its last tile with all adjoints zero, so that every wave of a block reaches every barrier.
+    const int64_t per_path = rows * nblk * nblk;
+    const int64_t b = int64_t(blockIdx.x) / blocks_per_path;
+    int64_t w = (int64_t(blockIdx.x) - b * blocks_per_path) * kRowsWaves + wib;
+    const bool valid = w < per_path;
+    if (!valid) w = per_path - 1;
+    const int ga = int(w % nblk);
+    w /= nblk;
+    const int blk = int(w % nblk);
+    const int64_t r = w / nblk;
+    int pu[M - 1];                          // the shared prefix letters
+    {
+        int64_t q = r;
+#pragma unroll
+        for (int l = M - 2; l >= 0; --l) {
+            pu[l] = int(q % d);
+            q /= d;
+        }
+    }
+    const int a0 = ga * kRowLetters;
+    const int last = blk * kRowLetters + lane;      // this lane's last prefix letter
+    const bool active = valid && last < d;
+    const int lastc = last < d ? last : d - 1;      // idle lanes shadow a valid lane: every load stays in bounds
+    const int64_t q = r * d + lastc;
+
+    // ---- state and upstream gradient ------------------------------------
+    Tr S;
+    Ad A;
+    const T* srow = sig + b * sig_stride;
+    const T* grow = gsig + b * sig_stride;
+    int64_t leaf_off;
+    {
+        int64_t off = scalar ? 1 : 0, size = d;      // start and size of level l
+#pragma unroll
+        for (int l = 1; l <= M; ++l) {
+            int64_t span = 1;                        // d^(M - l): prefixes of full length below one level-l node
+#pragma unroll
+            for (int i = l; i < M; ++i) span *= d;
+            const int64_t idx = off + q / span;
+            // a chain node's adjoint is seeded in one lane only: the recursion is linear in the adjoint
+            const bool owner = active && ga == 0 && (q % span == 0);
+            S.c[l - 1] = srow[idx];
+            A.gc[l - 1] = owner ? grow[idx] : T(0);
+            off += size;
+            size *= d;
+        }
+        leaf_off = off;
+    }
+    // by prefix: this lane's prefix, the tile's letters
+    T gp[kRowLetters];
+    {
+        const T* g = grow + leaf_off + q * d + a0;
+#pragma unroll
+        for (int a = 0; a < kRowLetters; ++a) {
+            const bool ok = active && a0 + a < d;
+            const T v = g[ok ? a : 0];
+            gp[a] = ok ? v : T(0);
+        }
+    }
+    A.gs[0] = T(1);
+    S.s[0] = T(0);
+    // by letter: this lane's letter, the tile's prefixes
+    const bool letter_ok = a0 + lane < d;
+    T gt[kWave];
+    {
+        const bool lok = valid && letter_ok;
+        const T* g = grow + leaf_off + (r * d + int64_t(blk) * kRowLetters) * d + (lok ? a0 + lane : 0);
+#pragma unroll
+        for (int j = 0; j < kWave; ++j) {
+            const bool ok = lok && blk * kRowLetters + j < d;
+            const T v = g[ok ? int64_t(j) * d : 0];
+            gt[j] = ok ? v : T(0);
+        }
+    }
+
+    // ---- the sweep ---------------------------------------------------------
+    // Increments are [batch][L + 2][d] with a zero row at either end of a path.  The tile's slice of a step's row is
+    // wave-uniform and arrives through scalar loads, requested one step ahead; a slice that reaches past the row reads
+    // on into the next row of the same path (at most 63 elements, fewer than a row holds) and meets adjoints that are
+    // zero.  The Horner values U[p] go from the by-prefix lanes to the by-letter lanes through the wave's LDS slot: one
+    // write, then every lane reads all of it (same address in every lane: a broadcast).
+    //
+    // Gradient pieces of a step: the by-letter sums and the pieces of the last prefix letter (one per lane each) go to
+    // words of the wave's own in LDS with plain writes (a float LDS atomic of a full wave costs about 500 cycles here);
+    // the few pieces of the shared prefix letters are added to the block's row tile with LDS atomics.  After `chunk`
+    // steps the whole block sums, per step and letter, the tile and the words of the waves that cover the letter, adds
+    // the sum to the gradient row and clears the tile, while the waves already fill the other buffer: one barrier per
+    // chunk.
+    extern __shared__ float rows_lds[];
+    __shared__ __attribute__((aligned(16))) T ul_all[kRowsWaves][kWave];
+    __shared__ int wave_a0[kRowsWaves], wave_l0[kRowsWaves];
+    T* ul = ul_all[wib];
+    const int tile_elems = chunk * d;                               // per buffer
+    const int priv_elems = chunk * kRowsWaves * kRowsPriv;          // per buffer
+    T* tile = rows_lds;                                             // [2][chunk][d]
+    T* priv = rows_lds + 2 * tile_elems;                            // [2][chunk][wave][kRowsPriv]
+    for (int e = threadIdx.x; e < 2 * tile_elems; e += kRowsBlock) tile[e] = T(0);
+    if (lane == 0) {
+        wave_a0[wib] = a0;
+        wave_l0[wib] = blk * kRowLetters;
+    }
+    __syncthreads();
+
+    const T* zrow = inc + (b * (L + 2) + L) * d;        // row of the last step
+    typename Tr::Inc in;
+    in.z[0] = T(0);
+    T zs[kRowLetters];
+    T pz_next[M];
+    auto fetch = [&](const T* row) {
+#pragma unroll
+        for (int l = 0; l < M - 1; ++l) pz_next[l] = row[pu[l]];
+        pz_next[M - 1] = row[lastc];
+#pragma unroll
+        for (int a = 0; a < kRowLetters; ++a) zs[a] = row[a0 + a];
+    };
+    fetch(zrow);
+    int buf = 0, sidx = 0;
+    int64_t t_first = L - 1;                // step held by row 0 of the current buffer
+    for (int64_t t = L - 1; t >= 0; --t) {
+#pragma unroll
+        for (int l = 0; l < M; ++l) in.pz[l] = pz_next[l];
+
+        // state before the step, and the prefix's Horner value towards the top level: it does not depend on the
+        // adjoints, so it is on its way through LDS while the contraction with the letters runs
+        typename Tr::Chain unmul;
+        S.template fwd_step<AllLetters, true>(in, &unmul);
+        if constexpr (Tr::kLockstep) {
+            typename Tr::Chain ch;
+            S.template chain_all<false>(in, ch, &unmul);
+            ul[lane] = ch.u[N][M - 1];
+        } else {
+            T u[M];
+            S.template chain_u<N, M>(in, u);
+            ul[lane] = u[M - 1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // by prefix: red = sum over the tile's letters of G[p, a] * z[a]
+        T red0 = T(0), red1 = T(0);
+#pragma unroll
+        for (int a = 0; a < kRowLetters; a += 2) {
+            red0 = fmadd(gp[a], zs[a], red0);
+            red1 = fmadd(gp[a + 1], zs[a + 1], red1);
+        }
+        in.zs[0] = red0 + red1;
+        __builtin_amdgcn_sched_barrier(0);
+        // the step before this one (step 0 fetches the zero row in front of the path)
+        zrow -= d;
+        fetch(zrow);
+        __builtin_amdgcn_sched_barrier(0);
+
+        typename Ad::DInc dz;
+        dz.dj[0] = T(0);
+        dz.da[0] = T(0);
+#pragma unroll
+        for (int l = 0; l < M; ++l) dz.dc[l] = T(0);
+        A.template pullback<-1, AllLetters>(S, in, dz, Tr::kLockstep ? &unmul : nullptr);
+
+        // the shared prefix letters: one sum over the wave each
+        T mine = T(0);
+        int where = 0;
+#pragma unroll
+        for (int l = 0; l < M - 1; ++l) {
+            const T s = wave_sum_rows(dz.dc[l]);
+            if (lane == l) {
+                mine = s;
+                where = pu[l];
+            }
+        }
+        if (lane < M - 1) lds_add_shared(&tile[(buf * chunk + sidx) * d + where], mine);
+
+        // by letter: dz[a] = sum over the tile's prefixes of G[p, a] * U[p]
+        T acc0 = T(0), acc1 = T(0);
+        const float4* us = reinterpret_cast<const float4*>(ul);
+#pragma unroll
+        for (int jb = 0; jb < kWave; jb += 16) {
+            float4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = us[jb / 4 + i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc0 = fmadd(gt[jb + 4 * i], v[i].x, acc0);
+                acc1 = fmadd(gt[jb + 4 * i + 1], v[i].y, acc1);
+                acc0 = fmadd(gt[jb + 4 * i + 2], v[i].z, acc0);
+                acc1 = fmadd(gt[jb + 4 * i + 3], v[i].w, acc1);
+            }
+        }
+        // idle lanes and shadow waves hold zero adjoints: what they write is zero
+        T* mine_row = priv + ((buf * chunk + sidx) * kRowsWaves + wib) * kRowsPriv;
+        mine_row[lane] = acc0 + acc1;
+        mine_row[kRowLetters + lane] = dz.dc[M - 1];
+
+        if (++sidx == chunk || t == 0) {
+            __syncthreads();
+            // rows 0 .. sidx - 1 of the buffer hold the steps t_first, t_first - 1, ..
+            T* src = tile + buf * tile_elems;
+            const T* pr = priv + buf * priv_elems;
+            T* out = dzinc + (b * L + t_first) * d;
+            for (int e = threadIdx.x; e < sidx * d; e += kRowsBlock) {
+                const int row = e / d, a = e - row * d;
+                T v = src[e];
+                src[e] = T(0);
+#pragma unroll 1
+                for (int k = 0; k < kRowsWaves; ++k) {
+                    const T* wr = pr + (row * kRowsWaves + k) * kRowsPriv;
+                    const unsigned ia = unsigned(a - wave_a0[k]), il = unsigned(a - wave_l0[k]);
+                    if (ia < unsigned(kRowLetters)) v += wr[ia];
+                    if (il < unsigned(kRowLetters)) v += wr[kRowLetters + il];
+                }
+                dev_add(&out[a - int64_t(row) * d], v);      // row `row` lies `row` gradient rows before t_first
+            }
+            t_first -= sidx;
+            sidx = 0;
+            buf ^= 1;
+        }
+    }
+}
+
+template <int N>
+hipError_t launch_rows(const BwdParams& p)
+{
+    const int nblk = (p.d + kRowLetters - 1) / kRowLetters;
+    int64_t rows = 1;
+    for (int i = 0; i < N - 2; ++i) rows *= p.d;
+    const int64_t per_path = rows * nblk * nblk;
+    const int64_t blocks_per_path = (per_path + kRowsWaves - 1) / kRowsWaves;
+    const int64_t blocks = p.batch * blocks_per_path;
+    if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
+    const int chunk = rows_chunk_steps(p.d);
+    const size_t lds = size_t(2) * chunk * (size_t(p.d) + kRowsWaves * kRowsPriv) * sizeof(float);
+    if (lds > kMaxDynLds) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((rows_bwd_kernel<N>), dim3(unsigned(blocks)), dim3(kRowsBlock), lds, p.stream,
+                       static_cast<const float*>(p.inc), static_cast<const float*>(p.sig), static_cast<const float*>(p.gsig),
+                       static_cast<float*>(p.dzinc), p.batch, p.L, p.d, p.sig_stride, p.scalar, rows, nblk, blocks_per_path, chunk);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool rows_bwd_supported(size_t elem_bytes, uint64_t d, uint64_t degree)
+{
+    return elem_bytes == 4 && d >= uint64_t(kRowsMinDim) && d <= uint64_t(kRowsTileElems) && degree >= uint64_t(kRowsMinDegree) &&
+           degree <= uint64_t(kRowsMaxDegree);
+}
+
+bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch)
+{
+    const uint64_t nblk = (d + kRowLetters - 1) / kRowLetters;
+    unsigned __int128 per_path = (unsigned __int128)nblk * nblk;
+    for (uint64_t i = 0; i + 2 < degree; ++i) {
+        per_path *= d;
+        if (per_path > (unsigned __int128)kMaxGridX * kRowsWaves) return false;
+    }
+    const unsigned __int128 blocks = (per_path + kRowsWaves - 1) / kRowsWaves * batch;
+    return blocks >= 1 && blocks <= (unsigned __int128)kMaxGridX;
+}
+
+hipError_t launch_rows_bwd_f32(const BwdParams& p, int degree)
+{
+    if (p.nseg != 1 || p.from_points || p.d < kRowsMinDim) return hipErrorInvalidConfiguration;
+    switch (degree) {
+        case 3: return launch_rows<3>(p);
+        case 4: return launch_rows<4>(p);
+        case 5: return launch_rows<5>(p);
+        case 6: return launch_rows<6>(p);
+        case 7: return launch_rows<7>(p);
+        case 8: return launch_rows<8>(p);
+        default: return hipErrorInvalidConfiguration;
+    }
+}
+
+}  // namespace sigamd

@@ -388,10 +388,13 @@ struct TreeAdj {
     //   dj[j]  -> letter j            (compile-time letters, subtree depth >= 2)
     //   da[a]  -> letter a0 + a       (subtree depth 1)
     //   dc[l]  -> letter p_{l+1}      (chain)
+    // top: the prefix word's Horner value towards the top level (depth-1 subtrees only): da[a] = gs[a] * top, for
+    // sweeps that form these products elsewhere
     struct DInc {
         T dj[DD];
         T da[K];
         T dc[M];
+        T top;
     };
     // depth-1 pieces can join dj in registers when the depth-1 letters are compile-time constants and dj is in use
     template <int G0>
@@ -412,6 +415,7 @@ struct TreeAdj {
         constexpr int NCH = (E == 1) ? K : DD;
         const T sc = rcp<T>(I - E + 1);
         const T v = (I - E + 1 == 1) ? upar : upar * sc;
+        if constexpr (TAIL == 1) dz.top = v;
         T red = T(0);
         T uc[NCH];
         if constexpr (E < I) {

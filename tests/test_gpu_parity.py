@@ -696,6 +696,45 @@ def test_extreme_shapes(P, oracle, shape, dtype):
     assert bwd_rel_err(got_b, ref_b) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("shape,aug,scalar_term", [
+    ((1, 5, 64, 4), {}, False),                                     # one tile of 64 prefixes x 64 letters per word row
+    ((2, 6, 49, 4), {}, True), ((2, 4, 52, 4), dict(time_aug=True), False),       # partly filled tiles
+    ((2, 5, 70, 4), {}, False), ((1, 4, 130, 3), {}, True),         # several tiles per row; degree 3 beyond the table
+    ((3, 6, 25, 4), dict(lead_lag=True, time_aug=True), False),     # 51 augmented channels
+    ((2, 4, 33, 5), {}, False),                                     # chains of four letters
+])
+def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
+    """Single-precision backward of many channels beyond the compiled table (sig_rows.hip) against the oracle, and the
+    general run-time kernels on the same input (hook off) as a second opinion on what the dispatch covers."""
+    import ctypes
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_set_rows_backward.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_rows_backward.restype = None
+    L.CUSIG.cusig_amd_last_kernel_name.restype = ctypes.c_char_p
+    b, length, d, deg = shape
+    rng = np.random.default_rng(b * 100000 + length * 1000 + d * 10 + deg)
+    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (1.5 / np.sqrt(d))).astype(np.float32)
+    ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+    g = rng.standard_normal(ref.shape).astype(np.float32)
+    want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+    ref32 = ref.astype(np.float32)
+    try:
+        L.CUSIG.cusig_amd_set_profiling(1)
+        got = P.sig_backprop(dev(x), dev(ref32), dev(g), deg, **aug).cpu().numpy()
+        assert L.CUSIG.cusig_amd_last_kernel_name().decode() == "rows_bwd_f32_n%d" % deg
+        L.CUSIG.cusig_amd_set_rows_backward(0)
+        other = P.sig_backprop(dev(x), dev(ref32), dev(g), deg, **aug).cpu().numpy()
+        assert not L.CUSIG.cusig_amd_last_kernel_name().decode().startswith("rows_bwd")
+    finally:
+        L.CUSIG.cusig_amd_set_rows_backward(1)
+        L.CUSIG.cusig_amd_set_profiling(0)
+    assert bwd_rel_err(got, want) <= TOL[np.float32], bwd_rel_err(got, want)
+    assert bwd_rel_err(other, want) <= TOL[np.float32], bwd_rel_err(other, want)
+    # double precision keeps the general kernels
+    assert bwd_rel_err(P.sig_backprop(dev(x.astype(np.float64)), dev(ref.astype(np.float64)), dev(g.astype(np.float64)),
+                                      deg, **aug).cpu().numpy(), want) <= TOL[np.float32]
+
+
 @pytest.mark.parametrize("shape", [(3, 9, 2, 5), (2, 7, 2, 9), (5, 12, 2, 12), (2, 6, 3, 4), (3, 10, 3, 7), (2, 9, 3, 10),
                                    (4, 8, 4, 3), (2, 11, 4, 6), (70, 5, 2, 6), (1, 300, 3, 5)])
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
