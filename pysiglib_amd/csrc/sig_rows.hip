@@ -28,8 +28,6 @@
 
 namespace sigamd {
 
-namespace {
-
 constexpr int kRowLetters = 64;
 constexpr int kRowsMinDim = 33;         // below, the compiled table or the other run-time kernels are faster
 constexpr int kRowsMinDegree = 3;
@@ -55,25 +53,32 @@ __device__ __forceinline__ float wave_sum_rows(float v)
     return (s0 + s1) + (s2 + s3);
 }
 
-constexpr int kRowsWaves = 8;                       // waves per block: one block fills a CU at two waves per SIMD
-constexpr int kRowsBlock = kRowsWaves * kWave;
+// Waves per block; a block fills a CU.  Degrees 3 and 4 fit 168 vector registers (three waves per SIMD: 7.0 ms against 7.7 ms
+// for 16 paths of 200 steps, 64 channels, degree 4); the longer chains above need more and run two waves per SIMD (a
+// third would spill: degree 5 9.4 -> 10.7 ms).
+template <int N>
+constexpr int kRowsWavesOf = N <= 4 ? 12 : 8;
+constexpr int kRowsMaxWaves = 12;
 constexpr int kRowsMaxChunk = 4;                    // steps a block collects before it adds them to the gradient
-constexpr int kRowsTileElems = 4096;                // per buffer: chunk steps * d stays below this (32 KB for both buffers)
+constexpr int kRowsMaxDim = 4096;                   // a row of the tile per step must leave room for the waves' words
 constexpr int kRowsPriv = 2 * kRowLetters;          // a wave's own words per step: by-letter sums, last-prefix-letter pieces
 
-inline int rows_chunk_steps(int d)
+// both buffers of the row tile and of the waves' own words stay within 64 KB of LDS
+inline int rows_chunk_steps(int d, int waves)
 {
-    const int c = kRowsTileElems / d;
+    const int c = int(kMaxDynLds / (2 * sizeof(float))) / (d + waves * kRowsPriv);
     return c < 1 ? 1 : c > kRowsMaxChunk ? kRowsMaxChunk : c;
 }
 
 template <int N>
-__global__ __launch_bounds__(kRowsBlock) void rows_bwd_kernel(
+__global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     const float* __restrict__ inc, const float* __restrict__ sig, const float* __restrict__ gsig,
     float* __restrict__ dzinc, int64_t batch, int64_t L, int d, int64_t sig_stride, int scalar, int64_t rows /* d^(N-2) */,
-    int nblk /* ceil(d / 64) */, int64_t blocks_per_path, int chunk /* rows_chunk_steps(d) */)
+    int nblk /* ceil(d / 64) */, int64_t blocks_per_path, int chunk /* rows_chunk_steps */)
 {
     using T = float;
+    constexpr int kRowsWaves = kRowsWavesOf<N>;
+    constexpr int kRowsBlock = kRowsWaves * kWave;
     using Tr = Tree<T, -1, N, 1, 1>;
     using Ad = TreeAdj<T, -1, N, 1, 1>;
     constexpr int M = N - 1;
@@ -269,6 +274,7 @@ __global__ __launch_bounds__(kRowsBlock) void rows_bwd_kernel(
                 acc0 = fmadd(gt[jb + 4 * i + 2], v[i].z, acc0);
                 acc1 = fmadd(gt[jb + 4 * i + 3], v[i].w, acc1);
             }
+            __builtin_amdgcn_sched_barrier(0);      // sixteen values in flight at a time: registers
         }
         // idle lanes and shadow waves hold zero adjoints: what they write is zero
         T* mine_row = priv + ((buf * chunk + sidx) * kRowsWaves + wib) * kRowsPriv;
@@ -307,24 +313,23 @@ hipError_t launch_rows(const BwdParams& p)
     const int nblk = (p.d + kRowLetters - 1) / kRowLetters;
     int64_t rows = 1;
     for (int i = 0; i < N - 2; ++i) rows *= p.d;
+    constexpr int kRowsWaves = kRowsWavesOf<N>;
     const int64_t per_path = rows * nblk * nblk;
     const int64_t blocks_per_path = (per_path + kRowsWaves - 1) / kRowsWaves;
     const int64_t blocks = p.batch * blocks_per_path;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
-    const int chunk = rows_chunk_steps(p.d);
+    const int chunk = rows_chunk_steps(p.d, kRowsWaves);
     const size_t lds = size_t(2) * chunk * (size_t(p.d) + kRowsWaves * kRowsPriv) * sizeof(float);
     if (lds > kMaxDynLds) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((rows_bwd_kernel<N>), dim3(unsigned(blocks)), dim3(kRowsBlock), lds, p.stream,
+    hipLaunchKernelGGL((rows_bwd_kernel<N>), dim3(unsigned(blocks)), dim3(kRowsWaves * kWave), lds, p.stream,
                        static_cast<const float*>(p.inc), static_cast<const float*>(p.sig), static_cast<const float*>(p.gsig),
                        static_cast<float*>(p.dzinc), p.batch, p.L, p.d, p.sig_stride, p.scalar, rows, nblk, blocks_per_path, chunk);
     return hipGetLastError();
 }
 
-}  // namespace
-
 bool rows_bwd_supported(size_t elem_bytes, uint64_t d, uint64_t degree)
 {
-    return elem_bytes == 4 && d >= uint64_t(kRowsMinDim) && d <= uint64_t(kRowsTileElems) && degree >= uint64_t(kRowsMinDegree) &&
+    return elem_bytes == 4 && d >= uint64_t(kRowsMinDim) && d <= uint64_t(kRowsMaxDim) && degree >= uint64_t(kRowsMinDegree) &&
            degree <= uint64_t(kRowsMaxDegree);
 }
 
@@ -334,9 +339,9 @@ bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch)
     unsigned __int128 per_path = (unsigned __int128)nblk * nblk;
     for (uint64_t i = 0; i + 2 < degree; ++i) {
         per_path *= d;
-        if (per_path > (unsigned __int128)kMaxGridX * kRowsWaves) return false;
+        if (per_path > (unsigned __int128)kMaxGridX * 8) return false;
     }
-    const unsigned __int128 blocks = (per_path + kRowsWaves - 1) / kRowsWaves * batch;
+    const unsigned __int128 blocks = (per_path + 7) / 8 * batch;      // at the smaller of the two block sizes
     return blocks >= 1 && blocks <= (unsigned __int128)kMaxGridX;
 }
 
