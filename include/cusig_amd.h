@@ -304,6 +304,9 @@ CUSIG_AMD_API void cusig_amd_force_deep(int enabled) CUSIG_AMD_NOEXCEPT;
  * them through LDS (the path taken anyway when a chunk of all channels does not fit). */
 CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: with a forced partition, shapes served by a run-time-dimension kernel take its wide-layout variant. */
+/* Tuning hook: nonzero makes every shape run the run-time-dimension kernels (and the by-row reverse sweep where it
+ * applies), as if the shape had no compiled instance: the yardstick for deciding which instances earn their place. */
+CUSIG_AMD_API void cusig_amd_ignore_instance_table(int on) CUSIG_AMD_NOEXCEPT;
 CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: prefer the compiled lane partition (tail, k) where a shape has several; tail = 0 restores
  * the defaults.  Not thread-safe; meant for offline sweeps. */

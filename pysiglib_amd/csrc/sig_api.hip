@@ -64,6 +64,7 @@ using Hook = std::atomic<int>;
 static Hook g_test_hooks{0};
 // tuning hook: when set (tail > 0), prefer the compiled partition with this (tail, k)
 static Hook g_force_tail{0}, g_force_k{0};
+static Hook g_ignore_table{0};          // tuning hook: every shape runs the run-time-dimension kernels, as if it had no compiled instance
 static Hook g_force_run_time_wide{0};   // with a forced partition: take the run-time-dimension kernel in the wide layout
 
 static const Table& table()
@@ -131,7 +132,7 @@ static const KernelEntry* find_entry(bool backward, bool f64, uint64_t d, uint64
     const auto& m = backward ? table().bwd : table().fwd;
     if (d <= 0x7fffffff && degree <= 0x7fffffff) {
         auto it = m.find(std::make_tuple(int(f64), int(d), int(degree)));
-        const bool run_time = it == m.end();
+        const bool run_time = it == m.end() || g_ignore_table != 0;
         if (run_time) it = m.find(std::make_tuple(int(f64), 0, int(degree)));
         if (it != m.end() && !it->second.empty()) {
             if (g_force_tail > 0) {
@@ -1161,8 +1162,12 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         // segment: segments start on even steps (a lead-lag path has an even number of steps)
         const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
         // many channels beyond the compiled table: the by-row sweep, whole paths only (its launches fill the chip)
-        const bool by_rows = !arena && e->D <= 0 && g_rows_backward != 0 && g_force_tail == 0 &&
-                             rows_bwd_supported(sizeof(T), s.d_aug, degree) && rows_bwd_fits(s.d_aug, degree, batch);
+        // (also where an instance would lose: measured at 48 .. 128 channels, degrees 3 and 4, the by-row sweep runs
+        // 1.1-4x faster than compiled single-precision instances and 1-12x faster than double-precision ones; the
+        // instance table leaves these backward shapes out)
+        const bool rows_win = e->D <= 0 || s.d_aug >= 48;
+        const bool by_rows = !arena && rows_win && g_rows_backward != 0 && g_force_tail == 0 &&
+                             rows_bwd_supported(sizeof(T), s.d_aug, degree) && rows_bwd_fits(sizeof(T), s.d_aug, degree, batch);
         int nseg = (arena || by_rows || !ef || degree > uint64_t(kCombMaxLevels)) ? 1
                    : g_force_bwd_segments > 0 ? int(std::min<uint64_t>(uint64_t(g_force_bwd_segments), s.L))
                                               : choose_bwd_segments(
@@ -1265,12 +1270,12 @@ static void sig_backprop_impl(const T* path, T* out, const T* sig_derivs, const 
         }
         e = e_run;
         const bool use_ll = !by_rows && sparse_ll && e->bwd_lead_lag && (s.L & 1) == 0;
-        const std::string shown = by_rows ? "rows_bwd_f32_n" + std::to_string(degree)
+        const std::string shown = by_rows ? std::string(sizeof(T) == 8 ? "rows_bwd_f64_n" : "rows_bwd_f32_n") + std::to_string(degree)
                                   : use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str(), !arena);
         if (turn) turn->dirty[mine] = dz_bytes;        // from here on the accumulator holds sums
         if (by_rows) {
-            if constexpr (sizeof(T) == 4) SIG_HIP(launch_rows_bwd_f32(p, int(degree)));
+            SIG_HIP(launch_rows_bwd<T>(p, int(degree)));
         } else {
             SIG_HIP(use_ll ? e->bwd_lead_lag(p) : e->bwd(p));
         }
@@ -1478,6 +1483,7 @@ CUSIG_AMD_API void cusig_amd_force_deep(int enabled) noexcept { if (g_test_hooks
 
 CUSIG_AMD_API void cusig_amd_set_degree2_staged(int enabled) noexcept { if (g_test_hooks) g_degree2_staged = enabled; }
 
+CUSIG_AMD_API void cusig_amd_ignore_instance_table(int on) noexcept { if (g_test_hooks) g_ignore_table = on; }
 CUSIG_AMD_API void cusig_amd_force_run_time_wide(int enabled) noexcept { if (g_test_hooks) g_force_run_time_wide = enabled; }
 
 CUSIG_AMD_API void cusig_amd_force_partition(int tail, int k) noexcept
@@ -1506,6 +1512,7 @@ CUSIG_AMD_API void cusig_amd_enable_test_hooks(int enabled) noexcept
     g_force_deep = 0;
     g_degree2_staged = 1;
     g_force_run_time_wide = 0;
+    g_ignore_table = 0;
     g_force_tail = 0;
     g_force_k = 0;
     g_alloc_limit = 0;

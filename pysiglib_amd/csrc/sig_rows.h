@@ -11,9 +11,10 @@ namespace sigamd {
 bool rows_bwd_supported(size_t elem_bytes, uint64_t d, uint64_t degree);
 
 // whether a launch for `batch` paths fits the grid limits (to be checked before anything is enqueued)
-bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch);
+bool rows_bwd_fits(size_t elem_bytes, uint64_t d, uint64_t degree, uint64_t batch);
 
 // whole-path reverse sweeps (p.nseg must be 1, p.inc holds increments); p.d is the augmented dimension
-hipError_t launch_rows_bwd_f32(const BwdParams& p, int degree);
+template <typename T>
+hipError_t launch_rows_bwd(const BwdParams& p, int degree);
 
 }  // namespace sigamd

@@ -1,5 +1,5 @@
-// Reverse signature sweep for paths of many channels (33 and more) at degrees the compiled instance table does not
-// reach, single precision.
+// Reverse signature sweep for paths of many channels (33 and more) at degrees 3 .. 8, where the compiled instance table
+// has no faster kernel.
 //
 // Arithmetic: siglib/cpsig/cp_signature.h:1137-1187 (per step: un-multiply the state by exp(-z), pull the adjoint back
 // through the step, emit the increment gradient), regrouped per word as in sig_tree.h with a subtree of depth 1: a
@@ -15,8 +15,11 @@
 //               U[p] handed from lane p to all lanes through LDS.
 // No reduction is left but the one over the waves, which the atomic adds into the gradient rows perform.
 //
-// Tile of a wave: the 64 prefixes (r, 64 blk + lane) that share their first N - 2 letters r, times the 64 letters
-// [64 ga, 64 ga + 64); paths of d channels have ceil(d / 64) values of blk and of ga.  The first N - 2 prefix letters
+// Tile of a wave: the 64 prefixes (r, 64 blk + lane) that share their first N - 2 letters r, times the KB letters
+// [KB ga, KB ga + KB), KB = 64 in single and 32 in double precision (the two copies of the tile take 128 registers
+// either way); paths of d channels have ceil(d / 64) values of blk and ceil(d / KB) of ga.  With 32 letters the
+// by-letter copy is held by lane = (half h, letter): lanes of half h cover the prefixes 32 h .. 32 h + 31, and the two
+// halves' sums meet when the block adds its pieces up.  The first N - 2 prefix letters
 // are wave-uniform: their increments come from scalar loads and their gradient pieces need one sum over the wave; the
 // last prefix letter differs from lane to lane and its pieces go to the gradient row directly.  The chain and its
 // adjoint run through the code of the compiled kernels (Tree / TreeAdj with a one-letter subtree whose adjoint is 1 and
@@ -28,56 +31,68 @@
 
 namespace sigamd {
 
-constexpr int kRowLetters = 64;
+template <typename T>
+constexpr int kRowLettersOf = sizeof(T) == 8 ? 32 : 64;
 constexpr int kRowsMinDim = 33;         // below, the compiled table or the other run-time kernels are faster
 constexpr int kRowsMinDegree = 3;
 constexpr int kRowsMaxDegree = 8;
 
 template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v)
+__device__ __forceinline__ float dpp_moved(float v)
 {
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
-    return v + __int_as_float(moved);
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_moved(double v)
+{
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+__device__ __forceinline__ double lane_value(double v, int l)
+{
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), l), __builtin_amdgcn_readlane(__double2loint(v), l));
 }
 // sum over the 64 lanes, valid in every lane
-__device__ __forceinline__ float wave_sum_rows(float v)
+template <typename T>
+__device__ __forceinline__ T wave_sum_rows(T v)
 {
-    v = dpp_add<0xB1>(v);       // quad_perm [1, 0, 3, 2]
-    v = dpp_add<0x4E>(v);       // quad_perm [2, 3, 0, 1]
-    v = dpp_add<0x141>(v);      // row_half_mirror
-    v = dpp_add<0x140>(v);      // row_mirror: every lane holds the sum of its row of 16
-    const float s0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-    const float s1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-    const float s2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-    const float s3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-    return (s0 + s1) + (s2 + s3);
+    v += dpp_moved<0xB1>(v);        // quad_perm [1, 0, 3, 2]
+    v += dpp_moved<0x4E>(v);        // quad_perm [2, 3, 0, 1]
+    v += dpp_moved<0x141>(v);       // row_half_mirror
+    v += dpp_moved<0x140>(v);       // row_mirror: every lane holds the sum of its row of 16
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
 // Waves per block; a block fills a CU.  Degrees 3 and 4 fit 168 vector registers (three waves per SIMD: 7.0 ms against 7.7 ms
 // for 16 paths of 200 steps, 64 channels, degree 4); the longer chains above need more and run two waves per SIMD (a
-// third would spill: degree 5 9.4 -> 10.7 ms).
-template <int N>
-constexpr int kRowsWavesOf = N <= 4 ? 12 : 8;
+// third would spill: degree 5 9.4 -> 10.7 ms); double precision always runs two.
+template <typename T, int N>
+constexpr int kRowsWavesOf = (N <= 4 && sizeof(T) == 4) ? 12 : 8;
 constexpr int kRowsMaxWaves = 12;
 constexpr int kRowsMaxChunk = 4;                    // steps a block collects before it adds them to the gradient
 constexpr int kRowsMaxDim = 4096;                   // a row of the tile per step must leave room for the waves' words
-constexpr int kRowsPriv = 2 * kRowLetters;          // a wave's own words per step: by-letter sums, last-prefix-letter pieces
+constexpr int kRowsPriv = 2 * kWave;                // a wave's own words per step: by-letter sums, last-prefix-letter pieces (one per lane each)
 
 // both buffers of the row tile and of the waves' own words stay within 64 KB of LDS
-inline int rows_chunk_steps(int d, int waves)
+inline int rows_chunk_steps(int d, int waves, size_t elem_bytes)
 {
-    const int c = int(kMaxDynLds / (2 * sizeof(float))) / (d + waves * kRowsPriv);
+    const int c = int(kMaxDynLds / (2 * elem_bytes)) / (d + waves * kRowsPriv);
     return c < 1 ? 1 : c > kRowsMaxChunk ? kRowsMaxChunk : c;
 }
 
-template <int N>
-__global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
-    const float* __restrict__ inc, const float* __restrict__ sig, const float* __restrict__ gsig,
-    float* __restrict__ dzinc, int64_t batch, int64_t L, int d, int64_t sig_stride, int scalar, int64_t rows /* d^(N-2) */,
-    int nblk /* ceil(d / 64) */, int64_t blocks_per_path, int chunk /* rows_chunk_steps */)
+template <typename T, int N>
+__global__ __launch_bounds__((kRowsWavesOf<T, N> * kWave)) void rows_bwd_kernel(
+    const T* __restrict__ inc, const T* __restrict__ sig, const T* __restrict__ gsig,
+    T* __restrict__ dzinc, int64_t batch, int64_t L, int d, int64_t sig_stride, int scalar, int64_t rows /* d^(N-2) */,
+    int nblk /* ceil(d / 64): blocks of last prefix letters */, int nga /* ceil(d / KB): letter tiles */,
+    int64_t blocks_per_path, int chunk /* rows_chunk_steps */)
 {
-    using T = float;
-    constexpr int kRowsWaves = kRowsWavesOf<N>;
+    constexpr int kRowsWaves = kRowsWavesOf<T, N>;
+    constexpr int KB = kRowLettersOf<T>;            // letters per tile
+    constexpr int HALVES = kWave / KB;              // lane groups of the by-letter copy (1 or 2)
+    constexpr int PB = kWave / HALVES;              // prefixes per lane of the by-letter copy
     constexpr int kRowsBlock = kRowsWaves * kWave;
     using Tr = Tree<T, -1, N, 1, 1>;
     using Ad = TreeAdj<T, -1, N, 1, 1>;
@@ -89,13 +104,13 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     // ---- the wave's tile (all wave-uniform) ------------------------------
     // The waves of a block belong to one path: they share the block's gradient tile.  Surplus waves of a path's last
     // block shadow its last tile with all adjoints zero, so that every wave of a block reaches every barrier.
-    const int64_t per_path = rows * nblk * nblk;
+    const int64_t per_path = rows * nblk * nga;
     const int64_t b = int64_t(blockIdx.x) / blocks_per_path;
     int64_t w = (int64_t(blockIdx.x) - b * blocks_per_path) * kRowsWaves + wib;
     const bool valid = w < per_path;
     if (!valid) w = per_path - 1;
-    const int ga = int(w % nblk);
-    w /= nblk;
+    const int ga = int(w % nga);
+    w /= nga;
     const int blk = int(w % nblk);
     const int64_t r = w / nblk;
     int pu[M - 1];                          // the shared prefix letters
@@ -107,8 +122,8 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
             q /= d;
         }
     }
-    const int a0 = ga * kRowLetters;
-    const int last = blk * kRowLetters + lane;      // this lane's last prefix letter
+    const int a0 = ga * KB;
+    const int last = blk * kWave + lane;      // this lane's last prefix letter
     const bool active = valid && last < d;
     const int lastc = last < d ? last : d - 1;      // idle lanes shadow a valid lane: every load stays in bounds
     const int64_t q = r * d + lastc;
@@ -137,11 +152,11 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
         leaf_off = off;
     }
     // by prefix: this lane's prefix, the tile's letters
-    T gp[kRowLetters];
+    T gp[KB];
     {
         const T* g = grow + leaf_off + q * d + a0;
 #pragma unroll
-        for (int a = 0; a < kRowLetters; ++a) {
+        for (int a = 0; a < KB; ++a) {
             const bool ok = active && a0 + a < d;
             const T v = g[ok ? a : 0];
             gp[a] = ok ? v : T(0);
@@ -150,14 +165,17 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     A.gs[0] = T(1);
     S.s[0] = T(0);
     // by letter: this lane's letter, the tile's prefixes
-    const bool letter_ok = a0 + lane < d;
-    T gt[kWave];
+    const int my_letter = a0 + (lane & (KB - 1));
+    const int my_half = lane / KB;                  // prefixes PB * my_half .. of the tile
+    const bool letter_ok = my_letter < d;
+    T gt[PB];
     {
         const bool lok = valid && letter_ok;
-        const T* g = grow + leaf_off + (r * d + int64_t(blk) * kRowLetters) * d + (lok ? a0 + lane : 0);
+        const int p0 = blk * kWave + my_half * PB;  // first of this lane's prefixes (as last prefix letter)
+        const T* g = grow + leaf_off + (r * d + p0) * d + (lok ? my_letter : 0);
 #pragma unroll
-        for (int j = 0; j < kWave; ++j) {
-            const bool ok = lok && blk * kRowLetters + j < d;
+        for (int j = 0; j < PB; ++j) {
+            const bool ok = lok && p0 + j < d;
             const T v = g[ok ? int64_t(j) * d : 0];
             gt[j] = ok ? v : T(0);
         }
@@ -166,8 +184,7 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     // ---- the sweep ---------------------------------------------------------
     // Increments are [batch][L + 2][d] with a zero row at either end of a path.  The tile's slice of a step's row is
     // wave-uniform and arrives through scalar loads, requested one step ahead; a slice that reaches past the row reads
-    // on into the next row of the same path (at most 63 elements, fewer than a row holds) and meets adjoints that are
-    // zero.  The Horner values U[p] go from the by-prefix lanes to the by-letter lanes through the wave's LDS slot: one
+    // on into the next row of the same path (fewer elements than a row holds) and meets adjoints that are zero.  The Horner values U[p] go from the by-prefix lanes to the by-letter lanes through the wave's LDS slot: one
     // write, then every lane reads all of it (same address in every lane: a broadcast).
     //
     // Gradient pieces of a step: the by-letter sums and the pieces of the last prefix letter (one per lane each) go to
@@ -176,7 +193,8 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     // steps the whole block sums, per step and letter, the tile and the words of the waves that cover the letter, adds
     // the sum to the gradient row and clears the tile, while the waves already fill the other buffer: one barrier per
     // chunk.
-    extern __shared__ float rows_lds[];
+    extern __shared__ double rows_lds_raw[];
+    T* rows_lds = reinterpret_cast<T*>(rows_lds_raw);
     __shared__ __attribute__((aligned(16))) T ul_all[kRowsWaves][kWave];
     __shared__ int wave_a0[kRowsWaves], wave_l0[kRowsWaves];
     T* ul = ul_all[wib];
@@ -187,21 +205,21 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     for (int e = threadIdx.x; e < 2 * tile_elems; e += kRowsBlock) tile[e] = T(0);
     if (lane == 0) {
         wave_a0[wib] = a0;
-        wave_l0[wib] = blk * kRowLetters;
+        wave_l0[wib] = blk * kWave;
     }
     __syncthreads();
 
     const T* zrow = inc + (b * (L + 2) + L) * d;        // row of the last step
     typename Tr::Inc in;
     in.z[0] = T(0);
-    T zs[kRowLetters];
+    T zs[KB];
     T pz_next[M];
     auto fetch = [&](const T* row) {
 #pragma unroll
         for (int l = 0; l < M - 1; ++l) pz_next[l] = row[pu[l]];
         pz_next[M - 1] = row[lastc];
 #pragma unroll
-        for (int a = 0; a < kRowLetters; ++a) zs[a] = row[a0 + a];
+        for (int a = 0; a < KB; ++a) zs[a] = row[a0 + a];
     };
     fetch(zrow);
     int buf = 0, sidx = 0;
@@ -228,7 +246,7 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
         // by prefix: red = sum over the tile's letters of G[p, a] * z[a]
         T red0 = T(0), red1 = T(0);
 #pragma unroll
-        for (int a = 0; a < kRowLetters; a += 2) {
+        for (int a = 0; a < KB; a += 2) {
             red0 = fmadd(gp[a], zs[a], red0);
             red1 = fmadd(gp[a + 1], zs[a + 1], red1);
         }
@@ -259,27 +277,27 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
         }
         if (lane < M - 1) lds_add_shared(&tile[(buf * chunk + sidx) * d + where], mine);
 
-        // by letter: dz[a] = sum over the tile's prefixes of G[p, a] * U[p]
+        // by letter: dz[a] = sum over this lane's prefixes of G[p, a] * U[p]
         T acc0 = T(0), acc1 = T(0);
-        const float4* us = reinterpret_cast<const float4*>(ul);
+        constexpr int V = int(16 / sizeof(T));                  // values per 16-byte LDS read
+        struct alignas(16) Vec { T v[V]; };
+        const Vec* us = reinterpret_cast<const Vec*>(ul + my_half * PB);
 #pragma unroll
-        for (int jb = 0; jb < kWave; jb += 16) {
-            float4 v[4];
+        for (int jb = 0; jb < PB; jb += 16) {
+            Vec v[16 / V];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = us[jb / 4 + i];
+            for (int i = 0; i < 16 / V; ++i) v[i] = us[jb / V + i];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc0 = fmadd(gt[jb + 4 * i], v[i].x, acc0);
-                acc1 = fmadd(gt[jb + 4 * i + 1], v[i].y, acc1);
-                acc0 = fmadd(gt[jb + 4 * i + 2], v[i].z, acc0);
-                acc1 = fmadd(gt[jb + 4 * i + 3], v[i].w, acc1);
+            for (int i = 0; i < 16; i += 2) {
+                acc0 = fmadd(gt[jb + i], v[i / V].v[i % V], acc0);
+                acc1 = fmadd(gt[jb + i + 1], v[(i + 1) / V].v[(i + 1) % V], acc1);
             }
             __builtin_amdgcn_sched_barrier(0);      // sixteen values in flight at a time: registers
         }
         // idle lanes and shadow waves hold zero adjoints: what they write is zero
         T* mine_row = priv + ((buf * chunk + sidx) * kRowsWaves + wib) * kRowsPriv;
         mine_row[lane] = acc0 + acc1;
-        mine_row[kRowLetters + lane] = dz.dc[M - 1];
+        mine_row[kWave + lane] = dz.dc[M - 1];
 
         if (++sidx == chunk || t == 0) {
             __syncthreads();
@@ -295,8 +313,11 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
                 for (int k = 0; k < kRowsWaves; ++k) {
                     const T* wr = pr + (row * kRowsWaves + k) * kRowsPriv;
                     const unsigned ia = unsigned(a - wave_a0[k]), il = unsigned(a - wave_l0[k]);
-                    if (ia < unsigned(kRowLetters)) v += wr[ia];
-                    if (il < unsigned(kRowLetters)) v += wr[kRowLetters + il];
+                    if (ia < unsigned(KB)) {
+                        v += wr[ia];
+                        if constexpr (HALVES == 2) v += wr[KB + ia];
+                    }
+                    if (il < unsigned(kWave)) v += wr[kWave + il];
                 }
                 dev_add(&out[a - int64_t(row) * d], v);      // row `row` lies `row` gradient rows before t_first
             }
@@ -307,36 +328,37 @@ __global__ __launch_bounds__(kRowsWavesOf<N> * kWave) void rows_bwd_kernel(
     }
 }
 
-template <int N>
+template <typename T, int N>
 hipError_t launch_rows(const BwdParams& p)
 {
-    const int nblk = (p.d + kRowLetters - 1) / kRowLetters;
+    constexpr int kRowsWaves = kRowsWavesOf<T, N>;
+    const int nblk = (p.d + kWave - 1) / kWave, nga = (p.d + kRowLettersOf<T> - 1) / kRowLettersOf<T>;
     int64_t rows = 1;
     for (int i = 0; i < N - 2; ++i) rows *= p.d;
-    constexpr int kRowsWaves = kRowsWavesOf<N>;
-    const int64_t per_path = rows * nblk * nblk;
+    const int64_t per_path = rows * nblk * nga;
     const int64_t blocks_per_path = (per_path + kRowsWaves - 1) / kRowsWaves;
     const int64_t blocks = p.batch * blocks_per_path;
     if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
-    const int chunk = rows_chunk_steps(p.d, kRowsWaves);
-    const size_t lds = size_t(2) * chunk * (size_t(p.d) + kRowsWaves * kRowsPriv) * sizeof(float);
+    const int chunk = rows_chunk_steps(p.d, kRowsWaves, sizeof(T));
+    const size_t lds = size_t(2) * chunk * (size_t(p.d) + kRowsWaves * kRowsPriv) * sizeof(T);
     if (lds > kMaxDynLds) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((rows_bwd_kernel<N>), dim3(unsigned(blocks)), dim3(kRowsWaves * kWave), lds, p.stream,
-                       static_cast<const float*>(p.inc), static_cast<const float*>(p.sig), static_cast<const float*>(p.gsig),
-                       static_cast<float*>(p.dzinc), p.batch, p.L, p.d, p.sig_stride, p.scalar, rows, nblk, blocks_per_path, chunk);
+    hipLaunchKernelGGL((rows_bwd_kernel<T, N>), dim3(unsigned(blocks)), dim3(kRowsWaves * kWave), lds, p.stream,
+                       static_cast<const T*>(p.inc), static_cast<const T*>(p.sig), static_cast<const T*>(p.gsig),
+                       static_cast<T*>(p.dzinc), p.batch, p.L, p.d, p.sig_stride, p.scalar, rows, nblk, nga, blocks_per_path, chunk);
     return hipGetLastError();
 }
 
 bool rows_bwd_supported(size_t elem_bytes, uint64_t d, uint64_t degree)
 {
-    return elem_bytes == 4 && d >= uint64_t(kRowsMinDim) && d <= uint64_t(kRowsMaxDim) && degree >= uint64_t(kRowsMinDegree) &&
+    if (elem_bytes == 8 && degree > 7) return false;     // (its 56 chain values per lane no longer fit the registers)
+    return (elem_bytes == 4 || elem_bytes == 8) && d >= uint64_t(kRowsMinDim) && d <= uint64_t(kRowsMaxDim) && degree >= uint64_t(kRowsMinDegree) &&
            degree <= uint64_t(kRowsMaxDegree);
 }
 
-bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch)
+bool rows_bwd_fits(size_t elem_bytes, uint64_t d, uint64_t degree, uint64_t batch)
 {
-    const uint64_t nblk = (d + kRowLetters - 1) / kRowLetters;
-    unsigned __int128 per_path = (unsigned __int128)nblk * nblk;
+    const uint64_t nblk = (d + kWave - 1) / kWave, nga = elem_bytes == 8 ? (d + 31) / 32 : nblk;
+    unsigned __int128 per_path = (unsigned __int128)nblk * nga;
     for (uint64_t i = 0; i + 2 < degree; ++i) {
         per_path *= d;
         if (per_path > (unsigned __int128)kMaxGridX * 8) return false;
@@ -345,18 +367,23 @@ bool rows_bwd_fits(uint64_t d, uint64_t degree, uint64_t batch)
     return blocks >= 1 && blocks <= (unsigned __int128)kMaxGridX;
 }
 
-hipError_t launch_rows_bwd_f32(const BwdParams& p, int degree)
+template <typename T>
+hipError_t launch_rows_bwd(const BwdParams& p, int degree)
 {
-    if (p.nseg != 1 || p.from_points || p.d < kRowsMinDim) return hipErrorInvalidConfiguration;
+    if (p.nseg != 1 || p.from_points || p.d < kRowsMinDim || p.d > kRowsMaxDim) return hipErrorInvalidConfiguration;
     switch (degree) {
-        case 3: return launch_rows<3>(p);
-        case 4: return launch_rows<4>(p);
-        case 5: return launch_rows<5>(p);
-        case 6: return launch_rows<6>(p);
-        case 7: return launch_rows<7>(p);
-        case 8: return launch_rows<8>(p);
+        case 3: return launch_rows<T, 3>(p);
+        case 4: return launch_rows<T, 4>(p);
+        case 5: return launch_rows<T, 5>(p);
+        case 6: return launch_rows<T, 6>(p);
+        case 7: return launch_rows<T, 7>(p);
+        case 8:
+            if constexpr (sizeof(T) == 4) return launch_rows<T, 8>(p);
+            return hipErrorInvalidConfiguration;
         default: return hipErrorInvalidConfiguration;
     }
 }
+template hipError_t launch_rows_bwd<float>(const BwdParams&, int);
+template hipError_t launch_rows_bwd<double>(const BwdParams&, int);
 
 }  // namespace sigamd

@@ -704,8 +704,8 @@ def test_extreme_shapes(P, oracle, shape, dtype):
     ((2, 4, 33, 5), {}, False),                                     # chains of four letters
 ])
 def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
-    """Single-precision backward of many channels beyond the compiled table (sig_rows.hip) against the oracle, and the
-    general run-time kernels on the same input (hook off) as a second opinion on what the dispatch covers."""
+    """Backward of many channels where the compiled table has no faster kernel (sig_rows.hip), both precisions, against
+    the oracle; and the general run-time kernels on the same input (hook off) as a second opinion on the dispatch."""
     import ctypes
     from pysiglib_amd import _loader as L
     L.CUSIG.cusig_amd_set_rows_backward.argtypes = (ctypes.c_int,)
@@ -713,26 +713,24 @@ def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
     L.CUSIG.cusig_amd_last_kernel_name.restype = ctypes.c_char_p
     b, length, d, deg = shape
     rng = np.random.default_rng(b * 100000 + length * 1000 + d * 10 + deg)
-    x = (np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (1.5 / np.sqrt(d))).astype(np.float32)
-    ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
-    g = rng.standard_normal(ref.shape).astype(np.float32)
-    want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
-    ref32 = ref.astype(np.float32)
-    try:
-        L.CUSIG.cusig_amd_set_profiling(1)
-        got = P.sig_backprop(dev(x), dev(ref32), dev(g), deg, **aug).cpu().numpy()
-        assert L.CUSIG.cusig_amd_last_kernel_name().decode() == "rows_bwd_f32_n%d" % deg
-        L.CUSIG.cusig_amd_set_rows_backward(0)
-        other = P.sig_backprop(dev(x), dev(ref32), dev(g), deg, **aug).cpu().numpy()
-        assert not L.CUSIG.cusig_amd_last_kernel_name().decode().startswith("rows_bwd")
-    finally:
-        L.CUSIG.cusig_amd_set_rows_backward(1)
-        L.CUSIG.cusig_amd_set_profiling(0)
-    assert bwd_rel_err(got, want) <= TOL[np.float32], bwd_rel_err(got, want)
-    assert bwd_rel_err(other, want) <= TOL[np.float32], bwd_rel_err(other, want)
-    # double precision keeps the general kernels
-    assert bwd_rel_err(P.sig_backprop(dev(x.astype(np.float64)), dev(ref.astype(np.float64)), dev(g.astype(np.float64)),
-                                      deg, **aug).cpu().numpy(), want) <= TOL[np.float32]
+    x64 = np.cumsum(rng.standard_normal((b, length, d)), axis=1) * (1.5 / np.sqrt(d))
+    for dtype in (np.float32, np.float64):
+        x = x64.astype(dtype)
+        ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
+        g = rng.standard_normal(ref.shape).astype(dtype)
+        want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+        try:
+            L.CUSIG.cusig_amd_set_profiling(1)
+            got = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+            assert L.CUSIG.cusig_amd_last_kernel_name().decode() == "rows_bwd_%s_n%d" % ("f32" if dtype == np.float32 else "f64", deg)
+            L.CUSIG.cusig_amd_set_rows_backward(0)
+            other = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
+            assert not L.CUSIG.cusig_amd_last_kernel_name().decode().startswith("rows_bwd")
+        finally:
+            L.CUSIG.cusig_amd_set_rows_backward(1)
+            L.CUSIG.cusig_amd_set_profiling(0)
+        assert bwd_rel_err(got, want) <= TOL[dtype], (dtype, bwd_rel_err(got, want))
+        assert bwd_rel_err(other, want) <= TOL[dtype], (dtype, bwd_rel_err(other, want))
 
 
 @pytest.mark.parametrize("shape", [(3, 9, 2, 5), (2, 7, 2, 9), (5, 12, 2, 12), (2, 6, 3, 4), (3, 10, 3, 7), (2, 9, 3, 10),
@@ -985,7 +983,8 @@ def test_degree_two_closed_form(P, oracle, shape, aug, dtype):
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_every_specialised_dimension_above_12(P, oracle, dtype):
-    """One small forward + backward per compiled (dimension, degree) instance that the grid above does not reach:
+    """One small forward + backward per compiled (dimension, degree) instance that the grid above does not reach
+    (backward: up to 47 channels, beyond which the by-row reverse sweep takes over):
     dimensions 13..64 at degree 3, 13..32 and 41..48 at degree 4, 9..16 and 21..24 at degree 5, 7..12 at degree 6, 6..8 at degree 7, 5..6 at
     degree 8, 4..5 at degree 9, 4 at degree 10, 2 at degrees 13..16, 3 at degrees 13 and 14."""
     import ctypes
@@ -1019,9 +1018,14 @@ def test_every_specialised_dimension_above_12(P, oracle, dtype):
             assert level_rel_err(got, ref, d, deg) <= TOL[dtype], (d, deg)
             g = rng.standard_normal(ref.shape).astype(dtype)
             want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1)
-            pin(True, d, deg)
+            if d >= 48:
+                # from 48 channels on the backward has no compiled instance: the by-row reverse sweep serves it
+                C.cusig_amd_force_partition(0, 0)
+            else:
+                pin(True, d, deg)
             got_b = P.sig_backprop(dev(x), dev(ref), dev(g), deg).cpu().numpy()
-            assert ("_d%d_n%d_" % (d, deg)) in C.cusig_amd_last_kernel_name().decode()
+            name = C.cusig_amd_last_kernel_name().decode()
+            assert name.startswith("rows_bwd_") if d >= 48 else ("_d%d_n%d_" % (d, deg)) in name, (d, deg, name)
             assert bwd_rel_err(got_b, want) <= TOL[dtype], (d, deg)
     finally:
         C.cusig_amd_force_partition(0, 0)
