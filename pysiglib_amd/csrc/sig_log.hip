@@ -394,6 +394,41 @@ static void sig_to_log_sig_backprop_impl(const T* sig, T* out, const T* derivs, 
     SIG_HIP(hipStreamSynchronize(stream));
 }
 
+// values per path in the compressed (methods 1, 2) or expanded (method 0) logarithm
+static uint64_t log_row_len(uint64_t dimension, uint64_t degree, int method, const SigShape& s)
+{
+    if (!method) return s.stride;
+    std::lock_guard<std::mutex> lk(g_ws_mutex);
+    return find_lyndon(dimension, degree, method).count;
+}
+
+// the two operators with the batch taken in halves when the device cannot hold the workspace of the whole call
+// (siglib/cusig/cu_runtime_utils.h:103-105,212-235)
+template <typename T>
+static void sig_to_log_sig_entry(const T* sig, T* out, uint64_t batch, uint64_t dimension, uint64_t degree, int method,
+                                 bool scalar_term)
+{
+    check_method(method, "sig_to_log_sig_cuda");
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_cuda");
+    const uint64_t row = batch ? log_row_len(dimension, degree, method, s) : 0;
+    split_on_bad_alloc(batch, "sig_to_log_sig", [&](uint64_t first, uint64_t count) {
+        sig_to_log_sig_impl<T>(sig + first * s.stride, out + first * row, count, dimension, degree, method, scalar_term);
+    });
+}
+
+template <typename T>
+static void sig_to_log_sig_backprop_entry(const T* sig, T* out, const T* derivs, uint64_t batch, uint64_t dimension,
+                                          uint64_t degree, int method, bool scalar_term)
+{
+    check_method(method, "sig_to_log_sig_backprop_cuda");
+    const SigShape s = sig_shape(dimension, degree, scalar_term, "sig_to_log_sig_backprop_cuda");
+    const uint64_t row = batch ? log_row_len(dimension, degree, method, s) : 0;
+    split_on_bad_alloc(batch, "sig_to_log_sig_backprop", [&](uint64_t first, uint64_t count) {
+        sig_to_log_sig_backprop_impl<T>(sig + first * s.stride, out + first * s.stride, derivs + first * row, count, dimension,
+                                        degree, method, scalar_term);
+    });
+}
+
 }  // namespace sigamd
 
 using namespace sigamd;
@@ -403,18 +438,18 @@ extern "C" {
 CUSIG_AMD_API int sig_to_log_sig_cuda_f(const float* sig, float* out, uint64_t batch_size, uint64_t dimension, uint64_t degree,
                                         int method, bool scalar_term) noexcept
 {
-    return guarded([&] { sig_to_log_sig_impl<float>(sig, out, batch_size, dimension, degree, method, scalar_term); });
+    return guarded([&] { sig_to_log_sig_entry<float>(sig, out, batch_size, dimension, degree, method, scalar_term); });
 }
 CUSIG_AMD_API int sig_to_log_sig_cuda_d(const double* sig, double* out, uint64_t batch_size, uint64_t dimension,
                                         uint64_t degree, int method, bool scalar_term) noexcept
 {
-    return guarded([&] { sig_to_log_sig_impl<double>(sig, out, batch_size, dimension, degree, method, scalar_term); });
+    return guarded([&] { sig_to_log_sig_entry<double>(sig, out, batch_size, dimension, degree, method, scalar_term); });
 }
 CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_f(const float* sig, float* out, const float* log_sig_derivs, uint64_t batch_size,
                                                  uint64_t dimension, uint64_t degree, int method, bool scalar_term) noexcept
 {
     return guarded([&] {
-        sig_to_log_sig_backprop_impl<float>(sig, out, log_sig_derivs, batch_size, dimension, degree, method, scalar_term);
+        sig_to_log_sig_backprop_entry<float>(sig, out, log_sig_derivs, batch_size, dimension, degree, method, scalar_term);
     });
 }
 CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_d(const double* sig, double* out, const double* log_sig_derivs,
@@ -422,7 +457,7 @@ CUSIG_AMD_API int sig_to_log_sig_backprop_cuda_d(const double* sig, double* out,
                                                  bool scalar_term) noexcept
 {
     return guarded([&] {
-        sig_to_log_sig_backprop_impl<double>(sig, out, log_sig_derivs, batch_size, dimension, degree, method, scalar_term);
+        sig_to_log_sig_backprop_entry<double>(sig, out, log_sig_derivs, batch_size, dimension, degree, method, scalar_term);
     });
 }
 

@@ -629,6 +629,42 @@ def test_sig_to_log_sig_vs_oracle(P, oracle, chen_mode, chen_low, d, deg, batch,
         assert row_rel_err(gotb[:, off:], wantb[:, off:]) < TOL[dtype] * (1 if dtype == np.float64 else 10)
 
 
+@pytest.mark.parametrize("method", [0, 1, 2])
+def test_sig_to_log_sig_out_of_memory_halves_the_batch(P, method):
+    """A workspace the device cannot hold (forced from the host) makes sig_to_log_sig and its backward retry on halves
+    of the batch, like the reference's launchers (siglib/cusig/cu_runtime_utils.h:103-105,212-235): same results as the
+    undisturbed call, rows of either form (expanded, Lyndon coordinates) at their own stride."""
+    from pysiglib_amd import _loader as L
+    L.CUSIG.cusig_amd_set_alloc_limit.argtypes = (ctypes.c_uint64,)
+    L.CUSIG.cusig_amd_set_alloc_limit.restype = None
+    L.CUSIG.cusig_amd_alloc_retries.restype = ctypes.c_int
+    d, deg, batch = 4, 5, 48
+    rng = np.random.default_rng(91 + method)
+    x = np.cumsum(rng.standard_normal((batch, 12, d)), axis=1) * 0.3
+    sig = P.sig(dev(x), deg)
+    if method:
+        P.prepare_log_sig(d, deg, method)
+    want = P.sig_to_log_sig(sig, d, deg, method=method)
+    g = dev(rng.standard_normal(tuple(want.shape)))
+    wantb = P.sig_to_log_sig_backprop(sig, g, d, deg, method=method)
+    row_bytes = sig.shape[1] * 8
+    try:
+        L.CUSIG.cusig_shutdown()                     # grown workspaces would hide the limit
+        if method:
+            P.prepare_log_sig(d, deg, method)        # (the shutdown dropped the prepared tables)
+        before = L.CUSIG.cusig_amd_alloc_retries()
+        L.CUSIG.cusig_amd_set_alloc_limit(batch * row_bytes)         # the forward wants two rows per path: half the batch fits
+        got = P.sig_to_log_sig(sig, d, deg, method=method)
+        mid = L.CUSIG.cusig_amd_alloc_retries()
+        assert mid >= before + 1
+        gotb = P.sig_to_log_sig_backprop(sig, g, d, deg, method=method)
+        assert L.CUSIG.cusig_amd_alloc_retries() >= mid + 1
+    finally:
+        L.CUSIG.cusig_amd_set_alloc_limit(0)
+    assert torch.equal(got, want)
+    assert torch.equal(gotb, wantb)
+
+
 def test_log_sig_identities_shapes_and_errors(P):
     rng = np.random.default_rng(6)
     d, deg = 3, 5
