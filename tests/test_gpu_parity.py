@@ -700,6 +700,7 @@ def test_extreme_shapes(P, oracle, shape, dtype):
     ((1, 5, 64, 4), {}, False),                                     # one tile of 64 prefixes x 64 letters per word row
     ((2, 6, 49, 4), {}, True), ((2, 4, 52, 4), dict(time_aug=True), False),       # partly filled tiles
     ((2, 5, 70, 4), {}, False), ((1, 4, 130, 3), {}, True),         # several tiles per row; degree 3 beyond the table
+    ((1, 3, 300, 3), {}, False), ((3, 2, 64, 3), {}, True),         # 5 x 5 (10 in double precision) tiles per row; a single step
     ((3, 6, 25, 4), dict(lead_lag=True, time_aug=True), False),     # 51 augmented channels
     ((2, 4, 33, 5), {}, False),                                     # chains of four letters
 ])
