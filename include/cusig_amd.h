@@ -272,6 +272,10 @@ CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) CUSIG_AMD_NOEXCEPT
  * both by prefix and by letter, so no per-step reduction across lanes is left); 0 sends them to the general run-time
  * kernels. */
 CUSIG_AMD_API void cusig_amd_set_rows_backward(int on) CUSIG_AMD_NOEXCEPT;
+/* Test hook: the same switch for the forward sweep of such shapes (33 and more channels without a compiled instance,
+ * degrees 3 .. 8): 1 (default) runs the by-row forward sweep (64 or 32 top-level letters per lane), 0 the general
+ * run-time kernels. */
+CUSIG_AMD_API void cusig_amd_set_rows_forward(int on) CUSIG_AMD_NOEXCEPT;
 /* Tuning hook: how increments reach the waves: -1 automatic, 0 scalar loads, 1 LDS-staged where compiled. */
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) CUSIG_AMD_NOEXCEPT;
 /* Test hook: nonzero makes the coefficient-per-thread kernels use their 64-bit index arithmetic (otherwise only

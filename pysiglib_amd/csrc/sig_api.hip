@@ -435,6 +435,7 @@ static int choose_segments(int64_t waves, int64_t L, int waves_per_simd, uint64_
 // with the remaining segments.  That costs a segmented forward sweep, two chains of Chen products and one product
 // adjoint, all over (path, segment) rows.
 static Hook g_force_bwd_segments{0};   // tuning hook (0 = automatic)
+static Hook g_rows_forward{1};         // test hook: the same for the forward sweep
 static Hook g_rows_backward{1};        // test hook: 0 = shapes beyond the table never take the by-row reverse sweep (sig_rows.hip)
 
 // g pieces are chosen by the same kind of model as for the forward sweep (fullest SIMD, `pair_rate`, lane_step(g) =
@@ -807,7 +808,14 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         // lead-lag sweeps that skip the letters a step cannot move take the step's parity from its position in the
         // segment: segments start on even steps
         const bool sparse_ll = lead_lag && g_lead_lag_sparse != 0;
-        int nseg = g_force_segments > 0
+        // many channels without a compiled instance: the by-row sweep, whole paths only (its launches fill the chip).
+        // Measured against the general run-time kernels (16 / 32 letters per lane) at 33 .. 96 channels, degrees 4 to 6:
+        // double precision 1.0-1.46x faster; single precision 0.95-1.2x where 32 does not divide the channel count,
+        // 0.72-0.89x where it does (the 32-letter kernel then has no partly empty group and feeds from two buffers).
+        const bool rows_win = sizeof(T) == 8 || s.d_aug % 32 != 0;
+        const bool by_rows = e->D <= 0 && rows_win && g_rows_forward != 0 && g_force_tail == 0 &&
+                             rows_bwd_supported(sizeof(T), s.d_aug, degree) && rows_bwd_fits(sizeof(T), s.d_aug, degree, batch);
+        int nseg = by_rows ? 1 : g_force_segments > 0
                              ? int(std::min<uint64_t>(uint64_t(g_force_segments), s.L))
                              : choose_segments(total_waves(geom, int64_t(batch)), int64_t(s.L), e->waves_per_simd(),
                                                batch * (s.full_len - 1) * sizeof(T),
@@ -842,7 +850,7 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
         }
         e = pick_variant(false, e, total_waves(geom, p.batch), sparse_ll);
         // staged sweeps of plain narrow paths form the increments themselves while staging the points
-        if (e->staged && !time_aug && !lead_lag && e->D > 0 && e->D <= kPointFedMaxDim && g_point_fed) {
+        if (!by_rows && e->staged && !time_aug && !lead_lag && e->D > 0 && e->D <= kPointFedMaxDim && g_point_fed) {
             p.inc = path;
             p.from_points = 1;
         } else {
@@ -852,10 +860,12 @@ static void signature_impl(const T* path, T* out, uint64_t batch, uint64_t dimen
             compute_increments(path, inc, batch, dimension, length, time_aug, lead_lag, end_time, s, stream);
             p.inc = inc;
         }
-        const bool use_ll = sparse_ll && e->staged && e->fwd_lead_lag && !p.from_points;
-        const std::string shown = use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
+        const bool use_ll = !by_rows && sparse_ll && e->staged && e->fwd_lead_lag && !p.from_points;
+        const std::string shown = by_rows ? std::string(sizeof(T) == 8 ? "rows_fwd_f64_n" : "rows_fwd_f32_n") + std::to_string(degree)
+                                  : use_ll ? std::string(e->name) + "_ll" : std::string(e->name);
         MainKernelTimer timer(stream, shown.c_str());
-        SIG_HIP(use_ll ? e->fwd_lead_lag(p) : e->fwd(p));
+        if (by_rows) SIG_HIP(launch_rows_fwd<T>(p, int(degree)));
+        else SIG_HIP(use_ll ? e->fwd_lead_lag(p) : e->fwd(p));
         timer.stop(/*defer=*/true);
         if (nseg > 1) {
             // ordered product of the segment signatures by pairwise halving: ceil(log2(nseg)) launches.  An unpaired last
@@ -1465,6 +1475,7 @@ CUSIG_AMD_API void cusig_amd_set_lead_lag_sparse(int on) noexcept { if (g_test_h
 CUSIG_AMD_API void cusig_amd_force_bwd_segments(int segments) noexcept { if (g_test_hooks) g_force_bwd_segments = segments; }
 
 CUSIG_AMD_API void cusig_amd_set_rows_backward(int on) noexcept { if (g_test_hooks) g_rows_backward = on; }
+CUSIG_AMD_API void cusig_amd_set_rows_forward(int on) noexcept { if (g_test_hooks) g_rows_forward = on; }
 
 CUSIG_AMD_API void cusig_amd_force_staged(int mode) noexcept { if (g_test_hooks) g_force_staged = mode; }
 
@@ -1503,6 +1514,7 @@ CUSIG_AMD_API void cusig_amd_enable_test_hooks(int enabled) noexcept
     g_lead_lag_sparse = 1;
     g_force_bwd_segments = 0;
     g_rows_backward = 1;
+    g_rows_forward = 1;
     g_force_staged = -1;
     g_force_wide_index = 0;
     g_chen_adjoint_mode = 0;

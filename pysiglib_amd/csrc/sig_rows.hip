@@ -184,8 +184,9 @@ __global__ __launch_bounds__((kRowsWavesOf<T, N> * kWave)) void rows_bwd_kernel(
     // ---- the sweep ---------------------------------------------------------
     // Increments are [batch][L + 2][d] with a zero row at either end of a path.  The tile's slice of a step's row is
     // wave-uniform and arrives through scalar loads, requested one step ahead; a slice that reaches past the row reads
-    // on into the next row of the same path (fewer elements than a row holds) and meets adjoints that are zero.  The Horner values U[p] go from the by-prefix lanes to the by-letter lanes through the wave's LDS slot: one
-    // write, then every lane reads all of it (same address in every lane: a broadcast).
+    // on into the next row of the same path (fewer elements than a row holds) and meets adjoints that are zero.  The
+    // Horner values U[p] go from the by-prefix lanes to the by-letter lanes through the wave's LDS slot: one write, then
+    // every lane reads all of it (same address in every lane: a broadcast).
     //
     // Gradient pieces of a step: the by-letter sums and the pieces of the last prefix letter (one per lane each) go to
     // words of the wave's own in LDS with plain writes (a float LDS atomic of a full wave costs about 500 cycles here);
@@ -327,6 +328,173 @@ __global__ __launch_bounds__((kRowsWavesOf<T, N> * kWave)) void rows_bwd_kernel(
         }
     }
 }
+
+// ---------------------------------------------------------------------------
+// Forward sweep in the same tiling (arithmetic: siglib/cpsig/cp_signature.h:464-499): a lane owns the prefix
+// (r, 64 blk + lane), its chain, and the KB top-level coefficients (prefix, letter) of the wave's letter tile.  Per step
+// the top level costs one multiply-add per coefficient, S_N[p, a] += U[p] * z[a], with z[a] wave-uniform from scalar
+// loads; the chain work of a lane is shared by 64 (32) of them instead of the 16 or 32 of the general run-time kernels.
+// The letters are held in two halves: the next step's half is requested as soon as this step is done with it, so a
+// row never sits in the scalar registers twice.
+// ---------------------------------------------------------------------------
+template <typename T, int N>
+__global__ __launch_bounds__(kBlock) void rows_fwd_kernel(
+    const T* __restrict__ inc, T* __restrict__ out, int64_t batch, int64_t L, int d, int64_t out_stride, int scalar,
+    int64_t rows /* d^(N-2) */, int nblk, int nga, int* __restrict__ nonfinite)
+{
+    constexpr int KB = kRowLettersOf<T>;
+    constexpr int HB = KB / 2;
+    using Tr = Tree<T, -1, N, 1, 1>;
+    constexpr int M = N - 1;
+    static_assert(M >= 2, "degree 3 and up");
+    const int lane = threadIdx.x & (kWave - 1);
+    int64_t wave = int64_t(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    {
+        const uint32_t wlo = __builtin_amdgcn_readfirstlane(uint32_t(wave));
+        const uint32_t whi = __builtin_amdgcn_readfirstlane(uint32_t(uint64_t(wave) >> 32));
+        wave = int64_t((uint64_t(whi) << 32) | wlo);
+    }
+    const int64_t per_path = rows * nblk * nga;
+    const int64_t b = wave / per_path;
+    if (b >= batch) return;
+    int64_t w = wave - b * per_path;
+    const int ga = int(w % nga);
+    w /= nga;
+    const int blk = int(w % nblk);
+    const int64_t r = w / nblk;
+    int pu[M - 1];                          // the shared prefix letters
+    {
+        int64_t q = r;
+#pragma unroll
+        for (int l = M - 2; l >= 0; --l) {
+            pu[l] = int(q % d);
+            q /= d;
+        }
+    }
+    const int a0 = ga * KB;
+    const int last = blk * kWave + lane;
+    const bool active = last < d;
+    const int lastc = active ? last : d - 1;        // idle lanes shadow a valid lane: every load stays in bounds
+    const int64_t q = r * d + lastc;
+
+    Tr S;
+#pragma unroll
+    for (int l = 0; l < M; ++l) S.c[l] = T(0);
+    S.s[0] = T(0);
+    T leaf[KB];
+#pragma unroll
+    for (int a = 0; a < KB; ++a) leaf[a] = T(0);
+
+    // increments [batch][L + 2][d] with a zero row at either end of a path; a letter tile that reaches past the row reads
+    // on into the next row of the same path (fewer elements than a row holds): those coefficients are never stored
+    const T* zrow = inc + (b * (L + 2) + 1) * d;        // row of the first step
+    typename Tr::Inc in;
+    in.z[0] = T(0);
+    in.zs[0] = T(0);
+    T za[HB], zb[HB], pz_next[M];
+    auto fetch_prefix = [&](const T* row) {
+#pragma unroll
+        for (int l = 0; l < M - 1; ++l) pz_next[l] = row[pu[l]];
+        pz_next[M - 1] = row[lastc];
+    };
+    fetch_prefix(zrow);
+#pragma unroll
+    for (int a = 0; a < HB; ++a) za[a] = zrow[a0 + a];
+#pragma unroll
+    for (int a = 0; a < HB; ++a) zb[a] = zrow[a0 + HB + a];
+    for (int64_t t = 0; t < L; ++t) {
+#pragma unroll
+        for (int l = 0; l < M; ++l) in.pz[l] = pz_next[l];
+        zrow += d;                                      // after the last step: the zero row behind the path
+        fetch_prefix(zrow);
+        // the prefix's Horner value towards the top level, from the state before the step
+        T u;
+        if constexpr (Tr::kLockstep) {
+            typename Tr::Chain ch;
+            S.fwd_step(in, &ch);
+            u = ch.u[N][M - 1];
+        } else {
+            T uu[M];
+            S.template chain_u<N, M>(in, uu);
+            u = uu[M - 1];
+            S.fwd_step(in);
+        }
+#pragma unroll
+        for (int a = 0; a < HB; ++a) leaf[a] = fmadd(u, za[a], leaf[a]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < HB; ++a) za[a] = zrow[a0 + a];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < HB; ++a) leaf[HB + a] = fmadd(u, zb[a], leaf[HB + a]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < HB; ++a) zb[a] = zrow[a0 + HB + a];
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if (!active) return;
+    T* o = out + b * out_stride;
+    if (scalar && r == 0 && blk == 0 && ga == 0 && lane == 0) o[0] = T(1);
+    // chk stays 0 while every stored value is finite: x * 0 is NaN for x = NaN or +-Inf
+    T chk = T(0);
+    int64_t off = scalar ? 1 : 0, size = d;
+#pragma unroll
+    for (int l = 1; l <= M; ++l) {
+        int64_t span = 1;                            // d^(M - l): prefixes of full length below one level-l node
+#pragma unroll
+        for (int i = l; i < M; ++i) span *= d;
+        // a chain node is stored by the lane whose remaining prefix letters are 0, in the first letter tile
+        if (ga == 0 && q % span == 0) {
+            o[off + q / span] = S.c[l - 1];
+            chk = fmadd(S.c[l - 1], T(0), chk);
+        }
+        off += size;
+        size *= d;
+    }
+    T* top = o + off + q * d + a0;
+#pragma unroll
+    for (int a = 0; a < KB; ++a) {
+        if (a0 + a < d) {
+            top[a] = leaf[a];
+            chk = fmadd(leaf[a], T(0), chk);
+        }
+    }
+    if (nonfinite && !(chk == T(0))) *nonfinite = 1;
+}
+
+template <typename T, int N>
+hipError_t launch_rows_fwd_n(const FwdParams& p)
+{
+    const int nblk = (p.d + kWave - 1) / kWave, nga = (p.d + kRowLettersOf<T> - 1) / kRowLettersOf<T>;
+    int64_t rows = 1;
+    for (int i = 0; i < N - 2; ++i) rows *= p.d;
+    const int64_t waves = p.batch * rows * nblk * nga;
+    const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks < 1 || blocks > kMaxGridX) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((rows_fwd_kernel<T, N>), dim3(unsigned(blocks)), dim3(kBlock), 0, p.stream, static_cast<const T*>(p.inc),
+                       static_cast<T*>(p.out), p.batch, p.L, p.d, p.out_stride, p.scalar, rows, nblk, nga, p.nonfinite);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_rows_fwd(const FwdParams& p, int degree)
+{
+    if (p.nseg != 1 || p.from_points || p.d < kRowsMinDim || p.d > kRowsMaxDim) return hipErrorInvalidConfiguration;
+    switch (degree) {
+        case 3: return launch_rows_fwd_n<T, 3>(p);
+        case 4: return launch_rows_fwd_n<T, 4>(p);
+        case 5: return launch_rows_fwd_n<T, 5>(p);
+        case 6: return launch_rows_fwd_n<T, 6>(p);
+        case 7: return launch_rows_fwd_n<T, 7>(p);
+        case 8:
+            if constexpr (sizeof(T) == 4) return launch_rows_fwd_n<T, 8>(p);
+            return hipErrorInvalidConfiguration;
+        default: return hipErrorInvalidConfiguration;
+    }
+}
+template hipError_t launch_rows_fwd<float>(const FwdParams&, int);
+template hipError_t launch_rows_fwd<double>(const FwdParams&, int);
 
 template <typename T, int N>
 hipError_t launch_rows(const BwdParams& p)

@@ -711,6 +711,8 @@ def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
     from pysiglib_amd import _loader as L
     L.CUSIG.cusig_amd_set_rows_backward.argtypes = (ctypes.c_int,)
     L.CUSIG.cusig_amd_set_rows_backward.restype = None
+    L.CUSIG.cusig_amd_set_rows_forward.argtypes = (ctypes.c_int,)
+    L.CUSIG.cusig_amd_set_rows_forward.restype = None
     L.CUSIG.cusig_amd_last_kernel_name.restype = ctypes.c_char_p
     b, length, d, deg = shape
     rng = np.random.default_rng(b * 100000 + length * 1000 + d * 10 + deg)
@@ -720,8 +722,24 @@ def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
         ref = oracle.signature(x, deg, scalar_term=scalar_term, n_jobs=-1, **aug)
         g = rng.standard_normal(ref.shape).astype(dtype)
         want = oracle.sig_backprop(x, ref, g, deg, n_jobs=-1, **aug)
+        d_aug = (2 * d if aug.get("lead_lag") else d) + (1 if aug.get("time_aug") else 0)
+        off = 1 if scalar_term else 0
         try:
             L.CUSIG.cusig_amd_set_profiling(1)
+            # the forward sweep in the same tiling, where the shape has no compiled forward instance
+            fwd = P.sig(dev(x), deg, scalar_term=scalar_term, **aug).cpu().numpy()
+            name = L.CUSIG.cusig_amd_last_kernel_name().decode()
+            compiled = (deg == 3 and d_aug <= 128) or (deg == 4 and d_aug <= 48)
+            if not compiled and (dtype == np.float64 or d_aug % 32):
+                assert name == "rows_fwd_%s_n%d" % ("f32" if dtype == np.float32 else "f64", deg), name
+            assert L.CUSIG.cusig_amd_last_sig_nonfinite() == 0
+            if scalar_term:
+                np.testing.assert_array_equal(fwd[:, 0], 1.0)
+            assert level_rel_err(fwd[:, off:], ref[:, off:], d_aug, deg) <= TOL[dtype], (dtype, name)
+            L.CUSIG.cusig_amd_set_rows_forward(0)
+            fwd_other = P.sig(dev(x), deg, scalar_term=scalar_term, **aug).cpu().numpy()
+            assert not L.CUSIG.cusig_amd_last_kernel_name().decode().startswith("rows_fwd")
+            np.testing.assert_array_equal(fwd_other, fwd)       # the same arithmetic in the same order
             got = P.sig_backprop(dev(x), dev(ref), dev(g), deg, **aug).cpu().numpy()
             assert L.CUSIG.cusig_amd_last_kernel_name().decode() == "rows_bwd_%s_n%d" % ("f32" if dtype == np.float32 else "f64", deg)
             L.CUSIG.cusig_amd_set_rows_backward(0)
@@ -729,6 +747,7 @@ def test_by_row_reverse_sweep(P, oracle, shape, aug, scalar_term):
             assert not L.CUSIG.cusig_amd_last_kernel_name().decode().startswith("rows_bwd")
         finally:
             L.CUSIG.cusig_amd_set_rows_backward(1)
+            L.CUSIG.cusig_amd_set_rows_forward(1)
             L.CUSIG.cusig_amd_set_profiling(0)
         assert bwd_rel_err(got, want) <= TOL[dtype], (dtype, bwd_rel_err(got, want))
         assert bwd_rel_err(other, want) <= TOL[dtype], (dtype, bwd_rel_err(other, want))
