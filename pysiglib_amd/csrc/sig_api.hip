@@ -522,9 +522,11 @@ static Hook g_force_degree3{-1};    // tuning hook: -1 automatic, 0 never, 1 whe
 // rows buffer [paths of a chunk][L][d^2] of the degree-3 matrix form: paths are taken in chunks that fit this many bytes
 constexpr uint64_t kDeg3BufBytes = uint64_t(1) << 30;
 
-// degree 3 as library matrix products around a scan (sig_degree3.h): two products backward, one forward.  Measured against the sweep kernels at
-// batch 512, length 256: float32 1.3x faster from 48 channels (4.6x at 80, 11x at 128), float64 from 36 (10x at 80);
-// the scan needs a wave per SIMD to be worth it (a wave: 8 rows x 64 columns of one path's level 2).
+// degree 3 as library matrix products around a scan (sig_degree3.h): two products backward, one forward.  Measured at
+// batch 512 (256 at 128 channels), length 256, backward, against the by-row reverse sweep (which needs neither the
+// library nor the rows buffer): float32 48 channels 2.96 / 2.80 ms, 64: 4.23 / 4.27, 80: 9.3 / 19.4, 128: 9.2 / 15.6;
+// float64 64 channels 6.8 / 9.8, 80: 14.6 / 35.5, 128: 27.0 / 40.8 (below 48 channels the compiled float64 instances:
+// 1.3x from 36).  The scan needs a wave per SIMD to be worth it (a wave: 8 rows x 64 columns of one path's level 2).
 static bool want_degree3_gemm(uint64_t d_aug, uint64_t degree, uint64_t L, uint64_t batch, bool f64, bool backward)
 {
     if (degree != 3 || d_aug < 2 || d_aug > uint64_t(kDeg3MaxDim) || L > 0x7fffffff) return false;
@@ -532,7 +534,7 @@ static bool want_degree3_gemm(uint64_t d_aug, uint64_t degree, uint64_t L, uint6
     if (L > kDeg3BufBytes / (d_aug * d_aug * (f64 ? 8 : 4))) return false;
     if (g_force_degree3 >= 0) return g_force_degree3 != 0;
     const uint64_t waves = ((d_aug + kWave - 1) / kWave) * ((d_aug + kDeg3RowsPerThread - 1) / kDeg3RowsPerThread) * batch;
-    const uint64_t from = backward ? (f64 ? 36u : 48u) : 112u;      // forward: 1.3x at 128 channels, slower at 80
+    const uint64_t from = backward ? (f64 ? 36u : 65u) : 112u;      // forward: 1.3x at 128 channels, slower at 80
     return d_aug >= from && waves >= 1024;
 }
 
