@@ -194,7 +194,8 @@ __global__ __launch_bounds__((kRowsWavesOf<T, N> * kWave)) void rows_bwd_kernel(
     {
         const bool lok = valid && letter_ok;
         const int p0 = blk * kWave + my_half * PB;  // first of this lane's prefixes (as last prefix letter)
-        const T* g = grow + leaf_off + (r * d + p0) * d + (lok ? my_letter : 0);
+        // (a half that lies wholly beyond the row reads, and drops, the row's last prefix: every load stays in bounds)
+        const T* g = grow + leaf_off + (r * d + (p0 < d ? p0 : d - 1)) * d + (lok ? my_letter : 0);
 #pragma unroll
         for (int j = 0; j < PB; ++j) {
             const bool ok = lok && p0 + j < d;
